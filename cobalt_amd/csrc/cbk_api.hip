@@ -1,0 +1,196 @@
+// extern "C" surface of libcbk_hip.so: host-side descriptor checks and kernel dispatch.
+// No allocation, no host synchronisation, no global state.
+#include "cbk_device.h"
+
+namespace cbk {
+int launch_dequant(const DMat&, int, int, int, void*, int, int64_t, hipStream_t);
+int launch_gemv_generic(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*,
+                        hipStream_t);
+int launch_gemv_fast(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*, void*,
+                     size_t, hipStream_t);
+bool gemv_fast_takes(const DMat&, int M);
+size_t gemv_fast_workspace(const DMat&, int M);
+int launch_gemm(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*,
+                hipStream_t);
+
+static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+static int canon(const cbk_desc* in, cbk_desc* o) {
+  if (!in || !o) return CBK_ERR_NULL;
+  cbk_desc d = *in;
+  switch (d.layout) {
+    case CBK_DENSE4: d.bits = 4; d.group = 128; d.keep = 0; break;
+    case CBK_DENSE8: d.bits = 8; d.group = 128; d.keep = 0; break;
+    case CBK_SPARSE4: case CBK_SPARSE4X: case CBK_SPARSE4E: d.bits = 4; d.group = 128; d.keep = 0; break;
+    case CBK_BLK1632_4: d.bits = 4; d.group = 128; d.keep = 16; break;
+    case CBK_BLK1632_6: d.bits = 6; d.group = 128; d.keep = 16; break;
+    case CBK_BLKC:
+      if (!(d.bits == 2 || d.bits == 3 || d.bits == 4)) return CBK_ERR_LAYOUT;
+      if (d.keep < 1 || d.keep > 32) return CBK_ERR_LAYOUT;
+      break;
+    case CBK_DENSEB:
+      if (!(d.bits == 2 || d.bits == 3 || d.bits == 4 || d.bits == 8)) return CBK_ERR_LAYOUT;
+      d.keep = 0;
+      break;
+    default: return CBK_ERR_LAYOUT;
+  }
+  if (d.group != 64 && d.group != 128) return CBK_ERR_LAYOUT;
+  if (d.K <= 0 || d.N <= 0 || d.N % 128 != 0) return CBK_ERR_SHAPE;
+  if (d.cs_rows < 0 || d.cs_rows > 3) return CBK_ERR_SHAPE;
+  if (d.cs_rows == 3 && (d.cs_split0 < 0 || d.cs_split1 < 0 || d.cs_split0 + d.cs_split1 > d.K))
+    return CBK_ERR_SHAPE;
+  *o = d;
+  return CBK_OK;
+}
+
+static size_t stride_of(const cbk_desc& d) {
+  switch (family_of(d.layout)) {
+    case FAM_DENSE: return align_up(((size_t)d.N * d.bits + 7) / 8, 16);
+    case FAM_BLK: return (size_t)d.N / 8 + align_up(((size_t)(d.N / 32) * d.keep * d.bits + 7) / 8, 16);
+    case FAM_BLK6: return (size_t)d.N / 2;
+    default: return 0;
+  }
+}
+
+static int to_dmat(const cbk_desc* in, DMat* m, bool need_device_ptrs) {
+  cbk_desc d;
+  int rc = canon(in, &d);
+  if (rc) return rc;
+  const bool sparse = family_of(d.layout) == FAM_SPARSE;
+  if (need_device_ptrs) {
+    if (!d.data || !d.scale || !d.zero) return CBK_ERR_NULL;
+    if (sparse && !d.row_off) return CBK_ERR_NULL;
+    if (d.cs_rows > 0 && !d.col_scale) return CBK_ERR_NULL;
+    if (((uintptr_t)d.data & 15) || ((uintptr_t)d.scale & 3) || ((uintptr_t)d.zero & 3) ||
+        ((uintptr_t)d.col_scale & 15) || ((uintptr_t)d.row_off & 3))
+      return CBK_ERR_ALIGN;
+  }
+  m->data = (const uint8_t*)d.data;
+  m->row_off = (const uint32_t*)d.row_off;
+  m->scale = (const uint16_t*)d.scale;
+  m->zero = (const uint8_t*)d.zero;
+  m->cs = d.cs_rows > 0 ? (const uint16_t*)d.col_scale : nullptr;
+  m->K = d.K; m->N = d.N; m->G = d.N / d.group;
+  m->layout = d.layout; m->bits = d.bits; m->group = d.group; m->keep = d.keep;
+  m->cs_rows = d.cs_rows; m->cs_split0 = d.cs_split0; m->cs_split1 = d.cs_split1;
+  m->stride = (uint32_t)stride_of(d);
+  m->code_off = family_of(d.layout) == FAM_DENSE ? 0u : (uint32_t)(d.N / 8);
+  return CBK_OK;
+}
+
+static int check_io(const void* x, int xdt, int M, int64_t ldx, const void* y, int ydt, int64_t ldy, int N,
+                    int K) {
+  if (!x || !y) return CBK_ERR_NULL;
+  if (xdt != CBK_F16 && xdt != CBK_BF16T) return CBK_ERR_DTYPE;
+  if (ydt != CBK_F32 && ydt != CBK_F16 && ydt != CBK_BF16T) return CBK_ERR_DTYPE;
+  if (M < 1 || ldx < N || ldy < K) return CBK_ERR_SHAPE;
+  if (((uintptr_t)x & 15) || (ldx & 7)) return CBK_ERR_ALIGN;
+  if ((uintptr_t)y & (ydt == CBK_F32 ? 3 : 1)) return CBK_ERR_ALIGN;
+  return CBK_OK;
+}
+
+}  // namespace cbk
+
+using namespace cbk;
+
+extern "C" {
+
+int cbk_abi_version(void) { return CBK_ABI_VERSION; }
+
+const char* cbk_strerror(int s) {
+  switch (s) {
+    case CBK_OK: return "ok";
+    case CBK_ERR_NULL: return "a required pointer is NULL";
+    case CBK_ERR_LAYOUT: return "unknown layout or invalid bits/group/keep for it";
+    case CBK_ERR_SHAPE: return "shape, leading dimension or row range out of range";
+    case CBK_ERR_ALIGN: return "pointer or leading dimension not aligned as required";
+    case CBK_ERR_DTYPE: return "unsupported element type";
+    case CBK_ERR_WORKSPACE: return "workspace missing or too small";
+    case CBK_ERR_HIP: return "HIP runtime error at launch";
+    case CBK_ERR_UNSUPPORTED: return "operation does not support this layout";
+    default: return "unknown status";
+  }
+}
+
+int cbk_desc_check(const cbk_desc* in, cbk_desc* out) { return canon(in, out); }
+
+size_t cbk_row_stride(const cbk_desc* in) {
+  cbk_desc d;
+  if (canon(in, &d)) return 0;
+  return stride_of(d);
+}
+
+size_t cbk_stream_bytes(const cbk_desc* in, size_t sparse_data_bytes) {
+  cbk_desc d;
+  if (canon(in, &d)) return 0;
+  const size_t meta = (size_t)d.K * (d.N / d.group) * 3;
+  if (family_of(d.layout) == FAM_SPARSE) return sparse_data_bytes + meta;
+  return (size_t)d.K * stride_of(d) + meta;
+}
+
+size_t cbk_workspace_bytes(const cbk_desc* in, int M) {
+  DMat m;
+  if (to_dmat(in, &m, false)) return 0;
+  if (M >= 1 && M <= 16 && gemv_fast_takes(m, M)) return gemv_fast_workspace(m, M);
+  return 0;
+}
+
+int cbk_dequant(const cbk_desc* in, int row0, int nrows, int with_col_scale, void* out, int out_dtype,
+                int64_t ld_out, void* stream) {
+  DMat m;
+  int rc = to_dmat(in, &m, true);
+  if (rc) return rc;
+  if (!out) return CBK_ERR_NULL;
+  if (row0 < 0 || nrows < 0 || row0 + nrows > m.K || ld_out < m.N) return CBK_ERR_SHAPE;
+  if (out_dtype != CBK_F32 && out_dtype != CBK_F16 && out_dtype != CBK_BF16T) return CBK_ERR_DTYPE;
+  return launch_dequant(m, row0, nrows, with_col_scale, out, out_dtype, ld_out, (hipStream_t)stream);
+}
+
+int cbk_gemv(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ldx, void* y, int y_dtype,
+             int64_t ldy, const void* bias, void* workspace, size_t workspace_bytes, void* stream) {
+  DMat m;
+  int rc = to_dmat(in, &m, true);
+  if (rc) return rc;
+  rc = check_io(x, x_dtype, M, ldx, y, y_dtype, ldy, m.N, m.K);
+  if (rc) return rc;
+  if (M > 16) return CBK_ERR_SHAPE;
+  if (gemv_fast_takes(m, M)) {
+    const size_t need = gemv_fast_workspace(m, M);
+    if (need && (!workspace || workspace_bytes < need)) return CBK_ERR_WORKSPACE;
+    if ((uintptr_t)workspace & 255) return CBK_ERR_ALIGN;
+    return launch_gemv_fast(m, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, workspace, workspace_bytes,
+                            (hipStream_t)stream);
+  }
+  return launch_gemv_generic(m, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, (hipStream_t)stream);
+}
+
+int cbk_gemm(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ldx, void* y, int y_dtype,
+             int64_t ldy, const void* bias, void* workspace, size_t workspace_bytes, void* stream) {
+  (void)workspace; (void)workspace_bytes;
+  DMat m;
+  int rc = to_dmat(in, &m, true);
+  if (rc) return rc;
+  rc = check_io(x, x_dtype, M, ldx, y, y_dtype, ldy, m.N, m.K);
+  if (rc) return rc;
+  return launch_gemm(m, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, (hipStream_t)stream);
+}
+
+int cbk_linear(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ldx, void* y, int y_dtype,
+               int64_t ldy, const void* bias, void* workspace, size_t workspace_bytes, void* stream) {
+  if (M <= 16) return cbk_gemv(in, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, workspace, workspace_bytes, stream);
+  cbk_desc d;
+  if (in && canon(in, &d) == CBK_OK && family_of(d.layout) == FAM_SPARSE) {
+    // the variable-length layouts have no MFMA path: run the row GEMV in slices of 16 rows
+    for (int m0 = 0; m0 < M; m0 += 16) {
+      const int mc = M - m0 < 16 ? M - m0 : 16;
+      int rc = cbk_gemv(in, (const uint8_t*)x + (size_t)m0 * ldx * 2, x_dtype, mc, ldx,
+                        (uint8_t*)y + (size_t)m0 * ldy * (y_dtype == CBK_F32 ? 4 : 2), y_dtype, ldy, bias,
+                        workspace, workspace_bytes, stream);
+      if (rc) return rc;
+    }
+    return CBK_OK;
+  }
+  return cbk_gemm(in, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"

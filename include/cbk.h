@@ -1,0 +1,136 @@
+/* cbk.h -- C ABI of the MI355X (gfx950) CBK1 sparse low-bit linear layer.
+ *
+ * One packed weight matrix W_hat[K, N] (K output rows, N input columns) times fp16/bf16
+ * activations X[M, N]:   Y[M, K] = X . W_hat^T (+ bias),  with
+ *
+ *     W_hat[k, j] = ((q[k, j] - zero[k, j/group]) * scale[k, j/group]) * keep[k, j] * col_scale[cs(k), j]
+ *
+ * evaluated in float32 (reference: docs/FORMAT.md:43-45, src/cobaltkernel/dequant_ref.py:69-82).
+ *
+ * Every pointer is a DEVICE pointer owned by the caller.  The library never allocates or
+ * frees device memory, never synchronises the host, and launches only on the stream it
+ * is given (reference harness: src/cobaltkernel/csrc/test_gemv.cu:187-235 allocates its
+ * outputs itself; the runners pre-allocate everything, runner.py:492-521).
+ * All entry points return 0 on success or a negative cbk_status.
+ */
+#ifndef CBK_H_
+#define CBK_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CBK_ABI_VERSION 1
+
+/* Layout ids 0-7 are the reference's (src/cobaltkernel/csrc/cobalt_format.h:23-32,
+ * src/cobaltkernel/pack_cobalt.py:28-36).  8 and 9 generalise the two shipped families to
+ * 2/3/4-bit codes, a group of 64 or 128 and any per-32-column survivor count. */
+enum cbk_layout {
+  CBK_SPARSE4 = 0,   /* bitmap + variable-length nibble stream, per-row offsets          */
+  CBK_DENSE4 = 1,    /* 4-bit code per column, pruned columns hold the zero point        */
+  CBK_DENSE8 = 2,    /* 8-bit code per column                                            */
+  CBK_SPARSE4X = 3,  /* SPARSE4 + uint16 per-group code offsets                          */
+  CBK_BF16 = 4,      /* (not supported: unquantised passthrough)                         */
+  CBK_SPARSE4E = 5,  /* byte-identical to SPARSE4X                                       */
+  CBK_BLK1632_4 = 6, /* exactly 16 of every 32 columns kept, 4-bit survivors             */
+  CBK_BLK1632_6 = 7, /* the same mask, 6-bit survivors (nibble plane + hi2 plane)        */
+  CBK_BLKC = 8,      /* exactly `keep` of every 32 columns kept, `bits`-bit survivors as
+                        one LSB-first bit stream per row; (4,16,128) == BLK1632_4        */
+  CBK_DENSEB = 9     /* `bits`-bit code per column as one LSB-first bit stream per row;
+                        bits 4 == DENSE4, bits 8 == DENSE8                               */
+};
+
+enum cbk_dtype { CBK_F32 = 0, CBK_F16 = 1, CBK_BF16T = 2 };
+
+enum cbk_status {
+  CBK_OK = 0,
+  CBK_ERR_NULL = -1,        /* a required pointer is NULL                                 */
+  CBK_ERR_LAYOUT = -2,      /* unknown layout, or bits/group/keep not valid for it        */
+  CBK_ERR_SHAPE = -3,       /* K, N, M, leading dimension or row range out of range       */
+  CBK_ERR_ALIGN = -4,       /* a pointer or leading dimension is not aligned as required  */
+  CBK_ERR_DTYPE = -5,       /* unsupported element type                                   */
+  CBK_ERR_WORKSPACE = -6,   /* workspace missing or smaller than cbk_workspace_bytes()    */
+  CBK_ERR_HIP = -7,         /* the HIP runtime reported an error at launch                */
+  CBK_ERR_UNSUPPORTED = -8  /* valid descriptor, but this operation does not take it      */
+};
+
+/* One packed matrix.  Replaces cbk::Mat (cobalt_format.h:103-109) and the 9-int64 MatDesc
+ * device table entry (src/cobaltkernel/csrc/megakernel.cuh:21-28).
+ *   data      row regions; fixed-stride layouts: row k at data + k*cbk_row_stride(); 64 B of
+ *             readable padding after the last row (docs/FORMAT.md:22-24).  16-byte aligned.
+ *   row_off   uint32[K+1] byte offsets of the row regions (SPARSE4/4X/4E only), else NULL
+ *   scale     fp16  [K, N/group] row-major, 4-byte aligned
+ *   zero      uint8 [K, N/group] row-major integer zero points, 4-byte aligned
+ *   col_scale fp16  [cs_rows, N] or NULL (then the factor is 1), 16-byte aligned
+ *   cs_rows   1: one vector.  2: fused gate/up, row k uses vector k&1.  3: fused q|k|v, rows
+ *             [0,cs_split0) use vector 0, [cs_split0, cs_split0+cs_split1) vector 1, the rest 2
+ *             (cobalt_format.h:77-99, docs/FORMAT.md:134-151).
+ *   bits/group/keep  must be given for layouts 8/9; for 0-7 they may be 0 (implied). */
+typedef struct cbk_desc {
+  const void* data;
+  const void* row_off;
+  const void* scale;
+  const void* zero;
+  const void* col_scale;
+  int32_t K, N;
+  int32_t layout;
+  int32_t bits;
+  int32_t group;
+  int32_t keep;
+  int32_t cs_rows;
+  int32_t cs_split0, cs_split1;
+  int32_t reserved;
+} cbk_desc;
+
+int cbk_abi_version(void);
+const char* cbk_strerror(int status);
+
+/* Checks a descriptor on the host (no device access) and fills bits/group/keep for the
+ * reference layouts into *out (may alias in). */
+int cbk_desc_check(const cbk_desc* in, cbk_desc* out);
+
+/* Bytes per row of a fixed-stride layout (cobalt_format.h:59-68); 0 for SPARSE4/4X/4E
+ * or an invalid descriptor. */
+size_t cbk_row_stride(const cbk_desc* d);
+
+/* Weight bytes one pass over the matrix streams: rows + scale + zero
+ * (pack_cobalt.write_matrix :431-433 `stream_bytes`); SPARSE layouts need data_bytes. */
+size_t cbk_stream_bytes(const cbk_desc* d, size_t sparse_data_bytes);
+
+/* Device scratch needed by cbk_gemv / cbk_gemm / cbk_linear for M activation rows. */
+size_t cbk_workspace_bytes(const cbk_desc* d, int M);
+
+/* Rows [row0, row0+nrows) of W_hat -> out[nrows, ld_out] in out_dtype, bit-exact float32
+ * evaluation then one round-to-nearest-even cast.  with_col_scale = 0 leaves the column
+ * scale out, like cbk::dequant_row (src/cobaltkernel/csrc/cobalt_gemv.cuh:1218-1315,
+ * harness entry `dequant_rows`, test_gemv.cu:223-235). */
+int cbk_dequant(const cbk_desc* d, int row0, int nrows, int with_col_scale,
+                void* out, int out_dtype, int64_t ld_out, void* stream);
+
+/* Decode path, 1 <= M <= 16: y[m, k] = sum_j x[m, j] * W_hat[k, j] (+ bias[k]).
+ * x is [M, ldx] fp16 or bf16, y is [M, ldy] in y_dtype (f32 / f16 / bf16), bias is NULL or
+ * K values of y_dtype.  Replaces the harness entry `gemv` (test_gemv.cu:187-199) and
+ * cbk::gemv_rows (cobalt_gemv.cuh:1196-1213); unlike those it applies col_scale itself. */
+int cbk_gemv(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
+             void* y, int y_dtype, int64_t ldy, const void* bias,
+             void* workspace, size_t workspace_bytes, void* stream);
+
+/* Prefill path, any M >= 1 (built for M >= 256).  Same contract as cbk_gemv.  Replaces the
+ * harness entry `gemm` (test_gemm.cu:151-165) and cbk::gemm_tile (cobalt_gemm.cuh:243-609). */
+int cbk_gemm(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
+             void* y, int y_dtype, int64_t ldy, const void* bias,
+             void* workspace, size_t workspace_bytes, void* stream);
+
+/* The layer forward: cbk_gemv for M <= 16, cbk_gemm above (the module seam of
+ * benchmarks/benchmark_suite.py:1200-1217). */
+int cbk_linear(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
+               void* y, int y_dtype, int64_t ldy, const void* bias,
+               void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CBK_H_ */

@@ -1,0 +1,248 @@
+"""GPU parity: the HIP library, called through the C ABI, against the CPU oracle on the same
+seeded inputs.  Bars: dequantised weights bit-exact (value equality; -0.0 == 0.0, as the
+reference's own check does, src/prod/verify.py:139); layer outputs within relative Frobenius
+error 1e-3 of x @ W_hat.T with W_hat in float32 and a float64 accumulator."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cbk_ref as R
+from cobalt_amd import format as F
+from cobalt_amd import ops
+from cobalt_amd.linear import CobaltLinear
+from helpers import (FIXED_CASES, SPARSE_CASES, acts, case_id, kw_of, make_raw, oracle_pack, packed_from_oracle,
+                     product_pack, rel_fro)
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+TOL = 1e-3          # relative Frobenius error of a layer output (the bar this layer is held to)
+
+
+def _np(t):
+    return t.detach().float().cpu().numpy()
+
+
+def _bf16_round(a):
+    return _np(torch.from_numpy(np.asarray(a, np.float32)).to(torch.bfloat16))
+
+
+def _f16_round(a):
+    return _np(torch.from_numpy(np.asarray(a, np.float32)).to(torch.float16))
+
+
+# ------------------------------------------------------------------ dequant, bit-exact
+@pytest.mark.parametrize("case", FIXED_CASES + SPARSE_CASES, ids=case_id)
+def test_dequant_bit_exact(case):
+    for (K, N) in ((64, 1024), (40, 5376)):
+        raw = make_raw(case, K, N, seed=K + N + case[0])
+        pk = oracle_pack(case, raw)
+        pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV)
+        W = R.dequant(pk, K, N, case[0], col_scale=raw["col_scale"], **kw_of(case))
+        got = _np(ops.dequant(pm, torch.float32))
+        assert np.array_equal(got, W), f"{case_id(case)} {K}x{N}: {np.abs(got - W).max()}"
+        W0 = R.dequant(pk, K, N, case[0], **kw_of(case))
+        assert np.array_equal(_np(ops.dequant(pm, torch.float32, with_col_scale=False)), W0)
+        assert np.array_equal(_np(ops.dequant(pm, torch.bfloat16)), _bf16_round(W))
+        assert np.array_equal(_np(ops.dequant(pm, torch.float16)), _f16_round(W))
+        # a row window
+        assert np.array_equal(_np(ops.dequant(pm, torch.float32, row0=8, nrows=16)), W[8:24])
+
+
+def test_dequant_fused_col_scale_rows_and_subnormal_scales():
+    K, N = 48, 512
+    raw = R.synth_raw_matrix(K, N, 0.5, 4, seed=3, block=32)
+    raw["scale"][::5] = np.float16(6.7e-6)                # fp16 subnormal scale
+    pk = R.pack_matrix(raw["mask"], raw["q"], raw["scale"], raw["zero"], R.BLK1632_4)
+    rng = np.random.default_rng(0)
+    for cs_rows, splits in ((2, (0, 0)), (3, (32, 8))):
+        cs = (rng.random((cs_rows, N)) * 1.5 + 0.5).astype(np.float16)
+        pm = packed_from_oracle((F.BLK1632_4, 4, 128, 16), pk, cs, K, N, DEV, cs_splits=splits)
+        W = R.dequant(pk, K, N, R.BLK1632_4, col_scale=cs, cs_splits=splits)
+        assert np.array_equal(_np(ops.dequant(pm, torch.float32)), W)
+        assert (W[::5] != 0).any()
+
+
+def test_pruned_positions_exactly_zero_off_grid_zero_point():
+    K, N = 32, 1024
+    raw = R.synth_raw_matrix(K, N, 0.5, 4, seed=9, block=32)
+    keep = R.unpack_bits(raw["mask"], N)
+    off = np.full((K, N // 128), 15 + 37, np.float16)
+    pk = R.pack_matrix(raw["mask"], raw["q"], raw["scale"], off, R.BLK1632_4, fix_zero=False)
+    pm = packed_from_oracle((F.BLK1632_4, 4, 128, 16), pk, raw["col_scale"], K, N, DEV)
+    W = _np(ops.dequant(pm, torch.float32))
+    assert (W[~keep] == 0).all() and np.array_equal(W, R.dequant(pk, K, N, R.BLK1632_4, col_scale=raw["col_scale"]))
+
+
+# ------------------------------------------------------------------ decode GEMV
+@pytest.mark.parametrize("case", FIXED_CASES + SPARSE_CASES, ids=case_id)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+def test_gemv_matches_oracle(case, dtype):
+    for (K, N) in ((192, 4096), (80, 5376)):
+        raw = make_raw(case, K, N, seed=K + N + 31 * case[0])
+        pk = oracle_pack(case, raw)
+        pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV)
+        W = R.dequant(pk, K, N, case[0], col_scale=raw["col_scale"], **kw_of(case))
+        for M in (1, 2, 3, 4, 8, 16):
+            x = acts(M, N, dtype, seed=M)
+            ref = R.forward_ref(W, _np(x))
+            y = ops.gemv(pm, x.to(DEV), out_dtype=torch.float32)
+            err = rel_fro(_np(y), ref)
+            assert err < TOL, f"{case_id(case)} {K}x{N} M={M}: {err}"
+            # the reference's own GEMV gate (test_gemv.py:162-167) is max|err|/max|ref| < 2e-5
+            # for bf16 inputs with fp32 accumulation; hold the fp32 output to 1e-4
+            assert np.abs(_np(y) - ref).max() / np.abs(ref).max() < 1e-4
+
+
+def test_gemv_output_dtypes_bias_and_strided_x():
+    case = (F.BLK1632_4, 4, 128, 16)
+    K, N = 128, 2048
+    raw = make_raw(case, K, N, seed=5)
+    pk = oracle_pack(case, raw)
+    pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV)
+    W = R.dequant(pk, K, N, case[0], col_scale=raw["col_scale"])
+    for dtype in (torch.float16, torch.bfloat16):
+        bias = (torch.randn(K) * 0.5).to(dtype)
+        xb = acts(4, N + 64, dtype, seed=2)
+        x = xb[:, :N]                                       # leading dimension N + 64
+        ref = R.forward_ref(W, _np(x), bias=_np(bias))
+        y = ops.gemv(pm, x.to(DEV), bias=bias.to(DEV))
+        assert y.dtype == dtype and y.shape == (4, K)
+        tol = 3e-3 if dtype == torch.bfloat16 else 6e-4     # + one rounding of y to its dtype
+        assert rel_fro(_np(y), ref) < tol
+        y3 = ops.linear(pm, x.to(DEV).reshape(2, 2, N), bias=bias.to(DEV))
+        assert y3.shape == (2, 2, K) and torch.equal(y3.reshape(4, K), y)
+    # no col_scale at all
+    pm0 = packed_from_oracle(case, pk, None, K, N, DEV)
+    x = acts(2, N, torch.float16, seed=8)
+    assert rel_fro(_np(ops.gemv(pm0, x.to(DEV), out_dtype=torch.float32)),
+                   R.forward_ref(R.dequant(pk, K, N, case[0]), _np(x))) < TOL
+
+
+@pytest.mark.parametrize("case", [(F.BLK1632_4, 4, 128, 16), (F.BLKC, 3, 128, 10), (F.BLKC, 2, 64, 23),
+                                  (F.BLK1632_6, 6, 128, 16)], ids=case_id)
+def test_gemv_pruned_columns_contribute_exactly_zero(case):
+    """Restates test_gemv.py:403-455: a column-uniform mask, huge activations at the pruned
+    columns; the output must be bit-identical, with the zero point on and off the grid."""
+    layout, bits, group, keep = case
+    K, N = 256, 5376
+    rng = np.random.default_rng(7)
+    pat = np.zeros((N // 32, 32), bool)
+    idx = np.argsort(rng.random((N // 32, 32)), axis=1)[:, :keep]
+    np.put_along_axis(pat, idx, True, axis=1)
+    keepm = np.broadcast_to(pat.reshape(1, N), (K, N))
+    nl = (1 << bits) - 1
+    q = rng.integers(0, nl + 1, (K, N)).astype(np.uint8)
+    scale = (rng.random((K, N // group)) * 0.01 + 1e-3).astype(np.float16)
+    for zmode in ("ongrid", "offgrid"):
+        zero = rng.integers(0, nl + 1, (K, N // group)).astype(np.float16) if zmode == "ongrid" \
+            else np.full((K, N // group), nl + 37, np.float16)
+        pk = R.pack_matrix(R.pack_bits(keepm), q, scale, zero, layout, fix_zero=(zmode == "ongrid"), **kw_of(case))
+        pm = packed_from_oracle(case, pk, None, K, N, DEV)
+        for dtype in (torch.bfloat16, torch.float16):
+            x0 = acts(1, N, dtype, seed=1)
+            xh = x0.clone(); xh[0, torch.from_numpy(~pat.reshape(N))] = 1.0e4
+            for M in (1, 4):
+                y0 = ops.gemv(pm, x0.expand(M, N).contiguous().to(DEV), out_dtype=torch.float32)
+                yh = ops.gemv(pm, xh.expand(M, N).contiguous().to(DEV), out_dtype=torch.float32)
+                assert torch.equal(y0, yh), f"{case_id(case)} zero={zmode} {dtype} M={M}"
+        assert (_np(ops.dequant(pm))[:, ~pat.reshape(N)] == 0).all()
+
+
+def test_gemv_rows_are_independent_of_batch_and_run_to_run_identical():
+    """The reference's determinism gate: M=4 is bit-exact 4 x M=1 (docs/KERNELS.md:151-155)."""
+    case = (F.BLK1632_4, 4, 128, 16)
+    K, N = 512, 4096
+    pm = F.synth_packed(K, N, *case[:3], case[3], seed=11, device=DEV)
+    x = acts(4, N, torch.bfloat16, seed=3).to(DEV)
+    y4 = ops.gemv(pm, x, out_dtype=torch.float32)
+    for i in range(4):
+        assert torch.equal(ops.gemv(pm, x[i:i + 1], out_dtype=torch.float32)[0], y4[i])
+    assert torch.equal(ops.gemv(pm, x, out_dtype=torch.float32), y4)
+
+
+# ------------------------------------------------------------------ prefill GEMM
+@pytest.mark.parametrize("case", FIXED_CASES, ids=case_id)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+def test_gemm_matches_oracle(case, dtype):
+    K, N = 320, 1024
+    raw = make_raw(case, K, N, seed=77 + case[0])
+    pk = oracle_pack(case, raw)
+    pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV)
+    W = R.dequant(pk, K, N, case[0], col_scale=raw["col_scale"], **kw_of(case))
+    for M in (16, 100, 512):                                # the reference's M set (test_gemm.py:162-195)
+        x = acts(M, N, dtype, seed=M)
+        ref = R.forward_ref(W, _np(x))
+        y = ops.gemm(pm, x.to(DEV), out_dtype=torch.float32)
+        err = rel_fro(_np(y), ref)
+        assert err < TOL, f"{case_id(case)} M={M}: {err}"
+
+
+def test_gemm_bias_dtype_and_prune_zero():
+    case = (F.BLK1632_4, 4, 128, 16)
+    K, N, M = 256, 2048, 300
+    raw = make_raw(case, K, N, seed=4)
+    pk = oracle_pack(case, raw)
+    pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV)
+    W = R.dequant(pk, K, N, case[0], col_scale=raw["col_scale"])
+    bias = torch.randn(K).to(torch.bfloat16)
+    x = acts(M, N, torch.bfloat16, seed=6)
+    y = ops.linear(pm, x.to(DEV), bias=bias.to(DEV))
+    assert y.dtype == torch.bfloat16 and rel_fro(_np(y), R.forward_ref(W, _np(x), bias=_np(bias))) < 3e-3
+    # prune-zero through the tile (test_gemm.py:223-255): same mask in every row
+    pat = np.tile(np.r_[np.ones(16, bool), np.zeros(16, bool)], N // 32)
+    rng = np.random.default_rng(1)
+    q = rng.integers(0, 16, (K, N)).astype(np.uint8)
+    pk = R.pack_matrix(R.pack_bits(np.broadcast_to(pat, (K, N))), q, raw["scale"], np.full((K, N // 128), 52, np.float16),
+                       R.BLK1632_4, fix_zero=False)
+    pm = packed_from_oracle(case, pk, None, K, N, DEV)
+    x0 = acts(M, N, torch.float16, seed=9)
+    xh = x0.clone(); xh[:, torch.from_numpy(~pat)] = 1.0e4
+    assert torch.equal(ops.gemm(pm, x0.to(DEV), out_dtype=torch.float32), ops.gemm(pm, xh.to(DEV), out_dtype=torch.float32))
+
+
+# ------------------------------------------------------------------ the module seam
+def test_cobalt_linear_forward_matches_reference_module_math():
+    K, N = 256, 1024
+    raw = R.synth_raw_matrix(K, N, 0.5, 4, seed=2, block=32)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a))
+    bias = torch.randn(K).half()
+    lin = CobaltLinear.from_raw(t(raw["mask"]), t(raw["q"]), t(raw["scale"]), t(raw["zero"]), t(raw["col_scale"]),
+                                bias=bias).to(DEV)
+    pk = R.pack_matrix(raw["mask"], raw["q"], raw["scale"], raw["zero"], R.BLK1632_4)
+    W = R.dequant(pk, K, N, R.BLK1632_4, col_scale=raw["col_scale"])
+    assert np.array_equal(_np(lin.dequantize()), W)
+    for shape in ((1, N), (3, 5, N), (2, 200, N)):
+        x = (torch.randn(*shape) * 1.0).half()
+        y = lin(x.to(DEV))
+        assert y.shape == shape[:-1] + (K,) and y.dtype == torch.float16
+        ref = R.forward_ref(W, _np(x).reshape(-1, N), bias=_np(bias)).reshape(y.shape)
+        assert rel_fro(_np(y), ref) < 6e-4
+
+
+# ------------------------------------------------------------------ full-size properties
+@pytest.mark.parametrize("K,N,case", [(14336, 4096, (F.BLK1632_4, 4, 128, 16)), (4096, 14336, (F.BLKC, 3, 128, 10)),
+                                      (5376, 21504, (F.BLKC, 2, 64, 23))], ids=["mistral-gate", "mistral-down-b3", "gemma-down-b2g64"])
+def test_full_size_properties(K, N, case):
+    """Shapes of the benchmark configurations, where the CPU oracle is too slow for a full
+    comparison: linearity in x, agreement between the decode and the prefill kernel, agreement
+    of both with the dequantised dense weight on sampled rows (oracle on 32 rows)."""
+    pm = F.synth_packed(K, N, case[0], case[1], case[2], case[3] or None, seed=K % 97, device=DEV)
+    x = acts(2, N, torch.bfloat16, seed=5).to(DEV)
+    y = ops.gemv(pm, x, out_dtype=torch.float32)
+    # linearity: activations scaled by 2 and rows swapped
+    y2 = ops.gemv(pm, (x * 2).flip(0), out_dtype=torch.float32)
+    assert torch.equal(y2.flip(0), y * 2)
+    # decode kernel vs prefill kernel on the same inputs
+    yg = ops.gemm(pm, x, out_dtype=torch.float32)
+    assert rel_fro(_np(yg), _np(y)) < TOL
+    # sampled rows against the oracle
+    rows = np.linspace(0, K - 1, 32).astype(int)
+    pk = dict(data=pm.array("data").cpu().numpy(), scale=pm.array("scale").cpu().numpy().reshape(K, -1),
+              zero=pm.array("zero").cpu().numpy().reshape(K, -1), row_off=None)
+    stride = R.row_stride(case[0], N, case[1], case[2], case[3] or None)
+    sub = dict(data=np.concatenate([pk["data"][r * stride:(r + 1) * stride] for r in rows] + [np.zeros(64, np.uint8)]),
+               scale=pk["scale"][rows], zero=pk["zero"][rows], row_off=None)
+    Wsub = R.dequant(sub, len(rows), N, case[0], col_scale=pm.array("col_scale").cpu().numpy(), **kw_of(case))
+    Wg = _np(ops.dequant(pm, torch.float32))
+    assert np.array_equal(Wg[rows], Wsub)
+    assert rel_fro(_np(y)[:, rows], R.forward_ref(Wsub, _np(x))) < TOL

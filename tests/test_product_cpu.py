@@ -1,0 +1,185 @@
+"""CPU-side checks of the product package: its packer against the oracle's bytes, the C-ABI
+library's exports and host-side validation, and the nn.Module plumbing.  No kernel runs here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cbk_ref as R
+from cobalt_amd import _lib, format as F
+from cobalt_amd.linear import CobaltLinear, patch_model
+from helpers import FIXED_CASES, case_id, kw_of, make_raw, oracle_pack, product_pack
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.mark.parametrize("case", FIXED_CASES, ids=case_id)
+def test_product_packer_matches_oracle_bytes(case):
+    K, N = 12, 640
+    raw = make_raw(case, K, N, seed=7)
+    raw["zero"][0, 0] = -3        # one off-grid group, exercises the zero repair
+    raw["zero"][5, 1] = 99 if case[1] < 8 else 300
+    pk = oracle_pack(case, raw)
+    pm = product_pack(case, raw)
+    assert np.array_equal(pm.array("data").numpy(), pk["data"])
+    assert np.array_equal(pm.array("scale").numpy(), pk["scale"].reshape(-1))
+    assert np.array_equal(pm.array("zero").numpy(), pk["zero"].reshape(-1))
+    assert pm.n_zero_fixed == pk["n_zero_fixed"] == 2 and pm.n_survivors == pk["n_survivors"]
+    assert pm.data_bytes == K * R.row_stride(case[0], N, *case[1:]) and pm.stream_bytes() == R.stream_bytes(pk)
+    assert abs(pm.bpw() - R.bpw(pk, K, N)) < 1e-12
+    assert all(o % 256 == 0 for o in pm.offs.values())
+
+
+@pytest.mark.parametrize("case", FIXED_CASES, ids=case_id)
+def test_synth_packed_is_valid(case):
+    layout, bits, group, keep = case
+    K, N = 8, 384
+    pm = F.synth_packed(K, N, layout, bits, group, keep or None, seed=3)
+    pk = dict(data=pm.array("data").numpy(), scale=pm.array("scale").numpy().reshape(K, -1),
+              zero=pm.array("zero").numpy().reshape(K, -1), row_off=None)
+    q, kp = R.unpack_codes(pk, K, N, layout, **kw_of(case))
+    if keep:
+        assert (kp.reshape(K, N // 32, 32).sum(-1) == keep).all()
+    assert q.max() <= (1 << bits) - 1
+    # padding bits of the stream are zero, so re-packing the decoded codes reproduces the bytes
+    pk2 = R.pack_matrix(R.pack_bits(kp), q, pk["scale"], pk["zero"], layout, fix_zero=False, **kw_of(case))
+    assert np.array_equal(pk2["data"], pk["data"])
+
+
+def test_stream_helpers_roundtrip():
+    g = torch.Generator().manual_seed(0)
+    for bits in (2, 3, 4, 6, 8):
+        for n in (8, 40, 92, 250):
+            c = torch.randint(0, 1 << bits, (5, n), generator=g, dtype=torch.int32)
+            s = F.pack_stream(c, bits)
+            assert s.shape[1] == (n * bits + 7) // 8
+            assert torch.equal(F.unpack_stream(s, n, bits), c)
+            assert np.array_equal(s.numpy(), R._pack_stream(c.numpy(), bits))
+
+
+# ------------------------------------------------------------------ C ABI
+def test_library_exports_every_declared_symbol():
+    hdr = open(os.path.join(ROOT, "include", "cbk.h")).read()
+    names = set(re.findall(r"\b(cbk_[a-z_]+)\s*\(", hdr))
+    assert {"cbk_gemv", "cbk_gemm", "cbk_linear", "cbk_dequant", "cbk_workspace_bytes"} <= names
+    L = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(L, n), n
+    assert set(_lib.SIGNATURES) == names
+    assert _lib.lib().cbk_abi_version() == 1
+
+
+def test_descriptor_validation_and_strides():
+    L = _lib.lib()
+    for case in FIXED_CASES:
+        layout, bits, group, keep = case
+        for N in (128, 4096, 5376, 14336, 21504):
+            d = F.CbkDesc(K=16, N=N, layout=layout, bits=bits, group=group, keep=keep)
+            assert L.cbk_row_stride(ctypes.byref(d)) == R.row_stride(layout, N, bits, group, keep or None)
+    d = F.CbkDesc(K=16, N=4096, layout=F.BLK1632_4)
+    o = F.CbkDesc()
+    assert L.cbk_desc_check(ctypes.byref(d), ctypes.byref(o)) == 0 and (o.bits, o.group, o.keep) == (4, 128, 16)
+    assert L.cbk_stream_bytes(ctypes.byref(d), 0) == 16 * 4096 * 3 // 8 + 16 * 32 * 3
+    bad = [F.CbkDesc(K=16, N=4096, layout=11), F.CbkDesc(K=16, N=4096, layout=F.BLKC, bits=5, group=128, keep=16),
+           F.CbkDesc(K=16, N=4096, layout=F.BLKC, bits=4, group=32, keep=16),
+           F.CbkDesc(K=16, N=4096, layout=F.BLKC, bits=4, group=64, keep=33),
+           F.CbkDesc(K=16, N=4096, layout=F.BF16)]
+    for b in bad:
+        assert L.cbk_desc_check(ctypes.byref(b), ctypes.byref(o)) == -2
+    assert L.cbk_desc_check(ctypes.byref(F.CbkDesc(K=16, N=4000, layout=F.DENSE4)), ctypes.byref(o)) == -3
+    assert L.cbk_desc_check(ctypes.byref(F.CbkDesc(K=0, N=4096, layout=F.DENSE4)), ctypes.byref(o)) == -3
+    assert L.cbk_desc_check(None, ctypes.byref(o)) == -1
+
+
+def test_entry_points_reject_bad_arguments_before_any_launch():
+    L = _lib.lib()
+    d = F.CbkDesc(K=16, N=256, layout=F.BLK1632_4)
+    # NULL device arrays
+    assert L.cbk_gemv(ctypes.byref(d), None, 1, 1, 256, None, 0, 16, None, None, 0, None) == -1
+    assert L.cbk_dequant(ctypes.byref(d), 0, 16, 1, None, 0, 256, None) == -1
+    d.data, d.scale, d.zero = 0x1000, 0x2000, 0x3000           # never dereferenced: checks fail first
+    assert L.cbk_gemv(ctypes.byref(d), None, 1, 1, 256, None, 0, 16, None, None, 0, None) == -1
+    assert L.cbk_gemv(ctypes.byref(d), 0x4000, 0, 1, 256, 0x5000, 0, 16, None, None, 0, None) == -5
+    assert L.cbk_gemv(ctypes.byref(d), 0x4000, 1, 17, 256, 0x5000, 0, 16, None, None, 0, None) == -3
+    assert L.cbk_gemv(ctypes.byref(d), 0x4000, 1, 1, 128, 0x5000, 0, 16, None, None, 0, None) == -3
+    assert L.cbk_gemv(ctypes.byref(d), 0x4004, 1, 1, 256, 0x5000, 0, 16, None, None, 0, None) == -4
+    assert L.cbk_gemm(ctypes.byref(d), 0x4000, 2, 300, 260, 0x5000, 2, 16, None, None, 0, None) == -4
+    assert L.cbk_dequant(ctypes.byref(d), 8, 16, 1, 0x5000, 0, 256, None) == -3
+    d.data = 0x1004
+    assert L.cbk_gemv(ctypes.byref(d), 0x4000, 1, 1, 256, 0x5000, 0, 16, None, None, 0, None) == -4
+    d.data, d.cs_rows = 0x1000, 1
+    assert L.cbk_gemv(ctypes.byref(d), 0x4000, 1, 1, 256, 0x5000, 0, 16, None, None, 0, None) == -1
+    assert b"aligned" in L.cbk_strerror(-4)
+
+
+def test_ops_refuse_to_run_without_gpu_tensors():
+    from cobalt_amd import ops
+    pm = F.synth_packed(16, 256, F.BLK1632_4, seed=1)
+    with pytest.raises(_lib.CbkError):
+        ops.linear(pm, torch.zeros(1, 256, dtype=torch.float16))
+    with pytest.raises(_lib.CbkError):
+        ops.dequant(pm)
+
+
+# ------------------------------------------------------------------ module plumbing
+class _FakeSQL(torch.nn.Module):
+    """Same buffers as the reference's SparseQuantLinear (benchmark_suite.py:1178-1198)."""
+
+    def __init__(self, W_q, scales, zeros, mask, scale2, bias, meta):
+        super().__init__()
+        for n, v in dict(W_q=W_q, scales=scales, zeros=zeros, mask=mask, scale2=scale2).items():
+            self.register_buffer(n, v)
+        self.bias = torch.nn.Parameter(bias) if bias is not None else None
+        self.meta = meta
+
+
+def _fake_sql(K, N, bits, group, block, seed):
+    raw = R.synth_raw_matrix(K, N, 0.5, bits, seed=seed, block=block, group=group)
+    keep = torch.from_numpy(R.unpack_bits(raw["mask"], N))
+    m = _FakeSQL(torch.from_numpy(raw["q"]).half(), torch.from_numpy(raw["scale"]).reshape(K, -1, 1),
+                 torch.from_numpy(raw["zero"]).reshape(K, -1, 1), keep.half(),
+                 torch.from_numpy(raw["col_scale"]).reshape(1, N), torch.randn(K).half(),
+                 {"nbits": bits, "group_size": group})
+    return m, raw
+
+
+def test_from_sparse_quant_linear_layout_choice_and_bytes():
+    m, raw = _fake_sql(16, 256, 4, 128, 32, 1)
+    cl = CobaltLinear.from_sparse_quant_linear(m)
+    p = cl.packed()
+    assert (p.layout, p.bits, p.group, p.keep) == (F.BLK1632_4, 4, 128, 16)
+    pk = R.pack_matrix(raw["mask"], raw["q"], raw["scale"], raw["zero"], R.BLK1632_4)
+    assert np.array_equal(p.array("data").numpy(), pk["data"])
+    assert np.array_equal(p.array("col_scale").numpy(), raw["col_scale"])
+    m2, _ = _fake_sql(16, 256, 3, 64, 0, 2)               # unconstrained mask -> dense stream
+    p2 = CobaltLinear.from_sparse_quant_linear(m2).packed()
+    assert (p2.layout, p2.bits, p2.group) == (F.DENSEB, 3, 64)
+    m3, _ = _fake_sql(16, 256, 2, 64, 32, 3)
+    p3 = CobaltLinear.from_sparse_quant_linear(m3).packed()
+    assert (p3.layout, p3.bits, p3.group, p3.keep) == (F.BLKC, 2, 64, 16)
+    assert cl.bias is not None and cl.in_features == 256 and cl.out_features == 16
+    assert "BLK1632_4" in repr(cl)
+    with pytest.raises(ValueError):
+        cl.set_forward_backend("pytorch")
+
+
+def test_state_dict_roundtrip_and_patch_model():
+    m, _ = _fake_sql(16, 256, 4, 128, 32, 4)
+    cl = CobaltLinear.from_sparse_quant_linear(m)
+    sd = cl.state_dict()
+    assert set(sd) == {"blob", "cbk_meta", "bias"}
+    cl2 = CobaltLinear(F.synth_packed(16, 256, F.BLK1632_4, seed=9), bias=torch.zeros(16).half())
+    cl2.load_state_dict(sd)
+    assert torch.equal(cl2.blob, cl.blob) and cl2.packed().offs == cl.packed().offs
+
+    net = torch.nn.Sequential(torch.nn.Linear(256, 16), torch.nn.ReLU())
+    net.add_module("inner", torch.nn.Sequential(torch.nn.Linear(256, 16)))
+    done = patch_model(net, lambda name, mod: cl if isinstance(mod, torch.nn.Linear) and name == "inner.0" else None)
+    assert done == ["inner.0"] and net.inner[0] is cl
+    done = patch_model(net, {"0": cl2})
+    assert done == ["0"] and net[0] is cl2
+    with pytest.raises(TypeError):
+        F.dtype_code(torch.float64)
