@@ -73,6 +73,7 @@ static int to_dmat(const cbk_desc* in, DMat* m, bool need_device_ptrs) {
   m->K = d.K; m->N = d.N; m->G = d.N / d.group;
   m->layout = d.layout; m->bits = d.bits; m->group = d.group; m->keep = d.keep;
   m->cs_rows = d.cs_rows; m->cs_split0 = d.cs_split0; m->cs_split1 = d.cs_split1;
+  m->flags = d.flags;
   m->stride = (uint32_t)stride_of(d);
   m->code_off = family_of(d.layout) == FAM_DENSE ? 0u : (uint32_t)(d.N / 8);
   return CBK_OK;

@@ -26,6 +26,7 @@ struct DMat {
   int K, N, G;
   int layout, bits, group, keep;
   int cs_rows, cs_split0, cs_split1;
+  int flags;
   uint32_t stride;           // bytes per row (fixed-stride layouts)
   uint32_t code_off;         // byte offset of the code plane inside a row
 };

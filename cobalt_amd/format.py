@@ -31,6 +31,7 @@ _BLK = (BLK1632_4, BLK1632_6, BLKC)
 _SPARSE = (SPARSE4, SPARSE4X, SPARSE4E)
 
 F32, F16, BF16T = 0, 1, 2
+FLAG_ZERO_LE_128 = 1
 
 
 def dtype_code(dt: torch.dtype) -> int:
@@ -50,7 +51,7 @@ class CbkDesc(ctypes.Structure):
                 ("K", ctypes.c_int32), ("N", ctypes.c_int32), ("layout", ctypes.c_int32),
                 ("bits", ctypes.c_int32), ("group", ctypes.c_int32), ("keep", ctypes.c_int32),
                 ("cs_rows", ctypes.c_int32), ("cs_split0", ctypes.c_int32), ("cs_split1", ctypes.c_int32),
-                ("reserved", ctypes.c_int32)]
+                ("flags", ctypes.c_int32)]
 
 
 def _align(x: int, a: int) -> int:
@@ -190,6 +191,7 @@ class PackedMatrix:
     data_bytes: int = 0
     n_survivors: int = 0
     n_zero_fixed: int = 0
+    flags: int = 0
     meta: dict = field(default_factory=dict)
 
     @property
@@ -203,7 +205,7 @@ class PackedMatrix:
     def to(self, device) -> "PackedMatrix":
         return PackedMatrix(self.blob.to(device), dict(self.offs), self.K, self.N, self.layout, self.bits,
                             self.group, self.keep, self.cs_rows, self.cs_splits, self.data_bytes,
-                            self.n_survivors, self.n_zero_fixed, dict(self.meta))
+                            self.n_survivors, self.n_zero_fixed, self.flags, dict(self.meta))
 
     def clone(self) -> "PackedMatrix":
         p = self.to(self.device)
@@ -239,6 +241,7 @@ class PackedMatrix:
         d.K, d.N, d.layout = self.K, self.N, self.layout
         d.bits, d.group, d.keep = self.bits, self.group, self.keep
         d.cs_rows, d.cs_split0, d.cs_split1 = self.cs_rows, self.cs_splits[0], self.cs_splits[1]
+        d.flags = self.flags
         return d
 
 
@@ -332,8 +335,9 @@ def pack_raw(mask_bits: Optional[torch.Tensor], q: torch.Tensor, scale: torch.Te
         cs_rows = cs.shape[0]
         arrays["col_scale"] = cs
     blob, offs = _assemble(arrays, dev)
+    flags = FLAG_ZERO_LE_128 if int(out_zero.max()) <= 128 else 0
     return PackedMatrix(blob, offs, K, N, layout, bits, group, kpb, cs_rows, tuple(cs_splits),
-                        K * stride, n_surv, n_fixed)
+                        K * stride, n_surv, n_fixed, flags)
 
 
 def from_arrays(data, scale, zero, col_scale, K, N, layout, bits=None, group=None, keep=None, row_off=None,
@@ -353,8 +357,9 @@ def from_arrays(data, scale, zero, col_scale, K, N, layout, bits=None, group=Non
         cs_rows = cs.shape[0]
         arrays["col_scale"] = cs.contiguous().reshape(-1).view(torch.uint8)
     blob, offs = _assemble(arrays, dev)
+    flags = FLAG_ZERO_LE_128 if int(torch.as_tensor(zero).reshape(-1).view(torch.uint8).max()) <= 128 else 0
     return PackedMatrix(blob, offs, K, N, layout, bits, group, kpb, cs_rows, tuple(cs_splits),
-                        data.numel() - BLOB_TAIL)
+                        data.numel() - BLOB_TAIL, flags=flags)
 
 
 def synth_packed(K: int, N: int, layout: int, bits=None, group=None, keep=None, seed: int = 0,
@@ -394,4 +399,5 @@ def synth_packed(K: int, N: int, layout: int, bits=None, group=None, keep=None, 
     if cs_rows:
         arrays["col_scale"] = (torch.rand(cs_rows, N, generator=g, device=dev) * 1.5 + 0.5).half()
     blob, offs = _assemble(arrays, dev)
-    return PackedMatrix(blob, offs, K, N, layout, bits, group, kpb, cs_rows, (0, 0), K * stride, n_surv, 0)
+    return PackedMatrix(blob, offs, K, N, layout, bits, group, kpb, cs_rows, (0, 0), K * stride, n_surv, 0,
+                        FLAG_ZERO_LE_128)

@@ -14,7 +14,7 @@ from . import ops
 
 _META_FIELDS = ("K", "N", "layout", "bits", "group", "keep", "cs_rows", "cs_split0", "cs_split1",
                 "data_bytes", "off_data", "off_row_off", "off_scale", "off_zero", "off_col_scale",
-                "n_survivors")
+                "n_survivors", "flags")
 
 
 class CobaltLinear(nn.Module):
@@ -26,7 +26,7 @@ class CobaltLinear(nn.Module):
         self.register_buffer("cbk_meta", torch.tensor(
             [packed.K, packed.N, packed.layout, packed.bits, packed.group, packed.keep, packed.cs_rows,
              packed.cs_splits[0], packed.cs_splits[1], packed.data_bytes, o["data"], o.get("row_off", -1),
-             o["scale"], o["zero"], o.get("col_scale", -1), packed.n_survivors], dtype=torch.int64))
+             o["scale"], o["zero"], o.get("col_scale", -1), packed.n_survivors, packed.flags], dtype=torch.int64))
         self.bias = nn.Parameter(bias.detach().clone(), requires_grad=False) if bias is not None else None
         self.meta = dict(meta or {})
         self._backend = "hip"
@@ -78,7 +78,8 @@ class CobaltLinear(nn.Module):
         if d["off_col_scale"] >= 0:
             offs["col_scale"] = d["off_col_scale"]
         return F.PackedMatrix(self.blob, offs, d["K"], d["N"], d["layout"], d["bits"], d["group"], d["keep"],
-                              d["cs_rows"], (d["cs_split0"], d["cs_split1"]), d["data_bytes"], d["n_survivors"])
+                              d["cs_rows"], (d["cs_split0"], d["cs_split1"]), d["data_bytes"], d["n_survivors"],
+                              flags=d["flags"])
 
     def _apply(self, fn, recurse=True):
         out = super()._apply(fn, recurse)

@@ -43,6 +43,8 @@ enum cbk_layout {
                         bits 4 == DENSE4, bits 8 == DENSE8                               */
 };
 
+#define CBK_FLAG_ZERO_LE_128 1
+
 enum cbk_dtype { CBK_F32 = 0, CBK_F16 = 1, CBK_BF16T = 2 };
 
 enum cbk_status {
@@ -68,7 +70,12 @@ enum cbk_status {
  *   cs_rows   1: one vector.  2: fused gate/up, row k uses vector k&1.  3: fused q|k|v, rows
  *             [0,cs_split0) use vector 0, [cs_split0, cs_split0+cs_split1) vector 1, the rest 2
  *             (cobalt_format.h:77-99, docs/FORMAT.md:134-151).
- *   bits/group/keep  must be given for layouts 8/9; for 0-7 they may be 0 (implied). */
+ *   bits/group/keep  must be given for layouts 8/9; for 0-7 they may be 0 (implied).
+ *   flags     CBK_FLAG_ZERO_LE_128: the caller guarantees that every stored zero point is
+ *             <= 128 (always true for an on-grid zero point of a 2/3/4-bit code, and for the
+ *             reference's off-grid probe, src/cobaltkernel/test_gemv.py:428-431).  The int8
+ *             matrix-core decode kernel needs q - zero to fit a signed byte; without the flag
+ *             cbk_gemv runs the slower float row kernel, which takes any uint8 zero point. */
 typedef struct cbk_desc {
   const void* data;
   const void* row_off;
@@ -82,7 +89,7 @@ typedef struct cbk_desc {
   int32_t keep;
   int32_t cs_rows;
   int32_t cs_split0, cs_split1;
-  int32_t reserved;
+  int32_t flags;
 } cbk_desc;
 
 int cbk_abi_version(void);
