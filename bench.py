@@ -66,6 +66,9 @@ def main():
     ap.add_argument("--keep", type=int, default=16)
     ap.add_argument("--group", type=int, default=128)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--launch", default="phase", choices=["matrix", "phase", "layer"],
+                    help="GEMVs per launch: one matrix, one dependency phase (qkv | o | gate,up | down), or the layer set")
+    ap.add_argument("--no-graph", action="store_true", help="launch from the host instead of replaying HIP graphs")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -90,42 +93,66 @@ def main():
           for _, _, N in shapes}
     ys = [torch.empty(M, K, dtype=dt, device=dev) for _, K, _ in shapes]
     step_bytes = sum(algorithmic_bytes(pm, M) for pm in sets[0])
-    ws = [ops.workspace_for(pm, M) for pm in sets[0]]
 
     import ctypes
     from cobalt_amd import _lib
     L = _lib.lib()
-    stream = torch.cuda.current_stream(dev)
+    stream = torch.cuda.Stream(dev)
     sp = stream.cuda_stream
-    calls = []
+    xdt = F.dtype_code(dt)
+    groups = {"matrix": [[i] for i in range(len(shapes))],
+              "phase": [[0, 1, 2], [3], [4, 5], [6]],          # qkv | o | gate,up | down
+              "layer": [list(range(len(shapes)))]}[a.launch]
+    P = ctypes.c_void_p
+    calls = []                                                  # per layer set: list of batched calls
+    keep_alive = []
     for s in sets:
         cs = []
-        for pm, (_, K, N), y, w in zip(s, shapes, ys, ws):
-            d = pm.desc()
-            cs.append((d, xs[N].data_ptr(), y.data_ptr(), N, K, w.data_ptr() if w is not None else None,
-                       w.numel() if w is not None else 0))
+        for g in groups:
+            n = len(g)
+            descs = (F.CbkDesc * n)(*[s[i].desc() for i in g])
+            xp = (P * n)(*[xs[shapes[i][2]].data_ptr() for i in g])
+            yp = (P * n)(*[ys[i].data_ptr() for i in g])
+            ldx = (ctypes.c_int64 * n)(*[shapes[i][2] for i in g])
+            ldy = (ctypes.c_int64 * n)(*[shapes[i][1] for i in g])
+            need = L.cbk_gemv_batch_workspace_bytes(n, descs, M)
+            w = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
+            keep_alive.append((descs, xp, yp, ldx, ldy, w))
+            cs.append((n, descs, xp, ldx, yp, ldy, w.data_ptr(), w.numel()))
         calls.append(cs)
-    xdt = F.dtype_code(dt)
 
     def step(i):
-        for d, xp, yp, N, K, wp, wn in calls[i % n_copies]:
-            rc = L.cbk_gemv(ctypes.byref(d), xp, xdt, M, N, yp, xdt, K, None, wp, wn, sp)
+        for n, descs, xp, ldx, yp, ldy, wp, wn in calls[i % n_copies]:
+            rc = L.cbk_gemv_batch(n, descs, xp, ldx, xdt, M, yp, ldy, xdt, None, wp, wn, sp)
             if rc:
                 raise RuntimeError(L.cbk_strerror(rc).decode())
 
-    for i in range(a.warmup):
-        step(i)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for i in range(a.steps):
-        step(a.warmup + i)
-    e1.record(stream)
-    torch.cuda.synchronize()
+    launches = len(groups)
+    with torch.cuda.stream(stream):
+        for i in range(n_copies):
+            step(i)
+        stream.synchronize()
+        graphs = None
+        if not a.no_graph:                                      # one HIP graph per distinct layer set
+            graphs = []
+            for i in range(n_copies):
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=stream):
+                    step(i)
+                graphs.append(g)
+        run = (lambda i: graphs[i % n_copies].replay()) if graphs else step
+        for i in range(a.warmup):
+            run(i)
+        stream.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for i in range(a.steps):
+            run(a.warmup + i)
+        e1.record(stream)
+        stream.synchronize()
     ms = e0.elapsed_time(e1)
     ms_per_step = ms / a.steps
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
-    launches = len(shapes)
     us_per_launch = ms_per_step * 1e3 / launches
     bytes_per_launch = step_bytes / launches
     achieved = bytes_per_launch / (us_per_launch * 1e-6) / 1e9
@@ -140,7 +167,8 @@ def main():
         "config": {"workload": f"{a.workload} decode layer set, 7 GEMVs, M={M}, sparsity {1 - a.keep / 32:.4g}, "
                                f"{a.bits}-bit, group {a.group}, layout {F.LAYOUT_NAME[layout]}, {bpw:.4f} bpw",
                    "layer_set_bytes": step_bytes, "distinct_layer_sets": n_copies,
-                   "launches_per_step": launches},
+                   "launches_per_step": launches, "launch_grouping": a.launch,
+                   "hip_graph": not a.no_graph},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                      "kernel": "decode GEMV", "avg_launch_us": round(us_per_launch, 3),

@@ -7,7 +7,7 @@ from __future__ import annotations
 import ctypes
 import os
 
-from .format import CbkDesc
+from .format import CbkDesc  # noqa: F401 (re-exported for callers that build descriptor arrays)
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcbk_hip.so")
@@ -28,6 +28,10 @@ SIGNATURES = {
                                    ctypes.c_int64, _P]),
     "cbk_gemv": (ctypes.c_int, _MM),
     "cbk_gemm": (ctypes.c_int, _MM),
+    "cbk_gemv_batch_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, _DP, ctypes.c_int]),
+    "cbk_gemv_batch": (ctypes.c_int, [ctypes.c_int, _DP, ctypes.POINTER(_P), ctypes.POINTER(ctypes.c_int64),
+                                      ctypes.c_int, ctypes.c_int, ctypes.POINTER(_P), ctypes.POINTER(ctypes.c_int64),
+                                      ctypes.c_int, ctypes.POINTER(_P), _P, ctypes.c_size_t, _P]),
     "cbk_linear": (ctypes.c_int, _MM),
 }
 

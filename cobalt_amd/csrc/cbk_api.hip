@@ -6,10 +6,13 @@ namespace cbk {
 int launch_dequant(const DMat&, int, int, int, void*, int, int64_t, hipStream_t);
 int launch_gemv_generic(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*,
                         hipStream_t);
-int launch_gemv_fast(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*, void*,
-                     size_t, hipStream_t);
+struct GvCall { DMat m; const void* x; int64_t ldx; void* y; int64_t ldy; const void* bias; };
+int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, void* ws, size_t ws_bytes,
+                           hipStream_t);
 bool gemv_fast_takes(const DMat&, int M);
+bool gemv_same_config(const DMat&, const DMat&);
 size_t gemv_fast_workspace(const DMat&, int M);
+constexpr int kMaxBatch = 8;
 int launch_gemm(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*,
                 hipStream_t);
 
@@ -74,6 +77,8 @@ static int to_dmat(const cbk_desc* in, DMat* m, bool need_device_ptrs) {
   m->layout = d.layout; m->bits = d.bits; m->group = d.group; m->keep = d.keep;
   m->cs_rows = d.cs_rows; m->cs_split0 = d.cs_split0; m->cs_split1 = d.cs_split1;
   m->flags = d.flags;
+  m->tiled = (d.flags & CBK_FLAG_TILED16) ? 1 : 0;
+  if (m->tiled && sparse) return CBK_ERR_UNSUPPORTED;
   m->stride = (uint32_t)stride_of(d);
   m->code_off = family_of(d.layout) == FAM_DENSE ? 0u : (uint32_t)(d.N / 8);
   return CBK_OK;
@@ -132,8 +137,15 @@ size_t cbk_stream_bytes(const cbk_desc* in, size_t sparse_data_bytes) {
 size_t cbk_workspace_bytes(const cbk_desc* in, int M) {
   DMat m;
   if (to_dmat(in, &m, false)) return 0;
-  if (M >= 1 && M <= 16 && gemv_fast_takes(m, M)) return gemv_fast_workspace(m, M);
+  const int mc = M > 4 ? 4 : M;
+  if (M >= 1 && M <= 16 && gemv_fast_takes(m, mc)) return gemv_fast_workspace(m, mc);
   return 0;
+}
+
+size_t cbk_gemv_batch_workspace_bytes(int n, const cbk_desc* descs, int M) {
+  size_t total = 0;
+  for (int i = 0; i < n; ++i) total += cbk_workspace_bytes(descs + i, M);
+  return total;
 }
 
 int cbk_dequant(const cbk_desc* in, int row0, int nrows, int with_col_scale, void* out, int out_dtype,
@@ -147,6 +159,56 @@ int cbk_dequant(const cbk_desc* in, int row0, int nrows, int with_col_scale, voi
   return launch_dequant(m, row0, nrows, with_col_scale, out, out_dtype, ld_out, (hipStream_t)stream);
 }
 
+int cbk_gemv_batch(int n, const cbk_desc* descs, const void* const* xs, const int64_t* ldxs, int x_dtype, int M,
+                   void* const* ys, const int64_t* ldys, int y_dtype, const void* const* biases,
+                   void* workspace, size_t workspace_bytes, void* stream) {
+  if (n < 1 || n > kMaxBatch) return CBK_ERR_SHAPE;
+  if (!descs || !xs || !ldxs || !ys || !ldys) return CBK_ERR_NULL;
+  if (M > 16) return CBK_ERR_SHAPE;
+  GvCall calls[kMaxBatch];
+  bool fast = true;
+  for (int i = 0; i < n; ++i) {
+    int rc = to_dmat(descs + i, &calls[i].m, true);
+    if (rc) return rc;
+    rc = check_io(xs[i], x_dtype, M, ldxs[i], ys[i], y_dtype, ldys[i], calls[i].m.N, calls[i].m.K);
+    if (rc) return rc;
+    calls[i].x = xs[i]; calls[i].ldx = ldxs[i]; calls[i].y = ys[i]; calls[i].ldy = ldys[i];
+    calls[i].bias = biases ? biases[i] : nullptr;
+    fast = fast && gemv_fast_takes(calls[i].m, M > 4 ? 4 : M) && gemv_same_config(calls[0].m, calls[i].m);
+  }
+  hipStream_t st = (hipStream_t)stream;
+  if (fast) {
+    size_t need = 0;
+    for (int i = 0; i < n; ++i) need += gemv_fast_workspace(calls[i].m, M > 4 ? 4 : M);
+    if (!workspace || workspace_bytes < need) return CBK_ERR_WORKSPACE;
+    if ((uintptr_t)workspace & 255) return CBK_ERR_ALIGN;
+    const size_t ysz = y_dtype == CBK_F32 ? 4 : 2;
+    for (int m0 = 0; m0 < M; m0 += 4) {                 // at most 4 activation rows per launch
+      const int mc = M - m0 < 4 ? M - m0 : 4;
+      GvCall part[kMaxBatch];
+      for (int i = 0; i < n; ++i) {
+        part[i] = calls[i];
+        part[i].x = (const uint8_t*)calls[i].x + (size_t)m0 * calls[i].ldx * 2;
+        part[i].y = (uint8_t*)calls[i].y + (size_t)m0 * calls[i].ldy * ysz;
+      }
+      int rc = launch_gemv_fast_batch(n, part, x_dtype, mc, y_dtype, workspace, workspace_bytes, st);
+      if (rc) return rc;
+    }
+    return CBK_OK;
+  }
+  // mixed or unsupported configurations: one matrix at a time
+  size_t off = 0;
+  for (int i = 0; i < n; ++i) {
+    const size_t need = cbk_workspace_bytes(descs + i, M);
+    if (need && (!workspace || off + need > workspace_bytes)) return CBK_ERR_WORKSPACE;
+    int rc = cbk_gemv(descs + i, xs[i], x_dtype, M, ldxs[i], ys[i], y_dtype, ldys[i], biases ? biases[i] : nullptr,
+                      need ? (uint8_t*)workspace + off : nullptr, need, stream);
+    if (rc) return rc;
+    off += need;
+  }
+  return CBK_OK;
+}
+
 int cbk_gemv(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ldx, void* y, int y_dtype,
              int64_t ldy, const void* bias, void* workspace, size_t workspace_bytes, void* stream) {
   DMat m;
@@ -155,13 +217,8 @@ int cbk_gemv(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ldx,
   rc = check_io(x, x_dtype, M, ldx, y, y_dtype, ldy, m.N, m.K);
   if (rc) return rc;
   if (M > 16) return CBK_ERR_SHAPE;
-  if (gemv_fast_takes(m, M)) {
-    const size_t need = gemv_fast_workspace(m, M);
-    if (need && (!workspace || workspace_bytes < need)) return CBK_ERR_WORKSPACE;
-    if ((uintptr_t)workspace & 255) return CBK_ERR_ALIGN;
-    return launch_gemv_fast(m, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, workspace, workspace_bytes,
-                            (hipStream_t)stream);
-  }
+  if (gemv_fast_takes(m, M > 4 ? 4 : M))
+    return cbk_gemv_batch(1, in, &x, &ldx, x_dtype, M, &y, &ldy, y_dtype, &bias, workspace, workspace_bytes, stream);
   return launch_gemv_generic(m, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, (hipStream_t)stream);
 }
 

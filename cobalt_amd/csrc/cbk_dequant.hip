@@ -15,12 +15,12 @@ __global__ __launch_bounds__(256) void dequant_fixed_kernel(DMat m, int row0, in
   if (gid >= (int64_t)nrows * NB) return;
   const int r = (int)(gid / NB), t = (int)(gid % NB);
   const int k = row0 + r;
-  const uint8_t* row = m.data + (size_t)k * m.stride;
+  const RowView row = row_view(m, k);
   int q[32];
   const uint32_t keep = decode_block32(m, row, t, q);
   const int g = (t * BLOCK) / m.group;
-  const float s = h2f(m.scale[(size_t)k * m.G + g]);
-  const float z = (float)m.zero[(size_t)k * m.G + g];
+  const float s = h2f(m.scale[meta_index(m, k, g)]);
+  const float z = (float)m.zero[meta_index(m, k, g)];
   const uint16_t* cs = (with_cs && m.cs) ? m.cs + (size_t)cs_row_of(m, k) * m.N + t * BLOCK : nullptr;
   const bool dense = family_of(m.layout) == FAM_DENSE;
 #pragma unroll

@@ -1,6 +1,11 @@
 // Device-side view of a CBK1 packed matrix and the bit-level readers every kernel shares.
 // gfx950 only.  Byte layouts follow docs/FORMAT.md:83-122 of the reference for layouts 0-7;
 // layouts 8 (BLKC) and 9 (DENSEB) are one LSB-first bit stream per row (see include/cbk.h).
+//
+// Two byte orders of the same rows are read: the reference's row-major order, and the
+// 16-row tile-interleaved order (CBK_FLAG_TILED16) in which 16-byte unit u of row k sits at
+// (k/16)*16*stride + (u*16 + k%16)*16, so that the sixteen rows a wavefront decodes
+// together are one contiguous run in HBM.  Kernels address rows only through RowView.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
@@ -27,6 +32,7 @@ struct DMat {
   int layout, bits, group, keep;
   int cs_rows, cs_split0, cs_split1;
   int flags;
+  int tiled;                 // 1: 16-row tile-interleaved byte order
   uint32_t stride;           // bytes per row (fixed-stride layouts)
   uint32_t code_off;         // byte offset of the code plane inside a row
 };
@@ -40,6 +46,27 @@ __host__ __device__ inline int family_of(int layout) {
     case CBK_BLK1632_6: return FAM_BLK6;
     default: return FAM_SPARSE;
   }
+}
+
+// One row of a fixed-stride matrix in either byte order: unit(u) is the address of its
+// 16-byte unit u, dword(d) its d-th little-endian dword.
+struct RowView {
+  const uint8_t* base;
+  uint32_t ustride;          // bytes from one 16-byte unit of the row to the next
+  __device__ inline const uint8_t* unit(uint32_t u) const { return base + (size_t)u * ustride; }
+  __device__ inline uint32_t dword(uint32_t d) const {
+    return *(const uint32_t*)(base + (size_t)(d >> 2) * ustride + (d & 3u) * 4u);
+  }
+};
+__device__ inline RowView row_view(const DMat& m, int k) {
+  RowView r;
+  if (m.tiled) { r.base = m.data + (size_t)(k >> 4) * m.stride * 16 + (size_t)(k & 15) * 16; r.ustride = 256; }
+  else { r.base = m.data + (size_t)k * m.stride; r.ustride = 16; }
+  return r;
+}
+// index of the scale / zero entry of (row k, group g)
+__device__ inline size_t meta_index(const DMat& m, int k, int g) {
+  return m.tiled ? ((size_t)(k >> 4) * m.G + g) * 16 + (k & 15) : (size_t)k * m.G + g;
 }
 
 // ------------------------------------------------------------------ scalar conversions
@@ -73,31 +100,31 @@ __device__ inline int cs_row_of(const DMat& m, int k) {
 }
 
 // ------------------------------------------------------------------ generic 32-column reader
-// Codes of the 32 columns of block t of the row starting at `row` (fixed-stride layouts).
-// q[p] is the stored code for a kept column and 0 for a pruned one; the return value is
-// the keep bitmap (all ones for the dense family, whose pruned columns hold the zero point).
-// Everything is indexed with compile-time constants after unrolling, so q[] stays in VGPRs.
-__device__ inline uint32_t decode_block32(const DMat& m, const uint8_t* row, int t, int (&q)[32]) {
+// Codes of the 32 columns of block t of a row (fixed-stride layouts).  q[p] is the stored code
+// for a kept column and 0 for a pruned one; the return value is the keep bitmap (all ones for
+// the dense family, whose pruned columns hold the zero point).  Everything is indexed with
+// compile-time constants after unrolling, so q[] stays in VGPRs.
+__device__ inline uint32_t decode_block32(const DMat& m, const RowView& row, int t, int (&q)[32]) {
   const int fam = family_of(m.layout);
   const int b = m.bits;
   const uint32_t cm = (1u << b) - 1u;
   if (fam == FAM_DENSE) {
     // 32 codes = b dwords, dword aligned; code p at bits [p*b, p*b+b)
-    const uint32_t* w = (const uint32_t*)row + (size_t)t * b;
+    const uint32_t d0 = (uint32_t)t * b;
     uint64_t cur = 0; int have = 0, wi = 0;
 #pragma unroll
     for (int p = 0; p < 32; ++p) {
-      if (have < b) { cur |= ((uint64_t)w[wi++]) << have; have += 32; }
+      if (have < b) { cur |= ((uint64_t)row.dword(d0 + wi++)) << have; have += 32; }
       q[p] = (int)((uint32_t)cur & cm);
       cur >>= b; have -= b;
     }
     return 0xffffffffu;
   }
-  const uint32_t keep = ((const uint32_t*)row)[t];
+  const uint32_t keep = row.dword(t);
   if (fam == FAM_BLK6) {
-    const uint32_t* nib = (const uint32_t*)(row + (m.N >> 3)) + 2 * t;
-    uint64_t lo = (uint64_t)nib[0] | ((uint64_t)nib[1] << 32);
-    const uint32_t hw = ((const uint32_t*)(row + 3 * (m.N >> 3)))[t];
+    const uint32_t nd = (uint32_t)(m.N >> 5);              // dwords of the mask plane
+    uint64_t lo = (uint64_t)row.dword(nd + 2 * t) | ((uint64_t)row.dword(nd + 2 * t + 1) << 32);
+    const uint32_t hw = row.dword(3 * nd + t);
     uint32_t he = hw & 0xffffu, ho = hw >> 16;
     int i = 0;
 #pragma unroll
@@ -111,11 +138,11 @@ __device__ inline uint32_t decode_block32(const DMat& m, const uint8_t* row, int
   }
   // FAM_BLK: survivor i of block t at bits [(t*keep+i)*b, ...) of the code plane
   const uint32_t sb = (uint32_t)t * (uint32_t)(m.keep * b);
-  const uint32_t* w = (const uint32_t*)(row + m.code_off) + (sb >> 5);
+  const uint32_t d0 = (m.code_off >> 2) + (sb >> 5);
   const uint32_t sh = sb & 31u;
   uint32_t e[5];
 #pragma unroll
-  for (int i = 0; i < 5; ++i) e[i] = w[i];               // <= 128 code bits + 31 bits of skew
+  for (int i = 0; i < 5; ++i) e[i] = row.dword(d0 + i);    // <= 128 code bits + 31 bits of skew
   uint64_t lo = ((uint64_t)__builtin_amdgcn_alignbit(e[1], e[0], sh)) |
                 ((uint64_t)__builtin_amdgcn_alignbit(e[2], e[1], sh) << 32);
   uint64_t hi = ((uint64_t)__builtin_amdgcn_alignbit(e[3], e[2], sh)) |

@@ -40,7 +40,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(DMat m, const uint16_t* __res
   // this thread's weight block: row r0 + tid/2, 32-column block (c0/32 + tid%2)
   const int wrow = r0 + (tid >> 1);
   const bool wrow_ok = wrow < m.K;
-  const uint8_t* rowp = m.data + (size_t)(wrow_ok ? wrow : 0) * m.stride;
+  const RowView rowp = row_view(m, wrow_ok ? wrow : 0);
   const uint16_t* csp = m.cs ? m.cs + (size_t)cs_row_of(m, wrow_ok ? wrow : 0) * m.N : nullptr;
   const bool dense = family_of(m.layout) == FAM_DENSE;
 
@@ -72,8 +72,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(DMat m, const uint16_t* __res
         int q[32];
         const uint32_t keep = decode_block32(m, rowp, t, q);
         const int g = (t * BLOCK) / m.group;
-        const float s = h2f(m.scale[(size_t)wrow * m.G + g]);
-        const float z = (float)m.zero[(size_t)wrow * m.G + g];
+        const float s = h2f(m.scale[meta_index(m, wrow, g)]);
+        const float z = (float)m.zero[meta_index(m, wrow, g)];
 #pragma unroll
         for (int p = 0; p < 32; p += 2) {
           float w0 = __fmul_rn((float)q[p] - z, s), w1 = __fmul_rn((float)q[p + 1] - z, s);

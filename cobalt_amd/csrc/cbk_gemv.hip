@@ -7,7 +7,8 @@
 // for a pruned one) sixteen at a time, and hands each 16-byte fragment to
 // v_mfma_i32_16x16x64_i8 as the B operand.  The A operand is the activation vector in
 // block fixed point: per 128-column chunk, x' = x * col_scale is written as
-// delta * (256*hi + lo) with two int8 digits (|x' - delta*X| <= max|x'| / 65024).  The
+// delta * (65536*d2 + 256*d1 + d0) with three int8 digits (|x' - delta*X| <= max|x'| / 2^24,
+// i.e. float32 resolution relative to the largest activation of the chunk).  The
 // matrix core produces exact int32 dot products per (row, chunk, digit); one float FMA per
 // row and quantisation group applies scale * delta.  A pruned column multiplies a literal
 // zero byte, so it contributes exactly 0 whatever the zero point holds.
@@ -16,10 +17,12 @@
 // and on the 128-column chunk 4*S + l/16 of macro-step S (512 columns).  The four lane
 // quarters are four different quantisation groups, which one MFMA would add up; the rows of
 // the A operand therefore carry (activation row, quarter, digit) variants that are non-zero
-// in one quarter only, and the 16x16 result keeps the groups apart.  The eight wavefronts of
-// a workgroup split the macro-steps of a tile and combine through LDS in a fixed order, so
-// results are run-to-run identical.  Workgroups are persistent over row tiles; the
-// activation digits and the byte-permute selector table live in LDS for the whole launch.
+// in one quarter only, and the 16x16 result keeps the groups apart.  One persistent workgroup
+// of sixteen wavefronts per CU owns a contiguous range of row tiles; a tile is cut into up
+// to 16 column parts and the (tile, part) items are dealt round-robin to the wavefronts, which
+// run without a barrier per tile: the partial sums of a tile meet in an LDS slot and the
+// wavefront that arrives last adds them in part order, so results are run-to-run identical.
+// The activation digits and the byte-permute selector table live in LDS for the whole launch.
 //
 // Expansion of the bitmap.  For one mask byte (8 columns, r survivors before it in its
 // 32-column block) the survivor codes r .. r+7 are shifted out of the block's code bits,
@@ -30,43 +33,43 @@
 // Reference semantics: cbk::gemv_blk1632_multi / gemv_dense4_multi
 // (src/cobaltkernel/csrc/cobalt_gemv.cuh:617-712, :839-1123): same sums, other machinery.
 #include <atomic>
+#include <cstdio>
+#include <cstdlib>
 #include "cbk_device.h"
 
 namespace cbk {
 
-constexpr int GV_WAVES = 8;
+constexpr int GV_WAVES = 16;
 constexpr int GV_THREADS = GV_WAVES * 64;
-constexpr int LUT_LANES = 16;                 // lane-private copies of the selector table
+#ifndef CBK_LUT_LANES
+#define CBK_LUT_LANES 8
+#endif
+constexpr int LUT_LANES = CBK_LUT_LANES;      // lane-private copies of the selector table
 constexpr int LUT_BYTES = 256 * LUT_LANES * 8;
 constexpr int ZERO_BYTES = 256;
-constexpr int X_LDS_BUDGET = 112 * 1024;      // activation digits: M * 2 * N bytes
-constexpr int GV_MAX_M = 8;
+constexpr int X_LDS_BUDGET = 112 * 1024;      // activation digits: M * 3 * N bytes (of 160 KB LDS)
+constexpr int NDIG = 3;                       // int8 digits per activation
+constexpr int GV_MAX_M = 4;
+constexpr int GV_MAX_BATCH = 8;               // matrices per launch
 
-// ------------------------------------------------------------------ selector tables
-struct SelTable { uint32_t lo[256], hi[256]; };
-
+// ------------------------------------------------------------------ selector table
+// Entry for mask byte mb: eight v_perm_b32 selector bytes, one per column.  A kept column
+// with r survivors before it in the byte selects pool byte idx(r); a pruned column selects
+// 0x0C, the constant 0x00.
 // kind 0: pool = {even-rank codes (bytes 0-3), odd-rank codes (bytes 4-7)}   (4-bit codes)
 // kind 1: pool = {c0,c4,c1,c5 | c2,c6,c3,c7}                                   (2-bit codes)
-constexpr SelTable make_table(int kind) {
-  SelTable t{};
-  for (int mb = 0; mb < 256; ++mb) {
-    uint32_t sel[8] = {};
-    int r = 0;
-    for (int p = 0; p < 8; ++p) {
-      if ((mb >> p) & 1) {
-        sel[p] = kind == 0 ? (uint32_t)((r >> 1) + 4 * (r & 1)) : (uint32_t)(((r & 3) << 1) | (r >> 2));
-        ++r;
-      } else {
-        sel[p] = 0x0Cu;                        // v_perm_b32: constant 0x00
-      }
-    }
-    t.lo[mb] = sel[0] | (sel[1] << 8) | (sel[2] << 16) | (sel[3] << 24);
-    t.hi[mb] = sel[4] | (sel[5] << 8) | (sel[6] << 16) | (sel[7] << 24);
+__device__ inline uint2 make_selectors(uint32_t mb, int kind) {
+  uint32_t lo = 0, hi = 0, r = 0;
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    const uint32_t idx = kind == 0 ? ((r >> 1) + 4u * (r & 1u)) : (((r & 3u) << 1) | (r >> 2));
+    const bool kp = (mb >> p) & 1u;
+    const uint32_t sel = kp ? idx : 0x0Cu;
+    if (p < 4) lo |= sel << (8 * p); else hi |= sel << (8 * (p - 4));
+    r += kp ? 1u : 0u;
   }
-  return t;
+  return make_uint2(lo, hi);
 }
-__device__ const SelTable g_sel4 = make_table(0);
-__device__ const SelTable g_sel2 = make_table(1);
 
 // ------------------------------------------------------------------ small helpers
 __device__ inline uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) {
@@ -112,7 +115,7 @@ __device__ inline uint32_t bias_pool(uint32_t codes, uint32_t nz) { return (code
 
 // ------------------------------------------------------------------ kernel configuration
 // BITS: code width.  KEEP: survivors per 32 columns, 0 = dense family.  GRP: group size.
-// MP: MFMA passes per fragment = ceil(M / 2).
+// MP: MFMA passes per fragment = activation rows M.
 template <int BITS, int KEEP, int GRP, int MP>
 struct Cfg {
   static constexpr bool DENSE = KEEP == 0;
@@ -120,289 +123,401 @@ struct Cfg {
   static constexpr int CHB = 4 * CB;                              // per 128-column chunk
   static constexpr bool ALIGNED = CHB % 32 == 0;
   static constexpr int ND = (CHB + 31) / 32;                      // dwords of chunk code bits
-  static constexpr int NL = ALIGNED ? ND : ND + 1;                // dwords loaded (skew)
-  static constexpr bool VEC16 = CHB % 128 == 0;                   // 16-byte aligned chunks
+  static constexpr bool VEC16 = CHB % 128 == 0;                   // chunks start on 16-byte units
+  static constexpr int NL = VEC16 ? ND : 4 * ((CHB + 254) / 128); // dwords loaded: whole units covering any skew
   static constexpr int NIB = DENSE ? 32 : KEEP;                   // codes per block
   static constexpr int SB = BITS == 3 ? 4 : BITS;                 // stream code width after expansion
   static constexpr int NW = (NIB * SB + 31) / 32;                 // dwords of a block's code stream
   static constexpr int NGC = 128 / GRP;                           // groups per chunk (1 or 2)
+  static constexpr int SEL_KIND = (BITS == 2) ? 1 : 0;
 };
 
-struct GvArgs {
+// One matrix of a batched launch.
+struct GvMat {
   DMat m;
-  const uint16_t* x;
-  int64_t ldx;
-  int M;
+  const int8_t* xq;        // activation digits [M][3][N] (most significant plane first)
+  const float* delta;      // [M][N/128 + 4], zero beyond N/128
   void* y;
-  int ydt;
-  int64_t ldy;
   const void* bias;
-  int xdt;
-  int ntiles;
+  int64_t ldy;
+  int ntiles;              // ceil(K / 16)
+  int nS;                  // macro-steps per tile = ceil(N / 512)
+  int cost0;               // sum of ntiles * nS over the matrices before this one
+  int spi, sk;             // macro-steps per work item, work items per tile
 };
 
-// Column order of the activation digits inside a 16-column fragment (dense family only):
-// the byte order in which the spread codes come out without a permute.
-template <int BITS, bool DENSE>
-__device__ constexpr int frag_col(int bi) {
-  if (!DENSE) return bi;
-  if (BITS == 2) return (bi >> 2) + 4 * (bi & 3);                                 // byte 4k+j <- column k+4j
+struct GvBatch {
+  GvMat mat[GV_MAX_BATCH];
+  int n, M, ydt, total_cost;
+  int xq_cap, delta_cap;   // LDS bytes reserved for digits / floats reserved for delta
+  int sk_cap, nslot, red_floats;   // reduction slots: nslot x sk_cap x M x 16 floats
+};
+
+// Column order of the activation digits inside a 16-column fragment: the byte order in which
+// the decoder emits the weights.  The bitmap layouts come out in column order (the permute
+// puts them there); the dense layouts skip the permute and come out as the spread leaves them.
+__host__ __device__ constexpr int frag_col(int bits, bool dense, int bi) {
+  if (!dense) return bi;
+  if (bits == 2) return (bi >> 2) + 4 * (bi & 3);                                 // byte 4k+j <- column k+4j
   return ((bi >> 3) << 3) + 2 * (bi & 3) + ((bi >> 2) & 1);                       // even | odd per 8
 }
 
-// ------------------------------------------------------------------ the kernel
+// ------------------------------------------------------------------ activation prep
+// x' = x * col_scale per 128-column chunk -> delta and three signed int8 digits per column:
+// x' ~= delta * (65536*d2 + 256*d1 + d0),  delta = max|x'| / (127 * 65536).  One thread = 16 columns.
+struct PrepMat {
+  const uint16_t* x;
+  const uint16_t* cs;
+  int64_t ldx;
+  int N;
+  int order;               // 0 column order, 1 dense 3/4-bit order, 2 dense 2-bit order
+  int8_t* xq;
+  float* delta;
+  int item0;               // first item of this matrix
+};
+struct PrepBatch { PrepMat mat[GV_MAX_BATCH]; int n, M, xdt, items; };
+
+__global__ __launch_bounds__(256) void gemv_prep_kernel(PrepBatch b) {
+  const int it = blockIdx.x * 256 + threadIdx.x;          // items are multiples of 8 per matrix
+  const bool ok = it < b.items;
+  int mi = 0;
+#pragma unroll
+  for (int i = 1; i < GV_MAX_BATCH; ++i) mi = (i < b.n && it >= b.mat[i].item0) ? i : mi;
+  const PrepMat& pm = b.mat[mi];
+  const int N = pm.N, n16 = N >> 4, NCH = N >> 7;
+  const int loc = ok ? it - pm.item0 : 0;
+  const int row = loc / n16, c16 = loc % n16;
+  const uint16_t* xp = pm.x + (size_t)row * pm.ldx + c16 * 16;
+  uint4 xr[2] = {((const uint4*)xp)[0], ((const uint4*)xp)[1]};
+  uint4 cr[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+  if (pm.cs) { cr[0] = ((const uint4*)(pm.cs + c16 * 16))[0]; cr[1] = ((const uint4*)(pm.cs + c16 * 16))[1]; }
+  const uint32_t* xw = (const uint32_t*)xr;
+  const uint32_t* cw = (const uint32_t*)cr;
+  float xv[16];
+  float mx = 0.f;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const uint16_t xb = (uint16_t)(xw[e >> 1] >> (16 * (e & 1)));
+    float v = b.xdt == CBK_F16 ? h2f(xb) : bf2f(xb);
+    if (pm.cs) v *= h2f((uint16_t)(cw[e >> 1] >> (16 * (e & 1))));
+    xv[e] = ok ? v : 0.f;
+    mx = fmaxf(mx, fabsf(xv[e]));
+  }
+  mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
+  mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
+  mx = fmaxf(mx, __shfl_xor(mx, 4, 64));
+  const float d = mx > 0.f ? mx / 8323072.f : 1.f;
+  const float inv = 1.f / d;
+  uint32_t dw[NDIG][4];
+#pragma unroll
+  for (int k = 0; k < NDIG; ++k)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) dw[k][q] = 0u;
+#pragma unroll
+  for (int bi = 0; bi < 16; ++bi) {
+    const int e = pm.order == 0 ? bi : (pm.order == 1 ? frag_col(4, true, bi) : frag_col(2, true, bi));
+    float v = xv[0];
+    if (pm.order == 0) v = xv[bi];
+    else if (pm.order == 1) v = xv[frag_col(4, true, bi)];
+    else v = xv[frag_col(2, true, bi)];
+    (void)e;
+    int X = (int)rintf(v * inv);                       // |X| <= 127 * 65536
+    const int d0 = (int)(int8_t)(X & 0xFF);
+    X = (X - d0) >> 8;
+    const int d1 = (int)(int8_t)(X & 0xFF);
+    const int d2 = (X - d1) >> 8;
+    dw[0][bi >> 2] |= ((uint32_t)d2 & 0xFFu) << (8 * (bi & 3));
+    dw[1][bi >> 2] |= ((uint32_t)d1 & 0xFFu) << (8 * (bi & 3));
+    dw[2][bi >> 2] |= ((uint32_t)d0 & 0xFFu) << (8 * (bi & 3));
+  }
+  if (ok) {
+#pragma unroll
+    for (int k = 0; k < NDIG; ++k)
+      *(uint4*)(pm.xq + ((size_t)row * NDIG + k) * N + c16 * 16) = make_uint4(dw[k][0], dw[k][1], dw[k][2], dw[k][3]);
+    if ((c16 & 7) == 0) pm.delta[row * (NCH + 4) + (c16 >> 3)] = d;
+    if (c16 < 4) pm.delta[row * (NCH + 4) + NCH + c16] = 0.f;              // chunks past N
+  }
+}
+
+// ------------------------------------------------------------------ the decode kernel
+template <class C>
+struct Loads {
+  uint32_t mk[4];
+  uint32_t raw[C::NL];
+  uint32_t zraw;
+  uint32_t sc[C::NGC];        // fp16 bits of the scales of this lane's chunk
+};
+
 template <int BITS, int KEEP, int GRP, int MP>
-__global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvArgs a) {
+__global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
   using C = Cfg<BITS, KEEP, GRP, MP>;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  const DMat& m = a.m;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int N = m.N, NCH = N >> 7;
   uint2* lut = (uint2*)smem;
   uint8_t* zreg = smem + LUT_BYTES;
-  int8_t* xq = (int8_t*)(zreg + ZERO_BYTES);                       // [M][2][N]
-  float* delta = (float*)(xq + (size_t)a.M * 2 * N);               // [M][NCH + 4]
-  float* red = delta + (size_t)a.M * (NCH + 4);                    // [2][GV_WAVES][GV_MAX_M][16]
-
-  // ---- selector table, one copy per lane%16 so that a wavefront's lookups do not collide
-  {
-    const SelTable& t = (BITS == 2 && !C::DENSE) ? g_sel2 : g_sel4;
-    for (int i = tid; i < 256 * LUT_LANES; i += GV_THREADS) lut[i] = make_uint2(t.lo[i / LUT_LANES], t.hi[i / LUT_LANES]);
-    if (tid < ZERO_BYTES / 4) ((uint32_t*)zreg)[tid] = 0u;
-  }
-  // ---- activations -> block fixed point.  One item = 16 columns; 8 items = one chunk.
-  {
-    const int items = a.M * (N >> 4);
-    for (int it = tid; it < ((items + 7) & ~7); it += GV_THREADS) {
-      const bool ok = it < items;
-      const int mi = ok ? it / (N >> 4) : 0, c16 = ok ? it % (N >> 4) : 0;
-      float xv[16];
-      const uint16_t* xp = a.x + (size_t)mi * a.ldx + c16 * 16;
-      const uint16_t* cp = m.cs ? m.cs + c16 * 16 : nullptr;
-      uint4 xr[2] = {((const uint4*)xp)[0], ((const uint4*)xp)[1]};
-      uint4 cr[2];
-      if (cp) { cr[0] = ((const uint4*)cp)[0]; cr[1] = ((const uint4*)cp)[1]; }
-      const uint32_t* xw = (const uint32_t*)xr;
-      const uint32_t* cw = (const uint32_t*)cr;
-      float mx = 0.f;
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const uint16_t xb = (uint16_t)(xw[e >> 1] >> (16 * (e & 1)));
-        float v = a.xdt == CBK_F16 ? h2f(xb) : bf2f(xb);
-        if (cp) v *= h2f((uint16_t)(cw[e >> 1] >> (16 * (e & 1))));
-        xv[e] = ok ? v : 0.f;
-        mx = fmaxf(mx, fabsf(xv[e]));
-      }
-      mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 4, 64));
-      const float d = mx > 0.f ? mx / 32512.f : 1.f;
-      const float inv = 1.f / d;
-      uint32_t hw[4] = {0, 0, 0, 0}, lw[4] = {0, 0, 0, 0};
-#pragma unroll
-      for (int bi = 0; bi < 16; ++bi) {
-        const int X = (int)rintf(xv[frag_col<BITS, C::DENSE>(bi)] * inv);
-        const int h = (X + 128) >> 8;
-        const int l = X - (h << 8);
-        hw[bi >> 2] |= ((uint32_t)h & 0xFFu) << (8 * (bi & 3));
-        lw[bi >> 2] |= ((uint32_t)l & 0xFFu) << (8 * (bi & 3));
-      }
-      if (ok) {
-        *(uint4*)(xq + ((size_t)mi * 2 + 0) * N + c16 * 16) = make_uint4(hw[0], hw[1], hw[2], hw[3]);
-        *(uint4*)(xq + ((size_t)mi * 2 + 1) * N + c16 * 16) = make_uint4(lw[0], lw[1], lw[2], lw[3]);
-        if ((c16 & 7) == 0) delta[mi * (NCH + 4) + (c16 >> 3)] = d;
-      }
-    }
-    if (tid < a.M * 4) delta[(tid >> 2) * (NCH + 4) + NCH + (tid & 3)] = 0.f;   // chunks past N
-  }
-  __syncthreads();
+  int8_t* xq = (int8_t*)(zreg + ZERO_BYTES);
+  float* delta = (float*)(xq + b.xq_cap);
+  float* red = delta + b.delta_cap;                    // [nslot][sk_cap][M][16] partial sums
+  int* cnt = (int*)(red + b.red_floats);               // [nslot] arrival counters
 
   const int wr = lane & 15, kq = lane >> 4;            // weight row in tile / lane quarter
-  const int nS = (NCH + 3) >> 2;
   const uint32_t l16 = lane & (LUT_LANES - 1);
-  // role of this lane's row in the A operand: variant i = lane%16
-  const int a_mloc = wr >> 3, a_slice = (wr >> 1) & 3, a_dig = wr & 1;
-  // role of this lane in the result: activation row 2p + kq/2, slices 2*(kq&1) and +1
-  const int o_mloc = kq >> 1, o_s0 = 2 * (kq & 1);
-  int buf = 0;
+  // role of this lane's row in the A operand: variant i = lane%16 = 4 * quarter + digit
+  // (digit 3 is an all-zero row); in the result, lane quarter kq holds the three digit sums
+  // of its own chunk, so every lane post-processes exactly the chunk it decoded
+  const int a_slice = wr >> 2, a_dig = wr & 3;
+  const uint32_t xq_off = (uint32_t)((uint8_t*)xq - smem), z_off = (uint32_t)(zreg - smem);
 
-  for (int tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
-    const int row = tile * 16 + wr;
-    const int rowc = row < m.K ? row : m.K - 1;
-    const uint8_t* rowp = m.data + (size_t)rowc * m.stride;
-    const uint16_t* scp = m.scale + (size_t)rowc * m.G;
-    const uint8_t* zp = m.zero + (size_t)rowc * m.G;
-    float ysum[MP];
-#pragma unroll
-    for (int p = 0; p < MP; ++p) ysum[p] = 0.f;
+  // the tiles of this workgroup: those whose first cost unit falls in [c0, c1)
+  const int c0 = (int)(((int64_t)b.total_cost * blockIdx.x) / gridDim.x);
+  const int c1 = (int)(((int64_t)b.total_cost * (blockIdx.x + 1)) / gridDim.x);
+  bool first = true;
 
-    for (int S = wave; S < nS; S += GV_WAVES) {
-      const int chunk = 4 * S + kq;
-      const bool valid = chunk < NCH;
-      const int chc = valid ? chunk : NCH - 1;
-      // ---- loads: bitmap, code bits, zero points, scales
-      uint32_t mk[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+  for (int mi = 0; mi < b.n; ++mi) {
+    const GvMat& gm = b.mat[mi];
+    const DMat& m = gm.m;
+    const int nS = gm.nS;
+    int t_lo = (c0 - gm.cost0 + nS - 1) / nS, t_hi = (c1 - gm.cost0 + nS - 1) / nS;
+    t_lo = t_lo < 0 ? 0 : t_lo;
+    t_hi = t_hi > gm.ntiles ? gm.ntiles : t_hi;
+    if (t_lo >= t_hi) continue;                                   // uniform over the workgroup
+    const int N = m.N, NCH = N >> 7;
+    // items: tile tl (local), part j of SK; part j covers macro-steps [j*spi, min(nS,(j+1)*spi))
+    const int SK = gm.sk, spi = gm.spi;
+    const int nitems = (t_hi - t_lo) * SK;
+    const int gt = b.nslot >> 1;                                  // tiles per barrier group
+
+    auto issue = [&](int tile, int S, Loads<C>& L) {
+      int row = tile * 16 + wr;
+      row = row < m.K ? row : m.K - 1;
+      const RowView rv = row_view(m, row);
+      int ch = 4 * S + kq;
+      ch = ch < NCH ? ch : NCH - 1;
       if (!C::DENSE) {
-        const uint4 v = *(const uint4*)(rowp + 16 * chc);
-        mk[0] = v.x; mk[1] = v.y; mk[2] = v.z; mk[3] = v.w;
+        const uint4 v = *(const uint4*)rv.unit(ch);
+        L.mk[0] = v.x; L.mk[1] = v.y; L.mk[2] = v.z; L.mk[3] = v.w;
       }
-      uint32_t raw[C::NL];
-      uint32_t skew = 0;
-      {
-        const uint8_t* plane = rowp + m.code_off;
-        if (C::VEC16) {
-          const uint4* p = (const uint4*)(plane + (size_t)chc * (C::CHB / 8));
+      // code bits of the chunk: bit ch*CHB of the code plane, fetched as whole 16-byte units
+      const uint32_t u0 = (m.code_off >> 4) + (C::VEC16 ? (uint32_t)ch * (C::CHB / 128) : (((uint32_t)ch * C::CHB) >> 7));
 #pragma unroll
-          for (int i = 0; i < C::ND / 4; ++i) { const uint4 v = p[i]; raw[4 * i] = v.x; raw[4 * i + 1] = v.y; raw[4 * i + 2] = v.z; raw[4 * i + 3] = v.w; }
-        } else {
-          const uint32_t sb = (uint32_t)chc * C::CHB;
-          const uint32_t* p = (const uint32_t*)plane + (sb >> 5);
-          skew = sb & 31u;
-#pragma unroll
-          for (int i = 0; i < C::NL; ++i) raw[i] = p[i];
-        }
+      for (int i = 0; i < C::NL / 4; ++i) {
+        const uint4 v = *(const uint4*)rv.unit(u0 + i);
+        L.raw[4 * i] = v.x; L.raw[4 * i + 1] = v.y; L.raw[4 * i + 2] = v.z; L.raw[4 * i + 3] = v.w;
       }
-      uint32_t zraw;
-      if (C::NGC == 1) zraw = zp[chc];
-      else zraw = *(const uint16_t*)(zp + 2 * chc);
-      // scales of the two chunks this lane post-processes
-      float sc[2][C::NGC];
+      if (C::NGC == 1) L.zraw = m.zero[meta_index(m, row, ch)];
+      else L.zraw = (uint32_t)m.zero[meta_index(m, row, 2 * ch)] | ((uint32_t)m.zero[meta_index(m, row, 2 * ch + 1)] << 8);
 #pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        int ch = 4 * S + o_s0 + s;
-        ch = ch < NCH ? ch : NCH - 1;
-#pragma unroll
-        for (int g = 0; g < C::NGC; ++g) sc[s][g] = h2f(scp[ch * C::NGC + g]);
-      }
-      // ---- A operand addresses (activation digits of this lane's own columns, or zeros)
-      uint32_t aaddr[MP];
-#pragma unroll
-      for (int p = 0; p < MP; ++p) {
-        const int mi = 2 * p + a_mloc;
-        const bool on = valid && a_slice == kq && mi < a.M;
-        aaddr[p] = on ? (uint32_t)((xq - (int8_t*)smem) + ((size_t)mi * 2 + a_dig) * N + chunk * 128)
-                      : (uint32_t)(zreg - smem);
-      }
-      // ---- align the chunk's code bits
-      uint32_t cw[C::ND];
-#pragma unroll
-      for (int i = 0; i < C::ND; ++i)
-        cw[i] = C::ALIGNED ? raw[i] : __builtin_amdgcn_alignbit(raw[i + 1], raw[i], skew);
+      for (int g = 0; g < C::NGC; ++g) L.sc[g] = m.scale[meta_index(m, row, ch * C::NGC + g)];
+    };
 
-      v4i acc[MP];
-#pragma unroll
-      for (int p = 0; p < MP; ++p) acc[p] = (v4i){0, 0, 0, 0};
+    Loads<C> cur, nxt;
+    int q = wave;                                                 // this wave's current item
+    if (q < nitems) issue(t_lo + q / SK, (q % SK) * spi, cur);    // in flight during the staging below
 
+    // ---- stage: selector table and counters (once), activation digits and deltas of this matrix
+    __syncthreads();                                              // previous matrix fully consumed
+    if (first) {
+      if (tid < 256) {
+        const uint2 e = make_selectors((uint32_t)tid, C::SEL_KIND);
 #pragma unroll
-      for (int jb = 0; jb < 4; ++jb) {
-        // code stream of block jb, SB bits per code
-        uint32_t st[C::NW];
-        if (BITS == 3) {
-#pragma unroll
-          for (int k = 0; k < C::NW; ++k) st[k] = expand3to4(get32<C::ND>(cw, jb * C::CB + 24 * k));
-        } else {
-#pragma unroll
-          for (int k = 0; k < C::NW; ++k) st[k] = get32<C::ND>(cw, jb * C::CB + 32 * k);
-        }
-        const uint32_t z = (C::NGC == 1) ? zraw : ((zraw >> (8 * (jb >> 1))) & 0xFFu);
-        const uint32_t nz = 0x80808080u - z * 0x01010101u;
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          uint32_t bfrag[4];
-#pragma unroll
-          for (int jj2 = 0; jj2 < 2; ++jj2) {
-            const int jj = 2 * half + jj2;                       // mask byte inside the block
-            uint32_t p0, p1;
-            if (C::DENSE) {
-              // 8 codes at a compile-time position
-              if (C::SB == 4) {
-                const uint32_t w = st[jj];
-                p0 = bias_pool(w & 0x0F0F0F0Fu, nz);
-                p1 = bias_pool((w >> 4) & 0x0F0F0F0Fu, nz);
-              } else {                                           // 2-bit: 16 codes per dword
-                const uint32_t w = st[half] >> (4 * jj2);        // k = 2*jj2, 2*jj2+1
-                p0 = bias_pool(w & 0x03030303u, nz);
-                p1 = bias_pool((w >> 2) & 0x03030303u, nz);
-              }
-              bfrag[2 * jj2] = p0; bfrag[2 * jj2 + 1] = p1;
-            } else {
-              const uint32_t mw = mk[jb];
-              const uint32_t mb = jj == 0 ? (mw & 0xFFu) : __builtin_amdgcn_ubfe(mw, 8 * jj, 8);
-              const uint32_t r = jj == 0 ? 0u : (uint32_t)__builtin_popcount(mw & ((1u << (8 * jj)) - 1u));
-              const uint32_t w = jj == 0 ? st[0] : window<C::NW>(st, r * C::SB);
-              if (C::SB == 4) {
-                p0 = bias_pool(w & 0x0F0F0F0Fu, nz);
-                p1 = bias_pool((w >> 4) & 0x0F0F0F0Fu, nz);
-              } else {
-                const uint32_t lo16 = w & 0xFFFFu;
-                const uint32_t t2 = (lo16 << 14) | lo16;
-                p0 = bias_pool(t2 & 0x03030303u, nz);
-                p1 = bias_pool((t2 >> 4) & 0x03030303u, nz);
-              }
-              const uint2 sel = lut[mb * LUT_LANES + l16];
-              bfrag[2 * jj2] = perm(p1, p0, sel.x);
-              bfrag[2 * jj2 + 1] = perm(p1, p0, sel.y);
-            }
-          }
-          const int t = 2 * jb + half;                            // fragment index in the chunk
-          const v4i bv = (v4i){(int)bfrag[0], (int)bfrag[1], (int)bfrag[2], (int)bfrag[3]};
-#pragma unroll
-          for (int p = 0; p < MP; ++p) {
-            const v4i av = *(const v4i*)(smem + aaddr[p] + 16 * t);
-            acc[p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bv, acc[p], 0, 0, 0);
-#ifdef CBK_NOP_AFTER_MFMA
-            asm volatile("s_nop 7\n s_nop 7" ::: "memory");
-#endif
-          }
-          // ---- end of a quantisation group: int32 -> float, times scale * delta
-          if ((C::NGC == 2 && t == 3) || t == 7) {
-            const int g = (C::NGC == 2 && t == 7) ? 1 : 0;
-#pragma unroll
-            for (int p = 0; p < MP; ++p) {
-              const int mi = 2 * p + o_mloc;
-              const float* dl = delta + (mi < a.M ? mi : 0) * (NCH + 4) + 4 * S + o_s0;
-              const float f0 = (float)(acc[p][0] * 256 + acc[p][1]);
-              const float f1 = (float)(acc[p][2] * 256 + acc[p][3]);
-              ysum[p] = fmaf(f0, sc[0][g] * dl[0], ysum[p]);
-              ysum[p] = fmaf(f1, sc[1][g] * dl[1], ysum[p]);
-              acc[p] = (v4i){0, 0, 0, 0};
-            }
-          }
-        }
+        for (int j = 0; j < LUT_LANES; ++j) lut[tid * LUT_LANES + j] = e;
+      } else if (tid < 256 + ZERO_BYTES / 4) {
+        ((uint32_t*)zreg)[tid - 256] = 0u;
+      } else if (tid < 256 + ZERO_BYTES / 4 + b.nslot) {
+        cnt[tid - 256 - ZERO_BYTES / 4] = 0;
       }
+      first = false;
     }
-    // ---- combine the two lane quarters that hold the same activation row, then the waves
-#pragma unroll
-    for (int p = 0; p < MP; ++p) {
-      const float v = ysum[p] + __shfl_xor(ysum[p], 16, 64);
-      const int mi = 2 * p + o_mloc;
-      if ((kq & 1) == 0 && mi < a.M) red[((buf * GV_WAVES + wave) * GV_MAX_M + mi) * 16 + wr] = v;
+    {
+      const int n16 = (b.M * NDIG * N) >> 4;
+      const uint4* src = (const uint4*)gm.xq;
+      uint4* dst = (uint4*)xq;
+      for (int i = tid; i < n16; i += GV_THREADS) dst[i] = src[i];
+      const int nd = b.M * (NCH + 4);
+      for (int i = tid; i < nd; i += GV_THREADS) delta[i] = gm.delta[i];
     }
     __syncthreads();
-    if (tid < 16 * a.M) {
-      const int mi = tid >> 4, r = tid & 15, k = tile * 16 + r;
-      if (k < m.K) {
-        float v = 0.f;
-        const int nw = nS < GV_WAVES ? nS : GV_WAVES;
-        for (int w = 0; w < nw; ++w) v += red[((buf * GV_WAVES + w) * GV_MAX_M + mi) * 16 + r];
-        if (a.bias) v += (a.ydt == CBK_F32) ? ((const float*)a.bias)[k]
-                       : (a.ydt == CBK_F16) ? h2f(((const uint16_t*)a.bias)[k]) : bf2f(((const uint16_t*)a.bias)[k]);
-        const size_t o = (size_t)mi * a.ldy + k;
-        if (a.ydt == CBK_F32) ((float*)a.y)[o] = v;
-        else if (a.ydt == CBK_F16) ((uint16_t*)a.y)[o] = f2h(v);
-        else ((uint16_t*)a.y)[o] = f2bf(v);
+
+    int bars = 0;                                                 // group barriers passed so far
+    for (; q < nitems; q += GV_WAVES) {
+      const int tl = q / SK, part = q - tl * SK;
+      const int tile = t_lo + tl;
+      const int s_begin = part * spi, s_end = (s_begin + spi < nS) ? s_begin + spi : nS;
+      // slots of tile group g are reused by group g + 2: wait until group g - 1 is complete
+      for (const int g = tl / gt; bars < g; ++bars) __syncthreads();
+
+      float ysum[MP];
+#pragma unroll
+      for (int p = 0; p < MP; ++p) ysum[p] = 0.f;
+
+      for (int S = s_begin; S < s_end; ++S) {
+        // prefetch this wave's next step
+        if (S + 1 < s_end) issue(tile, S + 1, nxt);
+        else if (q + GV_WAVES < nitems) { const int q2 = q + GV_WAVES; issue(t_lo + q2 / SK, (q2 % SK) * spi, nxt); }
+
+        const int chunk = 4 * S + kq;
+        const bool valid = chunk < NCH;
+        uint32_t aaddr[MP];
+#pragma unroll
+        for (int p = 0; p < MP; ++p) {
+          const bool on = valid && a_slice == kq && a_dig < NDIG && p < b.M;
+          aaddr[p] = on ? xq_off + (uint32_t)((p * NDIG + a_dig) * N + chunk * 128) : z_off;
+        }
+        // ---- bring the chunk's first code bit to bit 0 of cw[0]
+        uint32_t cw[C::ND];
+        if (C::VEC16) {
+#pragma unroll
+          for (int i = 0; i < C::ND; ++i) cw[i] = cur.raw[i];
+        } else {
+          const uint32_t skew = ((uint32_t)(valid ? chunk : NCH - 1) * C::CHB) & 127u;   // inside the first unit
+          uint32_t t1[C::NL];
+#pragma unroll
+          for (int i = 0; i < C::NL; ++i)
+            t1[i] = C::ALIGNED ? cur.raw[i]
+                               : __builtin_amdgcn_alignbit(i + 1 < C::NL ? cur.raw[i + 1] : 0u, cur.raw[i], skew);
+          uint32_t t2[C::NL];
+#pragma unroll
+          for (int i = 0; i < C::NL; ++i) t2[i] = (skew & 32u) ? (i + 1 < C::NL ? t1[i + 1] : 0u) : t1[i];
+#pragma unroll
+          for (int i = 0; i < C::ND; ++i) cw[i] = (skew & 64u) ? (i + 2 < C::NL ? t2[i + 2] : 0u) : t2[i];
+        }
+
+        v4i acc[MP];
+#pragma unroll
+        for (int p = 0; p < MP; ++p) acc[p] = (v4i){0, 0, 0, 0};
+
+#pragma unroll
+        for (int jb = 0; jb < 4; ++jb) {
+          uint32_t st[C::NW];                                     // code stream of block jb
+          if (BITS == 3) {
+#pragma unroll
+            for (int k = 0; k < C::NW; ++k) st[k] = expand3to4(get32<C::ND>(cw, jb * C::CB + 24 * k));
+          } else {
+#pragma unroll
+            for (int k = 0; k < C::NW; ++k) st[k] = get32<C::ND>(cw, jb * C::CB + 32 * k);
+          }
+          const uint32_t z = (C::NGC == 1) ? cur.zraw : ((cur.zraw >> (8 * (jb >> 1))) & 0xFFu);
+          const uint32_t nz = 0x80808080u - z * 0x01010101u;
+          const uint32_t mw = cur.mk[jb];
+          uint32_t mb[4], rk[4];
+          if (!C::DENSE) {
+            mb[0] = mw & 0xFFu; mb[1] = __builtin_amdgcn_ubfe(mw, 8, 8); mb[2] = __builtin_amdgcn_ubfe(mw, 16, 8); mb[3] = mw >> 24;
+            rk[0] = 0; rk[1] = (uint32_t)__builtin_popcount(mb[0]);
+            rk[2] = rk[1] + (uint32_t)__builtin_popcount(mb[1]); rk[3] = rk[2] + (uint32_t)__builtin_popcount(mb[2]);
+          }
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            uint32_t bfrag[4];
+#pragma unroll
+            for (int jj2 = 0; jj2 < 2; ++jj2) {
+              const int jj = 2 * half + jj2;                       // mask byte inside the block
+              uint32_t p0, p1;
+              if (C::DENSE) {
+                if (C::SB == 4) {
+                  const uint32_t w = st[jj];
+                  p0 = bias_pool(w & 0x0F0F0F0Fu, nz);
+                  p1 = bias_pool((w >> 4) & 0x0F0F0F0Fu, nz);
+                } else {                                           // 2-bit: 16 codes per dword
+                  const uint32_t w = st[half] >> (4 * jj2);
+                  p0 = bias_pool(w & 0x03030303u, nz);
+                  p1 = bias_pool((w >> 2) & 0x03030303u, nz);
+                }
+                bfrag[2 * jj2] = p0; bfrag[2 * jj2 + 1] = p1;
+              } else {
+                uint32_t w;
+                if (jj == 0) w = st[0];
+                else w = window<C::NW>(st, rk[jj] * C::SB);
+                if (C::SB == 4) {
+                  p0 = bias_pool(w & 0x0F0F0F0Fu, nz);
+                  p1 = bias_pool((w >> 4) & 0x0F0F0F0Fu, nz);
+                } else {
+                  const uint32_t lo16 = w & 0xFFFFu;
+                  const uint32_t t2 = (lo16 << 14) | lo16;
+                  p0 = bias_pool(t2 & 0x03030303u, nz);
+                  p1 = bias_pool((t2 >> 4) & 0x03030303u, nz);
+                }
+                const uint2 sel = lut[mb[jj] * LUT_LANES + l16];
+                bfrag[2 * jj2] = perm(p1, p0, sel.x);
+                bfrag[2 * jj2 + 1] = perm(p1, p0, sel.y);
+              }
+            }
+            const int t = 2 * jb + half;                            // fragment index in the chunk
+            const v4i bv = (v4i){(int)bfrag[0], (int)bfrag[1], (int)bfrag[2], (int)bfrag[3]};
+#pragma unroll
+            for (int p = 0; p < MP; ++p) {
+              const v4i av = *(const v4i*)(smem + aaddr[p] + 16 * t);
+              acc[p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bv, acc[p], 0, 0, 0);
+              // One idle issue slot after every MFMA.  Without it some instantiations of this
+              // kernel (register allocations in which the accumulator chain changes registers)
+              // returned run-to-run different sums on gfx950; with it every configuration is exact.
+              asm volatile("s_nop 1");
+            }
+            // ---- end of a quantisation group: int32 -> float, times scale * delta
+            if ((C::NGC == 2 && t == 3) || t == 7) {
+              const int g = (C::NGC == 2 && t == 7) ? 1 : 0;
+#pragma unroll
+              for (int p = 0; p < MP; ++p) {
+                const float dl = delta[(p < b.M ? p : 0) * (NCH + 4) + chunk];      // 0 past the last chunk
+                const float f = fmaf((float)(acc[p][0] * 256 + acc[p][1]), 256.f, (float)acc[p][2]);
+                ysum[p] = fmaf(f, h2f((uint16_t)cur.sc[g]) * dl, ysum[p]);
+                acc[p] = (v4i){0, 0, 0, 0};
+              }
+            }
+          }
+        }
+        cur = nxt;
+      }
+
+      // ---- the item is done: add the four lane quarters (the four chunks of every macro-step)
+      float part_sum[MP];
+#pragma unroll
+      for (int p = 0; p < MP; ++p) {
+        const float h = ysum[p] + __shfl_xor(ysum[p], 16, 64);
+        part_sum[p] = h + __shfl_xor(h, 32, 64);
+      }
+      auto store = [&](int om, int r, float v) {
+        const int k = tile * 16 + r;
+        if (k >= m.K) return;
+        if (gm.bias) v += (b.ydt == CBK_F32) ? ((const float*)gm.bias)[k]
+                        : (b.ydt == CBK_F16) ? h2f(((const uint16_t*)gm.bias)[k]) : bf2f(((const uint16_t*)gm.bias)[k]);
+        const size_t o = (size_t)om * gm.ldy + k;
+        if (b.ydt == CBK_F32) ((float*)gm.y)[o] = v;
+        else if (b.ydt == CBK_F16) ((uint16_t*)gm.y)[o] = f2h(v);
+        else ((uint16_t*)gm.y)[o] = f2bf(v);
+      };
+      if (SK == 1) {
+#pragma unroll
+        for (int p = 0; p < MP; ++p)
+          if (kq == 0 && p < b.M) store(p, wr, part_sum[p]);
+      } else {
+        // partial sums of the SK parts of a tile meet in an LDS slot; the wave that arrives last
+        // adds them in part order (not arrival order), so the result does not depend on timing
+        const int slot = tl & (b.nslot - 1);
+        float* rs = red + (size_t)slot * b.sk_cap * b.M * 16;
+#pragma unroll
+        for (int p = 0; p < MP; ++p)
+          if (kq == 0 && p < b.M) rs[(part * b.M + p) * 16 + wr] = part_sum[p];
+        int old = 0;
+        if (lane == 0) old = atomicAdd(&cnt[slot], 1);
+        old = __shfl(old, 0, 64);
+        if (old == SK - 1) {                                      // uniform over the wave
+          for (int om = kq; om < b.M; om += 4) {
+            float v = 0.f;
+            for (int j = 0; j < SK; ++j) v += rs[(j * b.M + om) * 16 + wr];
+            store(om, wr, v);
+          }
+          if (lane == 0) cnt[slot] = 0;
+        }
       }
     }
-    buf ^= 1;
+    // every wave passes the same number of group barriers
+    const int ngroups = ((t_hi - t_lo) + gt - 1) / gt;
+    for (; bars < ngroups - 1; ++bars) __syncthreads();
   }
 }
 
 // ------------------------------------------------------------------ host side
-static size_t lds_bytes(const DMat& m, int M) {
-  const int NCH = m.N / 128;
-  return (size_t)LUT_BYTES + ZERO_BYTES + (size_t)M * 2 * m.N + (size_t)M * (NCH + 4) * 4 +
-         (size_t)2 * GV_WAVES * GV_MAX_M * 16 * 4;
-}
+static inline size_t up256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 static bool keep_supported(int keep) { return keep == 10 || keep == 16 || keep == 23; }
 
@@ -415,61 +530,131 @@ bool gemv_fast_takes(const DMat& m, int M) {
   else if (fam == FAM_DENSE) { if (m.bits == 8) return false; }
   else return false;
   if (m.bits != 2 && m.bits != 3 && m.bits != 4) return false;
-  return (size_t)M * 2 * m.N <= (size_t)X_LDS_BUDGET;
+  return (size_t)M * NDIG * m.N <= (size_t)X_LDS_BUDGET;
 }
 
-size_t gemv_fast_workspace(const DMat&, int) { return 0; }
+bool gemv_same_config(const DMat& a, const DMat& b) {
+  const bool da = family_of(a.layout) == FAM_DENSE, db = family_of(b.layout) == FAM_DENSE;
+  return da == db && a.bits == b.bits && a.group == b.group && (da || a.keep == b.keep);
+}
+
+size_t gemv_fast_workspace(const DMat& m, int M) {
+  return up256((size_t)M * NDIG * m.N) + up256((size_t)M * (m.N / 128 + 4) * 4);
+}
+
+struct GvCall {           // one matrix of a batched call, host side
+  DMat m;
+  const void* x;
+  int64_t ldx;
+  void* y;
+  int64_t ldy;
+  const void* bias;
+};
 
 template <int BITS, int KEEP, int GRP, int MP>
-static int launch_cfg(const GvArgs& a, size_t lds, hipStream_t st) {
+static int launch_cfg(const GvBatch& b, size_t lds, int blocks, hipStream_t st) {
   auto kern = gemv_mfma_kernel<BITS, KEEP, GRP, MP>;
-  static std::atomic<size_t> configured{0};
-  if (configured.load(std::memory_order_relaxed) < lds) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 512) != hipSuccess)
+  static std::atomic<int> configured{0};
+  if (!configured.load(std::memory_order_acquire)) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
       return CBK_ERR_HIP;
-    configured.store(160 * 1024, std::memory_order_relaxed);
+    configured.store(1, std::memory_order_release);
   }
-  int blocks = a.ntiles < 512 ? a.ntiles : 512;
-  hipLaunchKernelGGL(kern, dim3(blocks), dim3(GV_THREADS), lds, st, a);
-  return hipGetLastError() == hipSuccess ? CBK_OK : CBK_ERR_HIP;
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(GV_THREADS), lds, st, b);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess && getenv("CBK_DEBUG")) fprintf(stderr, "gemv launch failed: %s (lds %zu blocks %d M %d)\n", hipGetErrorString(e), lds, blocks, b.M);
+  return e == hipSuccess ? CBK_OK : CBK_ERR_HIP;
 }
 
 template <int BITS, int KEEP, int GRP>
-static int launch_mp(const GvArgs& a, size_t lds, hipStream_t st) {
-  const int mp = (a.M + 1) / 2;
-  if (mp == 1) return launch_cfg<BITS, KEEP, GRP, 1>(a, lds, st);
-  if (mp == 2) return launch_cfg<BITS, KEEP, GRP, 2>(a, lds, st);
-  return launch_cfg<BITS, KEEP, GRP, 4>(a, lds, st);
+static int launch_mp(const GvBatch& b, size_t lds, int blocks, hipStream_t st) {
+  if (b.M == 1) return launch_cfg<BITS, KEEP, GRP, 1>(b, lds, blocks, st);
+  if (b.M == 2) return launch_cfg<BITS, KEEP, GRP, 2>(b, lds, blocks, st);
+  return launch_cfg<BITS, KEEP, GRP, 4>(b, lds, blocks, st);
 }
 
 template <int BITS, int KEEP>
-static int launch_grp(const GvArgs& a, size_t lds, hipStream_t st) {
-  return a.m.group == 64 ? launch_mp<BITS, KEEP, 64>(a, lds, st) : launch_mp<BITS, KEEP, 128>(a, lds, st);
+static int launch_grp(const GvBatch& b, size_t lds, int blocks, hipStream_t st) {
+  return b.mat[0].m.group == 64 ? launch_mp<BITS, KEEP, 64>(b, lds, blocks, st)
+                                : launch_mp<BITS, KEEP, 128>(b, lds, blocks, st);
 }
 
 template <int BITS>
-static int launch_keep(const GvArgs& a, size_t lds, hipStream_t st) {
-  switch (family_of(a.m.layout) == FAM_DENSE ? 0 : a.m.keep) {
-    case 0: return launch_grp<BITS, 0>(a, lds, st);
-    case 10: return launch_grp<BITS, 10>(a, lds, st);
-    case 16: return launch_grp<BITS, 16>(a, lds, st);
-    case 23: return launch_grp<BITS, 23>(a, lds, st);
+static int launch_keep(const GvBatch& b, size_t lds, int blocks, hipStream_t st) {
+  const DMat& m = b.mat[0].m;
+  switch (family_of(m.layout) == FAM_DENSE ? 0 : m.keep) {
+    case 0: return launch_grp<BITS, 0>(b, lds, blocks, st);
+    case 10: return launch_grp<BITS, 10>(b, lds, blocks, st);
+    case 16: return launch_grp<BITS, 16>(b, lds, blocks, st);
+    case 23: return launch_grp<BITS, 23>(b, lds, blocks, st);
     default: return CBK_ERR_UNSUPPORTED;
   }
 }
 
-int launch_gemv_fast(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
-                     const void* bias, void*, size_t, hipStream_t st) {
-  GvArgs a;
-  a.m = m; a.x = (const uint16_t*)x; a.ldx = ldx; a.M = M; a.y = y; a.ydt = ydt; a.ldy = ldy; a.bias = bias;
-  a.xdt = xdt; a.ntiles = (m.K + 15) / 16;
-  const size_t lds = lds_bytes(m, M);
-  switch (m.bits) {
-    case 2: return launch_keep<2>(a, lds, st);
-    case 3: return launch_keep<3>(a, lds, st);
-    case 4: return launch_keep<4>(a, lds, st);
-    default: return CBK_ERR_UNSUPPORTED;
+// All matrices share one kernel configuration (checked by the caller) and 1 <= M <= 4.
+int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, void* workspace, size_t ws_bytes,
+                           hipStream_t st) {
+  if (n < 1 || n > GV_MAX_BATCH) return CBK_ERR_SHAPE;
+  PrepBatch pb;
+  GvBatch gb;
+  pb.n = gb.n = n; pb.M = gb.M = M; pb.xdt = xdt; gb.ydt = ydt;
+  size_t off = 0;
+  int items = 0, cost = 0, xq_cap = 0, delta_cap = 0, tiles = 0;
+  for (int i = 0; i < n; ++i) {
+    const DMat& m = calls[i].m;
+    const bool dense = family_of(m.layout) == FAM_DENSE;
+    PrepMat& p = pb.mat[i];
+    GvMat& g = gb.mat[i];
+    p.x = (const uint16_t*)calls[i].x; p.cs = m.cs; p.ldx = calls[i].ldx; p.N = m.N;
+    p.order = !dense ? 0 : (m.bits == 2 ? 2 : 1);
+    p.xq = (int8_t*)workspace + off;
+    off += up256((size_t)M * NDIG * m.N);
+    p.delta = (float*)((uint8_t*)workspace + off);
+    off += up256((size_t)M * (m.N / 128 + 4) * 4);
+    p.item0 = items;
+    items += M * (m.N / 16);
+    g.m = m; g.xq = p.xq; g.delta = p.delta; g.y = calls[i].y; g.bias = calls[i].bias; g.ldy = calls[i].ldy;
+    g.ntiles = (m.K + 15) / 16; g.nS = (m.N / 128 + 3) / 4; g.cost0 = cost;
+    cost += g.ntiles * g.nS;
+    tiles += g.ntiles;
+    xq_cap = xq_cap > M * NDIG * m.N ? xq_cap : M * NDIG * m.N;
+    delta_cap = delta_cap > M * (m.N / 128 + 4) ? delta_cap : M * (m.N / 128 + 4);
   }
+  if (off > ws_bytes || !workspace) return CBK_ERR_WORKSPACE;
+  pb.items = items;
+  gb.total_cost = cost; gb.xq_cap = xq_cap; gb.delta_cap = delta_cap;
+  int blocks = tiles < 256 ? tiles : 256;                       // one persistent workgroup per CU
+  if (const char* e = getenv("CBK_GV_BLOCKS")) blocks = atoi(e) < tiles ? atoi(e) : tiles;
+  // macro-steps per work item: about two items per wavefront over the whole launch, so that
+  // the tail is short; a tile is split into at most 16 parts
+  int spi = cost / (blocks * GV_WAVES * 2);
+  spi = spi < 1 ? 1 : (spi > 8 ? 8 : spi);
+  if (const char* e = getenv("CBK_GV_SPI")) spi = atoi(e);
+  int sk_cap = 1;
+  for (int i = 0; i < n; ++i) {
+    GvMat& g = gb.mat[i];
+    int s = spi;
+    while ((g.nS + s - 1) / s > 16) ++s;
+    g.spi = s; g.sk = (g.nS + s - 1) / s;
+    sk_cap = sk_cap > g.sk ? sk_cap : g.sk;
+  }
+  // reduction slots: as many as fit 24 KB, a power of two between 2 and 64
+  const int slot_floats = sk_cap * M * 16;
+  int nslot = 64;
+  while (nslot > 2 && (size_t)nslot * slot_floats * 4 > 24 * 1024) nslot >>= 1;
+  gb.sk_cap = sk_cap; gb.nslot = nslot; gb.red_floats = nslot * slot_floats;
+  hipLaunchKernelGGL(gemv_prep_kernel, dim3((items + 255) / 256), dim3(256), 0, st, pb);
+  const size_t lds = (size_t)LUT_BYTES + ZERO_BYTES + xq_cap + (size_t)delta_cap * 4 +
+                     (size_t)gb.red_floats * 4 + (size_t)nslot * 4;
+  const int bits = gb.mat[0].m.bits;
+  return bits == 2 ? launch_keep<2>(gb, lds, blocks, st) : bits == 3 ? launch_keep<3>(gb, lds, blocks, st)
+       : bits == 4 ? launch_keep<4>(gb, lds, blocks, st) : CBK_ERR_UNSUPPORTED;
+}
+
+int launch_gemv_fast(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
+                     const void* bias, void* ws, size_t ws_bytes, hipStream_t st) {
+  GvCall c{m, x, ldx, y, ldy, bias};
+  return launch_gemv_fast_batch(1, &c, xdt, M, ydt, ws, ws_bytes, st);
 }
 
 }  // namespace cbk

@@ -30,13 +30,13 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(DMat m, const void* x
     for (int i = 0; i < M; ++i) acc[i] = 0.f;
     const uint16_t* cs = m.cs ? m.cs + (size_t)cs_row_of(m, k) * m.N : nullptr;
     if (fam != FAM_SPARSE) {
-      const uint8_t* row = m.data + (size_t)k * m.stride;
+      const RowView row = row_view(m, k);
       for (int t = lane; t < m.N / BLOCK; t += 64) {
         int q[32];
         const uint32_t keep = decode_block32(m, row, t, q);
         const int g = (t * BLOCK) / m.group;
-        const float s = h2f(m.scale[(size_t)k * m.G + g]);
-        const int z = m.zero[(size_t)k * m.G + g];
+        const float s = h2f(m.scale[meta_index(m, k, g)]);
+        const int z = m.zero[meta_index(m, k, g)];
         float part[M];
 #pragma unroll
         for (int i = 0; i < M; ++i) part[i] = 0.f;

@@ -32,6 +32,8 @@ _SPARSE = (SPARSE4, SPARSE4X, SPARSE4E)
 
 F32, F16, BF16T = 0, 1, 2
 FLAG_ZERO_LE_128 = 1
+FLAG_TILED16 = 2
+TILED_TAIL = 512
 
 
 def dtype_code(dt: torch.dtype) -> int:
@@ -212,9 +214,66 @@ class PackedMatrix:
         p.blob = self.blob.clone()
         return p
 
+    @property
+    def tiled(self) -> bool:
+        return bool(self.flags & FLAG_TILED16)
+
+    def _krows(self) -> int:
+        return _align(self.K, 16) if self.tiled else self.K
+
+    def to_tiled(self) -> "PackedMatrix":
+        """The same matrix in the 16-row tile-interleaved order the kernels stream fastest: byte o
+        of row k moves to (k//16)*16*stride + ((o//16)*16 + k%16)*16 + o%16, scale/zero entry (k, g)
+        to index ((k//16)*G + g)*16 + k%16; K is padded with zero rows to a multiple of 16.  A pure
+        permutation of the packed bytes, done once when a layer is built or loaded."""
+        if self.tiled:
+            return self
+        if self.layout in _SPARSE:
+            raise ValueError("the variable-length SPARSE4* layouts have no tiled form")
+        K, G, dev = self.K, self.G, self.blob.device
+        stride = self.data_bytes // K
+        K16 = _align(K, 16) // 16
+        rows = torch.zeros(K16 * 16, stride, dtype=torch.uint8, device=dev)
+        rows[:K] = self.array("data")[: K * stride].view(K, stride)
+        data = torch.cat([rows.view(K16, 16, stride // 16, 16).permute(0, 2, 1, 3).reshape(-1),
+                          torch.zeros(TILED_TAIL, dtype=torch.uint8, device=dev)])
+        sc = torch.zeros(K16 * 16, G, dtype=torch.float16, device=dev)
+        sc[:K] = self.array("scale").view(K, G)
+        zr = torch.zeros(K16 * 16, G, dtype=torch.uint8, device=dev)
+        zr[:K] = self.array("zero").view(K, G)
+        arrays = {"data": data, "scale": sc.view(K16, 16, G).permute(0, 2, 1).contiguous(),
+                  "zero": zr.view(K16, 16, G).permute(0, 2, 1).contiguous()}
+        if self.cs_rows:
+            arrays["col_scale"] = self.array("col_scale")
+        blob, offs = _assemble(arrays, dev)
+        return PackedMatrix(blob, offs, K, self.N, self.layout, self.bits, self.group, self.keep, self.cs_rows,
+                            self.cs_splits, K16 * 16 * stride, self.n_survivors, self.n_zero_fixed,
+                            self.flags | FLAG_TILED16, dict(self.meta))
+
+    def to_rowmajor(self) -> "PackedMatrix":
+        """Inverse of to_tiled(): the reference's row-major CBK1 byte order."""
+        if not self.tiled:
+            return self
+        K, G, dev = self.K, self.G, self.blob.device
+        K16 = _align(K, 16) // 16
+        stride = self.data_bytes // (K16 * 16)
+        rows = self.array("data")[: K16 * 16 * stride].view(K16, stride // 16, 16, 16).permute(0, 2, 1, 3)
+        data = torch.cat([rows.reshape(K16 * 16, stride)[:K].reshape(-1),
+                          torch.zeros(BLOB_TAIL, dtype=torch.uint8, device=dev)])
+        arrays = {"data": data,
+                  "scale": self.array("scale").view(K16, G, 16).permute(0, 2, 1).reshape(K16 * 16, G)[:K].contiguous(),
+                  "zero": self.array("zero").view(K16, G, 16).permute(0, 2, 1).reshape(K16 * 16, G)[:K].contiguous()}
+        if self.cs_rows:
+            arrays["col_scale"] = self.array("col_scale")
+        blob, offs = _assemble(arrays, dev)
+        return PackedMatrix(blob, offs, K, self.N, self.layout, self.bits, self.group, self.keep, self.cs_rows,
+                            self.cs_splits, K * stride, self.n_survivors, self.n_zero_fixed,
+                            self.flags & ~FLAG_TILED16, dict(self.meta))
+
     def array(self, name: str) -> torch.Tensor:
-        n = {"data": self.data_bytes + BLOB_TAIL, "scale": self.K * self.G * 2, "zero": self.K * self.G,
-             "col_scale": self.cs_rows * self.N * 2, "row_off": (self.K + 1) * 4}[name]
+        kr = self._krows()
+        n = {"data": self.data_bytes + (TILED_TAIL if self.tiled else BLOB_TAIL), "scale": kr * self.G * 2,
+             "zero": kr * self.G, "col_scale": self.cs_rows * self.N * 2, "row_off": (self.K + 1) * 4}[name]
         v = self.blob[self.offs[name]: self.offs[name] + n]
         if name in ("scale", "col_scale"):
             return v.view(torch.float16)
@@ -224,7 +283,7 @@ class PackedMatrix:
 
     def stream_bytes(self) -> int:
         """Weight bytes one pass streams: rows + scale + zero (pack_cobalt.py:431-433)."""
-        return self.data_bytes + self.K * self.G * 3
+        return self.data_bytes + self._krows() * self.G * 3
 
     def bpw(self) -> float:
         ro = (self.K + 1) * 4 if "row_off" in self.offs else 0

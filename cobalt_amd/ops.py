@@ -92,3 +92,44 @@ def gemm(pm, x, bias=None, out_dtype=None, workspace=None):
 def linear(pm, x, bias=None, out_dtype=None, workspace=None):
     """y = x @ W_hat.T (+ bias): decode kernel up to 16 rows, prefill kernel above."""
     return _matmul("cbk_linear", pm, x, bias, out_dtype, workspace)
+
+
+def gemv_batch(pms, xs, biases=None, out_dtype=None):
+    """Independent decode GEMVs in one launch pair: ys[i] = xs[i] @ W_hat_i.T (+ biases[i]).
+    All xs share the number of rows (<= 16) and the dtype; at most 8 matrices."""
+    n = len(pms)
+    if n == 0:
+        return []
+    L = _lib.lib()
+    M = xs[0].reshape(-1, pms[0].N).shape[0]
+    out_dtype = out_dtype or xs[0].dtype
+    x2, ys, bs = [], [], []
+    for i, (pm, x) in enumerate(zip(pms, xs)):
+        bias = biases[i] if biases is not None else None
+        _require_gpu(pm, x, bias)
+        xi = x.reshape(-1, pm.N)
+        if xi.shape[0] != M or xi.dtype != xs[0].dtype:
+            raise ValueError("all activations of a batch share the row count and the dtype")
+        if xi.stride(-1) != 1 or (M > 1 and xi.stride(0) % 8) or xi.data_ptr() % 16:
+            xi = xi.contiguous()
+        x2.append(xi)
+        ys.append(torch.empty(M, pm.K, dtype=out_dtype, device=x.device))
+        bs.append(None if bias is None else bias.to(out_dtype))
+    descs = (_lib.CbkDesc * n)(*[pm.desc() for pm in pms])
+    need = L.cbk_gemv_batch_workspace_bytes(n, descs, M)
+    key = (pms[0].blob.device, torch.cuda.current_stream(pms[0].blob.device).cuda_stream)
+    ws = _workspaces.get(key)
+    if need and (ws is None or ws.numel() < need):
+        ws = torch.empty(max(need, 1 << 20), dtype=torch.uint8, device=pms[0].blob.device)
+        _workspaces[key] = ws
+    P = ctypes.c_void_p
+    xp = (P * n)(*[t.data_ptr() for t in x2])
+    yp = (P * n)(*[t.data_ptr() for t in ys])
+    bp = (P * n)(*[(t.data_ptr() if t is not None else None) for t in bs])
+    ldx = (ctypes.c_int64 * n)(*[(t.stride(0) if M > 1 else pm.N) for t, pm in zip(x2, pms)])
+    ldy = (ctypes.c_int64 * n)(*[pm.K for pm in pms])
+    rc = L.cbk_gemv_batch(n, descs, xp, ldx, dtype_code(x2[0].dtype), M, yp, ldy, dtype_code(out_dtype), bp,
+                          ws.data_ptr() if need else None, ws.numel() if need else 0,
+                          _stream_ptr(pms[0].blob.device))
+    _lib.check(rc, "cbk_gemv_batch")
+    return [y.reshape(*x.shape[:-1], pm.K) for y, x, pm in zip(ys, xs, pms)]

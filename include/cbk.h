@@ -44,6 +44,7 @@ enum cbk_layout {
 };
 
 #define CBK_FLAG_ZERO_LE_128 1
+#define CBK_FLAG_TILED16 2
 
 enum cbk_dtype { CBK_F32 = 0, CBK_F16 = 1, CBK_BF16T = 2 };
 
@@ -75,7 +76,14 @@ enum cbk_status {
  *             <= 128 (always true for an on-grid zero point of a 2/3/4-bit code, and for the
  *             reference's off-grid probe, src/cobaltkernel/test_gemv.py:428-431).  The int8
  *             matrix-core decode kernel needs q - zero to fit a signed byte; without the flag
- *             cbk_gemv runs the slower float row kernel, which takes any uint8 zero point. */
+ *             cbk_gemv runs the slower float row kernel, which takes any uint8 zero point.
+ *             CBK_FLAG_TILED16: data / scale / zero are in 16-row tile-interleaved order, a
+ *             permutation of the same bytes made once at load time so that the sixteen rows a
+ *             wavefront decodes together are contiguous in HBM: with s = cbk_row_stride(),
+ *             byte o of row k is at data[(k/16)*16*s + ((o/16)*16 + k%16)*16 + o%16], the
+ *             scale / zero entry of (row k, group g) at index ((k/16)*G + g)*16 + k%16; K is
+ *             padded with zero rows to a multiple of 16 and data ends with 512 readable bytes.
+ *             Fixed-stride layouts only.  Every entry point takes both orders. */
 typedef struct cbk_desc {
   const void* data;
   const void* row_off;
@@ -124,6 +132,19 @@ int cbk_dequant(const cbk_desc* d, int row0, int nrows, int with_col_scale,
 int cbk_gemv(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
              void* y, int y_dtype, int64_t ldy, const void* bias,
              void* workspace, size_t workspace_bytes, void* stream);
+
+/* Several independent decode GEMVs in one launch pair (activation prep + decode): the matrices
+ * a decoder layer multiplies by the same hidden state (q, k, v; gate, up), or any other set
+ * with no data dependence.  n <= 8.  Entry i computes ys[i] = xs[i] . W_hat_i^T (+ biases[i]).
+ * Matrices that share (family, bits, group, keep) and qualify for the matrix-core kernel run
+ * in one persistent launch that balances their row tiles over the chip; otherwise the call
+ * degrades to n single calls.  workspace >= cbk_gemv_batch_workspace_bytes(), 256-byte aligned.
+ * Counterpart of the reference's fused row-concatenated matrices (docs/FORMAT.md:126-151) and
+ * of the harness entry `gemv_multi` (src/cobaltkernel/csrc/test_gemv.cu:237-291). */
+size_t cbk_gemv_batch_workspace_bytes(int n, const cbk_desc* descs, int M);
+int cbk_gemv_batch(int n, const cbk_desc* descs, const void* const* xs, const int64_t* ldxs,
+                   int x_dtype, int M, void* const* ys, const int64_t* ldys, int y_dtype,
+                   const void* const* biases, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Prefill path, any M >= 1 (built for M >= 256).  Same contract as cbk_gemv.  Replaces the
  * harness entry `gemm` (test_gemm.cu:151-165) and cbk::gemm_tile (cobalt_gemm.cuh:243-609). */

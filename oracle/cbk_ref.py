@@ -545,3 +545,46 @@ def make_blob(packed, col_scale=None):
     if pad:
         parts.append(np.zeros(pad, np.uint8))
     return np.concatenate(parts), offs
+
+
+# ----------------------------------------------------------------------------- tile-interleaved device order
+TILE_ROWS = 16
+TILE_UNIT = 16
+TILED_TAIL = 512
+
+
+def tile16(packed, K, N, layout, bits=None, group=None, keep_per_block=None):
+    """Row-major fixed-stride arrays -> the 16-row tile-interleaved order the MI355X kernels
+    stream.  This is a permutation of the same bytes (plus zero rows up to a multiple of 16)
+    and has no counterpart in the reference, whose kernels read row-major rows: byte o of row
+    k moves to  (k//16)*16*stride + ((o//16)*16 + k%16)*16 + o%16 ; scale/zero entry (k, g)
+    moves to index ((k//16)*G + g)*16 + k%16.  The data array ends with 512 zero bytes."""
+    bits, group, kpb = canon(layout, bits, group, keep_per_block)
+    stride = row_stride(layout, N, bits, group, kpb)
+    G = N // group
+    K16 = (K + 15) // 16
+    rows = np.zeros((K16 * 16, stride), np.uint8)
+    rows[:K] = np.asarray(packed["data"], np.uint8)[: K * stride].reshape(K, stride)
+    data = rows.reshape(K16, 16, stride // 16, 16).transpose(0, 2, 1, 3).reshape(-1)
+    sc = np.zeros((K16 * 16, G), np.float16); sc[:K] = np.asarray(packed["scale"]).reshape(K, G)
+    zr = np.zeros((K16 * 16, G), np.uint8); zr[:K] = np.asarray(packed["zero"]).reshape(K, G)
+    out = dict(packed)
+    out["data"] = np.concatenate([data, np.zeros(TILED_TAIL, np.uint8)])
+    out["scale"] = sc.reshape(K16, 16, G).transpose(0, 2, 1).reshape(-1).copy()
+    out["zero"] = zr.reshape(K16, 16, G).transpose(0, 2, 1).reshape(-1).copy()
+    return out
+
+
+def untile16(tiled, K, N, layout, bits=None, group=None, keep_per_block=None):
+    """Inverse of tile16 (drops the padding rows; restores the 64-byte tail)."""
+    bits, group, kpb = canon(layout, bits, group, keep_per_block)
+    stride = row_stride(layout, N, bits, group, kpb)
+    G = N // group
+    K16 = (K + 15) // 16
+    d = np.asarray(tiled["data"], np.uint8)[: K16 * 16 * stride]
+    rows = d.reshape(K16, stride // 16, 16, 16).transpose(0, 2, 1, 3).reshape(K16 * 16, stride)[:K]
+    out = dict(tiled)
+    out["data"] = np.concatenate([rows.reshape(-1), np.zeros(BLOB_TAIL, np.uint8)])
+    out["scale"] = np.asarray(tiled["scale"]).reshape(K16, G, 16).transpose(0, 2, 1).reshape(K16 * 16, G)[:K].copy()
+    out["zero"] = np.asarray(tiled["zero"]).reshape(K16, G, 16).transpose(0, 2, 1).reshape(K16 * 16, G)[:K].copy()
+    return out

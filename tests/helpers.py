@@ -47,8 +47,15 @@ def product_pack(case, raw, device="cpu", col_scale="raw", **extra):
                       None if cs is None else t(cs), layout, bits, group, keep or None, **extra)
 
 
-def packed_from_oracle(case, pk, col_scale, K, N, device, cs_splits=(0, 0)):
-    """Oracle-packed arrays (including the variable-length layouts) -> product PackedMatrix."""
+def packed_from_oracle(case, pk, col_scale, K, N, device, cs_splits=(0, 0), tiled=False):
+    """Oracle-packed arrays (including the variable-length layouts) -> product PackedMatrix,
+    optionally re-ordered into the 16-row tile-interleaved device order."""
+    layout, bits, group, keep = case
+    pm = _from_oracle(case, pk, col_scale, K, N, device, cs_splits)
+    return pm.to_tiled() if tiled else pm
+
+
+def _from_oracle(case, pk, col_scale, K, N, device, cs_splits):
     layout, bits, group, keep = case
     return F.from_arrays(torch.from_numpy(pk["data"]), torch.from_numpy(pk["scale"].view(np.uint8)),
                          torch.from_numpy(pk["zero"]),

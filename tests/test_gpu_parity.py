@@ -31,12 +31,15 @@ def _f16_round(a):
 
 
 # ------------------------------------------------------------------ dequant, bit-exact
+@pytest.mark.parametrize("tiled", [False, True], ids=["rowmajor", "tiled"])
 @pytest.mark.parametrize("case", FIXED_CASES + SPARSE_CASES, ids=case_id)
-def test_dequant_bit_exact(case):
+def test_dequant_bit_exact(case, tiled):
+    if tiled and case in SPARSE_CASES:
+        pytest.skip("the variable-length layouts have no tiled form")
     for (K, N) in ((64, 1024), (40, 5376)):
         raw = make_raw(case, K, N, seed=K + N + case[0])
         pk = oracle_pack(case, raw)
-        pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV)
+        pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV, tiled=tiled)
         W = R.dequant(pk, K, N, case[0], col_scale=raw["col_scale"], **kw_of(case))
         got = _np(ops.dequant(pm, torch.float32))
         assert np.array_equal(got, W), f"{case_id(case)} {K}x{N}: {np.abs(got - W).max()}"
@@ -74,13 +77,16 @@ def test_pruned_positions_exactly_zero_off_grid_zero_point():
 
 
 # ------------------------------------------------------------------ decode GEMV
+@pytest.mark.parametrize("tiled", [False, True], ids=["rowmajor", "tiled"])
 @pytest.mark.parametrize("case", FIXED_CASES + SPARSE_CASES, ids=case_id)
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
-def test_gemv_matches_oracle(case, dtype):
-    for (K, N) in ((192, 4096), (80, 5376)):
+def test_gemv_matches_oracle(case, dtype, tiled):
+    if tiled and case in SPARSE_CASES:
+        pytest.skip("the variable-length layouts have no tiled form")
+    for (K, N) in ((192, 4096), (72, 5376)):
         raw = make_raw(case, K, N, seed=K + N + 31 * case[0])
         pk = oracle_pack(case, raw)
-        pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV)
+        pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV, tiled=tiled)
         W = R.dequant(pk, K, N, case[0], col_scale=raw["col_scale"], **kw_of(case))
         for M in (1, 2, 3, 4, 8, 16):
             x = acts(M, N, dtype, seed=M)
@@ -91,6 +97,47 @@ def test_gemv_matches_oracle(case, dtype):
             # the reference's own GEMV gate (test_gemv.py:162-167) is max|err|/max|ref| < 2e-5
             # for bf16 inputs with fp32 accumulation; hold the fp32 output to 1e-4
             assert np.abs(_np(y) - ref).max() / np.abs(ref).max() < 1e-4
+
+
+ALL_MFMA_CASES = [(F.BLKC, b, g, k) for b in (2, 3, 4) for g in (64, 128) for k in (10, 16, 23)] + \
+                 [(F.DENSEB, b, g, 0) for b in (2, 3, 4) for g in (64, 128)]
+
+
+@pytest.mark.parametrize("tiled", [False, True], ids=["rowmajor", "tiled"])
+@pytest.mark.parametrize("case", ALL_MFMA_CASES, ids=case_id)
+def test_gemv_every_kernel_configuration(case, tiled):
+    """Every instantiation of the matrix-core decode kernel (code width x survivors per block x
+    group size x activation rows 1..8), on shapes that give one, two and several macro-steps per
+    wavefront and a partial last step, run twice: results must match the oracle and each other."""
+    for (K, N) in ((32, 4096), (48, 5376), (16, 14336)):
+        raw = make_raw(case, K, N, seed=K + N + 7 * case[1])
+        pk = oracle_pack(case, raw)
+        pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV, tiled=tiled)
+        W = R.dequant(pk, K, N, case[0], col_scale=raw["col_scale"], **kw_of(case))
+        for M in range(1, 9):
+            x = acts(M, N, torch.bfloat16, seed=M) * (1.0 + 99.0 * (M == 5))
+            ref = R.forward_ref(W, _np(x))
+            y = ops.gemv(pm, x.to(DEV), out_dtype=torch.float32)
+            assert rel_fro(_np(y), ref) < TOL, f"{case_id(case)} {K}x{N} M={M}"
+            assert torch.equal(ops.gemv(pm, x.to(DEV), out_dtype=torch.float32), y)
+
+
+def test_gemv_batch_matches_single_calls():
+    case = (F.BLK1632_4, 4, 128, 16)
+    shapes = [(4096, 4096), (1024, 4096), (1024, 4096), (512, 14336)]
+    pms = [F.synth_packed(K, N, *case[:3], case[3], seed=i, device=DEV).to_tiled() for i, (K, N) in enumerate(shapes)]
+    for M in (1, 3, 8, 12):
+        xs = [acts(M, N, torch.float16, seed=N + i).to(DEV) for i, (K, N) in enumerate(shapes)]
+        bs = [torch.randn(K, device=DEV).half() for K, N in shapes]
+        ys = ops.gemv_batch(pms, xs, biases=bs, out_dtype=torch.float32)
+        for pm, x, b, y in zip(pms, xs, bs, ys):
+            assert torch.equal(y, ops.gemv(pm, x, bias=b, out_dtype=torch.float32))
+    # a mixed batch (different code widths) degrades to single calls and still agrees
+    pm3 = F.synth_packed(256, 4096, F.BLKC, 3, 128, 10, seed=5, device=DEV)
+    xs = [acts(2, 4096, torch.bfloat16, seed=1).to(DEV)] * 2
+    ys = ops.gemv_batch([pms[0], pm3], xs, out_dtype=torch.float32)
+    assert torch.equal(ys[0], ops.gemv(pms[0], xs[0], out_dtype=torch.float32))
+    assert torch.equal(ys[1], ops.gemv(pm3, xs[1], out_dtype=torch.float32))
 
 
 def test_gemv_output_dtypes_bias_and_strided_x():
@@ -120,9 +167,14 @@ def test_gemv_output_dtypes_bias_and_strided_x():
 
 @pytest.mark.parametrize("case", [(F.BLK1632_4, 4, 128, 16), (F.BLKC, 3, 128, 10), (F.BLKC, 2, 64, 23),
                                   (F.BLK1632_6, 6, 128, 16)], ids=case_id)
-def test_gemv_pruned_columns_contribute_exactly_zero(case):
-    """Restates test_gemv.py:403-455: a column-uniform mask, huge activations at the pruned
-    columns; the output must be bit-identical, with the zero point on and off the grid."""
+@pytest.mark.parametrize("tiled", [False, True], ids=["rowmajor", "tiled"])
+def test_gemv_pruned_columns_contribute_exactly_zero(case, tiled):
+    """Restates test_gemv.py:403-455: a column-uniform mask and huge activations at the pruned
+    columns, with the zero point on and off the grid.  A pruned column multiplies a literal 0 in
+    every kernel.  The matrix-core kernel quantises activations per 128-column chunk relative to
+    the chunk's largest magnitude, so (a) activations that keep every chunk maximum unchanged must
+    leave the output bit-identical, and (b) 1e4 at every pruned column (which rescales the chunks)
+    must still agree with the oracle, which it could not if a pruned weight leaked at all."""
     layout, bits, group, keep = case
     K, N = 256, 5376
     rng = np.random.default_rng(7)
@@ -130,6 +182,7 @@ def test_gemv_pruned_columns_contribute_exactly_zero(case):
     idx = np.argsort(rng.random((N // 32, 32)), axis=1)[:, :keep]
     np.put_along_axis(pat, idx, True, axis=1)
     keepm = np.broadcast_to(pat.reshape(1, N), (K, N))
+    pruned = torch.from_numpy(~pat.reshape(N))
     nl = (1 << bits) - 1
     q = rng.integers(0, nl + 1, (K, N)).astype(np.uint8)
     scale = (rng.random((K, N // group)) * 0.01 + 1e-3).astype(np.float16)
@@ -137,14 +190,23 @@ def test_gemv_pruned_columns_contribute_exactly_zero(case):
         zero = rng.integers(0, nl + 1, (K, N // group)).astype(np.float16) if zmode == "ongrid" \
             else np.full((K, N // group), nl + 37, np.float16)
         pk = R.pack_matrix(R.pack_bits(keepm), q, scale, zero, layout, fix_zero=(zmode == "ongrid"), **kw_of(case))
-        pm = packed_from_oracle(case, pk, None, K, N, DEV)
+        pm = packed_from_oracle(case, pk, None, K, N, DEV, tiled=tiled)
+        W = R.dequant(pk, K, N, layout, **kw_of(case))
+        assert (W[:, ~pat.reshape(N)] == 0).all()
         for dtype in (torch.bfloat16, torch.float16):
             x0 = acts(1, N, dtype, seed=1)
-            xh = x0.clone(); xh[0, torch.from_numpy(~pat.reshape(N))] = 1.0e4
+            cmax = x0.float().abs().reshape(N // 128, 128).amax(1, keepdim=True).expand(N // 128, 128).reshape(1, N)
+            xm = x0.clone(); xm[0, pruned] = (-cmax).to(dtype)[0, pruned]      # chunk maxima unchanged
+            xh = x0.clone(); xh[0, pruned] = 1.0e4
+            ref = R.forward_ref(W, _np(x0))
             for M in (1, 4):
                 y0 = ops.gemv(pm, x0.expand(M, N).contiguous().to(DEV), out_dtype=torch.float32)
+                ym = ops.gemv(pm, xm.expand(M, N).contiguous().to(DEV), out_dtype=torch.float32)
                 yh = ops.gemv(pm, xh.expand(M, N).contiguous().to(DEV), out_dtype=torch.float32)
-                assert torch.equal(y0, yh), f"{case_id(case)} zero={zmode} {dtype} M={M}"
+                assert torch.equal(y0, ym), f"{case_id(case)} zero={zmode} {dtype} M={M}"
+                assert rel_fro(_np(yh)[0], ref[0]) < TOL, f"{case_id(case)} zero={zmode} {dtype} M={M}"
+                if layout == F.BLK1632_6:                      # float row kernel: exact in any case
+                    assert torch.equal(y0, yh)
         assert (_np(ops.dequant(pm))[:, ~pat.reshape(N)] == 0).all()
 
 
@@ -152,7 +214,7 @@ def test_gemv_rows_are_independent_of_batch_and_run_to_run_identical():
     """The reference's determinism gate: M=4 is bit-exact 4 x M=1 (docs/KERNELS.md:151-155)."""
     case = (F.BLK1632_4, 4, 128, 16)
     K, N = 512, 4096
-    pm = F.synth_packed(K, N, *case[:3], case[3], seed=11, device=DEV)
+    pm = F.synth_packed(K, N, *case[:3], case[3], seed=11, device=DEV).to_tiled()
     x = acts(4, N, torch.bfloat16, seed=3).to(DEV)
     y4 = ops.gemv(pm, x, out_dtype=torch.float32)
     for i in range(4):
@@ -161,13 +223,14 @@ def test_gemv_rows_are_independent_of_batch_and_run_to_run_identical():
 
 
 # ------------------------------------------------------------------ prefill GEMM
+@pytest.mark.parametrize("tiled", [False, True], ids=["rowmajor", "tiled"])
 @pytest.mark.parametrize("case", FIXED_CASES, ids=case_id)
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
-def test_gemm_matches_oracle(case, dtype):
-    K, N = 320, 1024
+def test_gemm_matches_oracle(case, dtype, tiled):
+    K, N = 328, 1024
     raw = make_raw(case, K, N, seed=77 + case[0])
     pk = oracle_pack(case, raw)
-    pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV)
+    pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV, tiled=tiled)
     W = R.dequant(pk, K, N, case[0], col_scale=raw["col_scale"], **kw_of(case))
     for M in (16, 100, 512):                                # the reference's M set (test_gemm.py:162-195)
         x = acts(M, N, dtype, seed=M)
@@ -226,7 +289,8 @@ def test_full_size_properties(K, N, case):
     """Shapes of the benchmark configurations, where the CPU oracle is too slow for a full
     comparison: linearity in x, agreement between the decode and the prefill kernel, agreement
     of both with the dequantised dense weight on sampled rows (oracle on 32 rows)."""
-    pm = F.synth_packed(K, N, case[0], case[1], case[2], case[3] or None, seed=K % 97, device=DEV)
+    pm_rm = F.synth_packed(K, N, case[0], case[1], case[2], case[3] or None, seed=K % 97, device=DEV)
+    pm = pm_rm.to_tiled()
     x = acts(2, N, torch.bfloat16, seed=5).to(DEV)
     y = ops.gemv(pm, x, out_dtype=torch.float32)
     # linearity: activations scaled by 2 and rows swapped
@@ -237,12 +301,13 @@ def test_full_size_properties(K, N, case):
     assert rel_fro(_np(yg), _np(y)) < TOL
     # sampled rows against the oracle
     rows = np.linspace(0, K - 1, 32).astype(int)
-    pk = dict(data=pm.array("data").cpu().numpy(), scale=pm.array("scale").cpu().numpy().reshape(K, -1),
-              zero=pm.array("zero").cpu().numpy().reshape(K, -1), row_off=None)
+    assert torch.equal(ops.gemv(pm_rm, x, out_dtype=torch.float32), y)          # both byte orders, same sums
+    pk = dict(data=pm_rm.array("data").cpu().numpy(), scale=pm_rm.array("scale").cpu().numpy().reshape(K, -1),
+              zero=pm_rm.array("zero").cpu().numpy().reshape(K, -1), row_off=None)
     stride = R.row_stride(case[0], N, case[1], case[2], case[3] or None)
     sub = dict(data=np.concatenate([pk["data"][r * stride:(r + 1) * stride] for r in rows] + [np.zeros(64, np.uint8)]),
                scale=pk["scale"][rows], zero=pk["zero"][rows], row_off=None)
-    Wsub = R.dequant(sub, len(rows), N, case[0], col_scale=pm.array("col_scale").cpu().numpy(), **kw_of(case))
+    Wsub = R.dequant(sub, len(rows), N, case[0], col_scale=pm_rm.array("col_scale").cpu().numpy(), **kw_of(case))
     Wg = _np(ops.dequant(pm, torch.float32))
     assert np.array_equal(Wg[rows], Wsub)
     assert rel_fro(_np(y)[:, rows], R.forward_ref(Wsub, _np(x))) < TOL

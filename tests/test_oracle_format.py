@@ -288,3 +288,26 @@ def test_blob_alignment():
     assert all(o % 256 == 0 for o in offs.values()) and blob.size % 256 == 0
     assert np.array_equal(blob[offs["data"]: offs["data"] + pk["data"].size], pk["data"])
     assert R.stream_bytes(pk) == 4 * 96 + 4 * 2 * 2 + 4 * 2
+
+
+# ------------------------------------------------------------------ tile-interleaved order
+@pytest.mark.parametrize("layout,kw", [c for c in LAYOUT_CASES if c[0] not in R.SPARSE_FAMILY])
+def test_tile16_is_a_byte_permutation(layout, kw):
+    K, N = 40, 384                       # 2.5 tiles: exercises the zero padding rows
+    raw, bits, group, kpb = _raw_for(layout, kw, K, N, 21)
+    pk = R.pack_matrix(raw["mask"], raw["q"], raw["scale"], raw["zero"], layout, **kw)
+    t = R.tile16(pk, K, N, layout, **kw)
+    stride = R.row_stride(layout, N, bits, group, kpb)
+    G = N // group
+    assert t["data"].size == 48 * stride + 512 and t["scale"].size == 48 * G and t["zero"].size == 48 * G
+    rng = np.random.default_rng(0)
+    for _ in range(200):                 # the closed-form index map, element by element
+        k, o, g = int(rng.integers(K)), int(rng.integers(stride)), int(rng.integers(G))
+        assert t["data"][(k // 16) * 16 * stride + ((o // 16) * 16 + k % 16) * 16 + o % 16] == pk["data"][k * stride + o]
+        assert t["scale"][((k // 16) * G + g) * 16 + k % 16] == pk["scale"].reshape(K, G)[k, g]
+        assert t["zero"][((k // 16) * G + g) * 16 + k % 16] == pk["zero"].reshape(K, G)[k, g]
+    assert sorted(t["data"][: 48 * stride].tolist()) == sorted(pk["data"][: K * stride].tolist() + [0] * (8 * stride))
+    u = R.untile16(t, K, N, layout, **kw)
+    assert np.array_equal(u["data"], pk["data"]) and np.array_equal(u["scale"], pk["scale"].reshape(K, G))
+    assert np.array_equal(u["zero"], pk["zero"].reshape(K, G))
+    assert np.array_equal(R.dequant(u, K, N, layout, **kw), R.dequant(pk, K, N, layout, **kw))
