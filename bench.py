@@ -87,7 +87,7 @@ def main():
     n_copies = max(2, -(-2 * 256 * 2**20 // set_bytes))
     sets = []
     for c in range(n_copies):
-        sets.append([F.synth_packed(K, N, layout, a.bits, a.group, a.keep, seed=1000 * c + i, device=dev)
+        sets.append([F.synth_packed(K, N, layout, a.bits, a.group, a.keep, seed=1000 * c + i, device=dev).to_tiled()
                      for i, (_, K, N) in enumerate(shapes)])
     xs = {N: torch.randn(M, N, device=dev, generator=torch.Generator(device=dev).manual_seed(N)).to(dt)
           for _, _, N in shapes}

@@ -144,6 +144,11 @@ struct GvMat {
   int nS;                  // macro-steps per tile = ceil(N / 512)
   int cost0;               // sum of ntiles * nS over the matrices before this one
   int spi, sk;             // macro-steps per work item, work items per tile
+  // branch-free addressing of either byte order: row k starts at data + (k >> rsh) * row_a +
+  // (k & rmask) * 16 and its 16-byte units are ustride apart; the scale / zero entry of
+  // (k, g) has index ((k >> rsh) * G + g) * (rmask + 1) + (k & rmask)
+  int rsh, rmask;
+  uint32_t row_a, ustride;
 };
 
 struct GvBatch {
@@ -287,32 +292,64 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     const int nitems = (t_hi - t_lo) * SK;
     const int gt = b.nslot >> 1;                                  // tiles per barrier group
 
+    // matrix constants, read from the kernel arguments once
+    const uint8_t* const m_data = m.data;
+    const uint16_t* const m_scale = m.scale;
+    const uint8_t* const m_zero = m.zero;
+    const int m_K = m.K, m_G = m.G, rsh = gm.rsh, rmask = gm.rmask, mmul = gm.rmask + 1;
+    const uint32_t row_a = gm.row_a, ustride = gm.ustride, code_u0 = m.code_off >> 4;
+    const int last_tile = t_hi - 1, last_S = nS - 1;
+
+    // ---- issue the loads of one (tile, macro-step) position; out-of-range positions are clamped
     auto issue = [&](int tile, int S, Loads<C>& L) {
+      tile = tile < last_tile ? tile : last_tile;
+      S = S < last_S ? S : last_S;
       int row = tile * 16 + wr;
-      row = row < m.K ? row : m.K - 1;
-      const RowView rv = row_view(m, row);
+      row = row < m_K ? row : m_K - 1;
+      const uint8_t* rb = m_data + (size_t)(row >> rsh) * row_a + (size_t)(row & rmask) * 16;
       int ch = 4 * S + kq;
       ch = ch < NCH ? ch : NCH - 1;
       if (!C::DENSE) {
-        const uint4 v = *(const uint4*)rv.unit(ch);
+        const uint4 v = *(const uint4*)(rb + (size_t)ch * ustride);
         L.mk[0] = v.x; L.mk[1] = v.y; L.mk[2] = v.z; L.mk[3] = v.w;
       }
       // code bits of the chunk: bit ch*CHB of the code plane, fetched as whole 16-byte units
-      const uint32_t u0 = (m.code_off >> 4) + (C::VEC16 ? (uint32_t)ch * (C::CHB / 128) : (((uint32_t)ch * C::CHB) >> 7));
+      const uint32_t u0 = code_u0 + (C::VEC16 ? (uint32_t)ch * (C::CHB / 128) : (((uint32_t)ch * C::CHB) >> 7));
 #pragma unroll
       for (int i = 0; i < C::NL / 4; ++i) {
-        const uint4 v = *(const uint4*)rv.unit(u0 + i);
+        const uint4 v = *(const uint4*)(rb + (size_t)(u0 + i) * ustride);
         L.raw[4 * i] = v.x; L.raw[4 * i + 1] = v.y; L.raw[4 * i + 2] = v.z; L.raw[4 * i + 3] = v.w;
       }
-      if (C::NGC == 1) L.zraw = m.zero[meta_index(m, row, ch)];
-      else L.zraw = (uint32_t)m.zero[meta_index(m, row, 2 * ch)] | ((uint32_t)m.zero[meta_index(m, row, 2 * ch + 1)] << 8);
-#pragma unroll
-      for (int g = 0; g < C::NGC; ++g) L.sc[g] = m.scale[meta_index(m, row, ch * C::NGC + g)];
+      const size_t mi0 = ((size_t)(row >> rsh) * m_G + (size_t)ch * C::NGC) * mmul + (row & rmask);
+      if (C::NGC == 1) {
+        L.zraw = m_zero[mi0];
+        L.sc[0] = m_scale[mi0];
+      } else {
+        L.zraw = (uint32_t)m_zero[mi0] | ((uint32_t)m_zero[mi0 + mmul] << 8);
+        L.sc[0] = m_scale[mi0];
+        L.sc[C::NGC - 1] = m_scale[mi0 + mmul];
+      }
     };
 
-    Loads<C> cur, nxt;
-    int q = wave;                                                 // this wave's current item
-    if (q < nitems) issue(t_lo + q / SK, (q % SK) * spi, cur);    // in flight during the staging below
+    // this wave's sequence of (tile, part, macro-step) positions: items wave, wave+16, ...
+    struct Pos { int tl, part, S; };
+    const int ntl = t_hi - t_lo;
+    const int dq_t = GV_WAVES / SK, dq_p = GV_WAVES % SK;
+    auto advance = [&](Pos& p) -> bool {                           // false past the last position
+      const int s_end = (p.part * spi + spi < nS) ? p.part * spi + spi : nS;
+      if (p.S + 1 < s_end) { ++p.S; return true; }
+      p.tl += dq_t; p.part += dq_p;
+      if (p.part >= SK) { p.part -= SK; ++p.tl; }
+      p.S = p.part * spi;
+      return p.tl < ntl;
+    };
+    Pos p0{wave / SK, wave % SK, (wave % SK) * spi};
+    bool v0 = p0.tl < ntl;
+    Pos p1 = p0; bool v1 = v0 && advance(p1);
+    Pos p2 = p1; bool v2 = v1 && advance(p2);
+    Loads<C> cur, nx1, nx2;                                       // two steps of loads stay in flight
+    issue(t_lo + p0.tl, p0.S, cur);
+    issue(t_lo + p1.tl, p1.S, nx1);
 
     // ---- stage: selector table and counters (once), activation digits and deltas of this matrix
     __syncthreads();                                              // previous matrix fully consumed
@@ -339,22 +376,19 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     __syncthreads();
 
     int bars = 0;                                                 // group barriers passed so far
-    for (; q < nitems; q += GV_WAVES) {
-      const int tl = q / SK, part = q - tl * SK;
+    float ysum[MP];
+    while (v0) {
+      const int tl = p0.tl, part = p0.part, S = p0.S;
       const int tile = t_lo + tl;
-      const int s_begin = part * spi, s_end = (s_begin + spi < nS) ? s_begin + spi : nS;
-      // slots of tile group g are reused by group g + 2: wait until group g - 1 is complete
-      for (const int g = tl / gt; bars < g; ++bars) __syncthreads();
-
-      float ysum[MP];
+      const int s_end = (part * spi + spi < nS) ? part * spi + spi : nS;
+      if (S == part * spi) {                                      // first step of an item
+        // slots of tile group g are reused by group g + 2: wait until group g - 1 is complete
+        for (const int g = tl / gt; bars < g; ++bars) __syncthreads();
 #pragma unroll
-      for (int p = 0; p < MP; ++p) ysum[p] = 0.f;
-
-      for (int S = s_begin; S < s_end; ++S) {
-        // prefetch this wave's next step
-        if (S + 1 < s_end) issue(tile, S + 1, nxt);
-        else if (q + GV_WAVES < nitems) { const int q2 = q + GV_WAVES; issue(t_lo + q2 / SK, (q2 % SK) * spi, nxt); }
-
+        for (int p = 0; p < MP; ++p) ysum[p] = 0.f;
+      }
+      issue(t_lo + p2.tl, p2.S, nx2);
+      {
         const int chunk = 4 * S + kq;
         const bool valid = chunk < NCH;
         uint32_t aaddr[MP];
@@ -450,7 +484,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
               // One idle issue slot after every MFMA.  Without it some instantiations of this
               // kernel (register allocations in which the accumulator chain changes registers)
               // returned run-to-run different sums on gfx950; with it every configuration is exact.
-              asm volatile("s_nop 1");
+              asm("s_nop 1" : "+v"(acc[p]));
             }
             // ---- end of a quantisation group: int32 -> float, times scale * delta
             if ((C::NGC == 2 && t == 3) || t == 7) {
@@ -465,9 +499,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
             }
           }
         }
-        cur = nxt;
       }
-
+      cur = nx1; nx1 = nx2;
+      if (S + 1 == s_end) {
       // ---- the item is done: add the four lane quarters (the four chunks of every macro-step)
       float part_sum[MP];
 #pragma unroll
@@ -509,6 +543,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
           if (lane == 0) cnt[slot] = 0;
         }
       }
+      }
+      p0 = p1; v0 = v1; p1 = p2; v1 = v2;
+      if (v2) v2 = advance(p2);
     }
     // every wave passes the same number of group barriers
     const int ngroups = ((t_hi - t_lo) + gt - 1) / gt;
@@ -615,6 +652,8 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
     items += M * (m.N / 16);
     g.m = m; g.xq = p.xq; g.delta = p.delta; g.y = calls[i].y; g.bias = calls[i].bias; g.ldy = calls[i].ldy;
     g.ntiles = (m.K + 15) / 16; g.nS = (m.N / 128 + 3) / 4; g.cost0 = cost;
+    g.rsh = m.tiled ? 4 : 0; g.rmask = m.tiled ? 15 : 0;
+    g.row_a = m.tiled ? m.stride * 16u : m.stride; g.ustride = m.tiled ? 256u : 16u;
     cost += g.ntiles * g.nS;
     tiles += g.ntiles;
     xq_cap = xq_cap > M * NDIG * m.N ? xq_cap : M * NDIG * m.N;
@@ -635,7 +674,8 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
     GvMat& g = gb.mat[i];
     int s = spi;
     while ((g.nS + s - 1) / s > 16) ++s;
-    g.spi = s; g.sk = (g.nS + s - 1) / s;
+    g.sk = (g.nS + s - 1) / s;
+    g.spi = (g.nS + g.sk - 1) / g.sk;                  // equal parts
     sk_cap = sk_cap > g.sk ? sk_cap : g.sk;
   }
   // reduction slots: as many as fit 24 KB, a power of two between 2 and 64
