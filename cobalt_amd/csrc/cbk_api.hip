@@ -180,8 +180,8 @@ int cbk_gemv_batch(int n, const cbk_desc* descs, const void* const* xs, const in
   if (fast) {
     size_t need = 0;
     for (int i = 0; i < n; ++i) need += gemv_fast_workspace(calls[i].m, M > 4 ? 4 : M);
-    if (!workspace || workspace_bytes < need) return CBK_ERR_WORKSPACE;
-    if ((uintptr_t)workspace & 255) return CBK_ERR_ALIGN;
+    if (need && (!workspace || workspace_bytes < need)) return CBK_ERR_WORKSPACE;
+    if (need && ((uintptr_t)workspace & 255)) return CBK_ERR_ALIGN;
     const size_t ysz = y_dtype == CBK_F32 ? 4 : 2;
     for (int m0 = 0; m0 < M; m0 += 4) {                 // at most 4 activation rows per launch
       const int mc = M - m0 < 4 ? M - m0 : 4;

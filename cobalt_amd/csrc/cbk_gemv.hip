@@ -135,8 +135,9 @@ struct Cfg {
 // One matrix of a batched launch.
 struct GvMat {
   DMat m;
-  const int8_t* xq;        // activation digits [M][3][N] (most significant plane first)
-  const float* delta;      // [M][N/128 + 4], zero beyond N/128
+  const uint16_t* x;       // activations [M][ldx], fp16 or bf16 bits
+  int64_t ldx;
+  int order;               // digit order inside a 16-column fragment: 0 column order, 1 / 2 dense
   void* y;
   const void* bias;
   int64_t ldy;
@@ -153,7 +154,7 @@ struct GvMat {
 
 struct GvBatch {
   GvMat mat[GV_MAX_BATCH];
-  int n, M, ydt, total_cost;
+  int n, M, xdt, ydt, total_cost;
   int xq_cap, delta_cap;   // LDS bytes reserved for digits / floats reserved for delta
   int sk_cap, nslot, red_floats;   // reduction slots: nslot x sk_cap x M x 16 floats
 };
@@ -169,78 +170,61 @@ __host__ __device__ constexpr int frag_col(int bits, bool dense, int bi) {
 
 // ------------------------------------------------------------------ activation prep
 // x' = x * col_scale per 128-column chunk -> delta and three signed int8 digits per column:
-// x' ~= delta * (65536*d2 + 256*d1 + d0),  delta = max|x'| / (127 * 65536).  One thread = 16 columns.
-struct PrepMat {
-  const uint16_t* x;
-  const uint16_t* cs;
-  int64_t ldx;
-  int N;
-  int order;               // 0 column order, 1 dense 3/4-bit order, 2 dense 2-bit order
-  int8_t* xq;
-  float* delta;
-  int item0;               // first item of this matrix
-};
-struct PrepBatch { PrepMat mat[GV_MAX_BATCH]; int n, M, xdt, items; };
-
-__global__ __launch_bounds__(256) void gemv_prep_kernel(PrepBatch b) {
-  const int it = blockIdx.x * 256 + threadIdx.x;          // items are multiples of 8 per matrix
-  const bool ok = it < b.items;
-  int mi = 0;
+// x' ~= delta * (65536*d2 + 256*d1 + d0),  delta = max|x'| / (127 * 65536).  Every workgroup
+// converts the activations it needs into its own LDS (a few hundred instructions per thread,
+// overlapped with the first weight loads).  One thread converts 16 columns at a time; the
+// eight threads of a chunk agree on its maximum with three lane exchanges.
+__device__ inline void stage_activations(const uint16_t* x, int64_t ldx, const uint16_t* cs, int xdt, int order,
+                                         int M, int N, int8_t* xq, float* delta, int tid) {
+  const int n16 = N >> 4, NCH = N >> 7, items = M * n16;          // a multiple of 8
+  for (int it = tid; it < items; it += GV_THREADS) {
+    const int row = it / n16, c16 = it - row * n16;
+    const uint16_t* xp = x + (size_t)row * ldx + c16 * 16;
+    const uint4 xr[2] = {((const uint4*)xp)[0], ((const uint4*)xp)[1]};
+    uint4 cr[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+    if (cs) { cr[0] = ((const uint4*)(cs + c16 * 16))[0]; cr[1] = ((const uint4*)(cs + c16 * 16))[1]; }
+    const uint32_t* xw = (const uint32_t*)xr;
+    const uint32_t* cw = (const uint32_t*)cr;
+    float xv[16];
+    float mx = 0.f;
 #pragma unroll
-  for (int i = 1; i < GV_MAX_BATCH; ++i) mi = (i < b.n && it >= b.mat[i].item0) ? i : mi;
-  const PrepMat& pm = b.mat[mi];
-  const int N = pm.N, n16 = N >> 4, NCH = N >> 7;
-  const int loc = ok ? it - pm.item0 : 0;
-  const int row = loc / n16, c16 = loc % n16;
-  const uint16_t* xp = pm.x + (size_t)row * pm.ldx + c16 * 16;
-  uint4 xr[2] = {((const uint4*)xp)[0], ((const uint4*)xp)[1]};
-  uint4 cr[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
-  if (pm.cs) { cr[0] = ((const uint4*)(pm.cs + c16 * 16))[0]; cr[1] = ((const uint4*)(pm.cs + c16 * 16))[1]; }
-  const uint32_t* xw = (const uint32_t*)xr;
-  const uint32_t* cw = (const uint32_t*)cr;
-  float xv[16];
-  float mx = 0.f;
-#pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    const uint16_t xb = (uint16_t)(xw[e >> 1] >> (16 * (e & 1)));
-    float v = b.xdt == CBK_F16 ? h2f(xb) : bf2f(xb);
-    if (pm.cs) v *= h2f((uint16_t)(cw[e >> 1] >> (16 * (e & 1))));
-    xv[e] = ok ? v : 0.f;
-    mx = fmaxf(mx, fabsf(xv[e]));
-  }
-  mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
-  mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
-  mx = fmaxf(mx, __shfl_xor(mx, 4, 64));
-  const float d = mx > 0.f ? mx / 8323072.f : 1.f;
-  const float inv = 1.f / d;
-  uint32_t dw[NDIG][4];
-#pragma unroll
-  for (int k = 0; k < NDIG; ++k)
-#pragma unroll
-    for (int q = 0; q < 4; ++q) dw[k][q] = 0u;
-#pragma unroll
-  for (int bi = 0; bi < 16; ++bi) {
-    const int e = pm.order == 0 ? bi : (pm.order == 1 ? frag_col(4, true, bi) : frag_col(2, true, bi));
-    float v = xv[0];
-    if (pm.order == 0) v = xv[bi];
-    else if (pm.order == 1) v = xv[frag_col(4, true, bi)];
-    else v = xv[frag_col(2, true, bi)];
-    (void)e;
-    int X = (int)rintf(v * inv);                       // |X| <= 127 * 65536
-    const int d0 = (int)(int8_t)(X & 0xFF);
-    X = (X - d0) >> 8;
-    const int d1 = (int)(int8_t)(X & 0xFF);
-    const int d2 = (X - d1) >> 8;
-    dw[0][bi >> 2] |= ((uint32_t)d2 & 0xFFu) << (8 * (bi & 3));
-    dw[1][bi >> 2] |= ((uint32_t)d1 & 0xFFu) << (8 * (bi & 3));
-    dw[2][bi >> 2] |= ((uint32_t)d0 & 0xFFu) << (8 * (bi & 3));
-  }
-  if (ok) {
+    for (int e = 0; e < 16; ++e) {
+      const uint16_t xb = (uint16_t)(xw[e >> 1] >> (16 * (e & 1)));
+      float v = xdt == CBK_F16 ? h2f(xb) : bf2f(xb);
+      if (cs) v *= h2f((uint16_t)(cw[e >> 1] >> (16 * (e & 1))));
+      xv[e] = v;
+      mx = fmaxf(mx, fabsf(v));
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 4, 64));
+    const float d = mx > 0.f ? mx / 8323072.f : 1.f;
+    const float inv = 1.f / d;
+    uint32_t dw[NDIG][4];
 #pragma unroll
     for (int k = 0; k < NDIG; ++k)
-      *(uint4*)(pm.xq + ((size_t)row * NDIG + k) * N + c16 * 16) = make_uint4(dw[k][0], dw[k][1], dw[k][2], dw[k][3]);
-    if ((c16 & 7) == 0) pm.delta[row * (NCH + 4) + (c16 >> 3)] = d;
-    if (c16 < 4) pm.delta[row * (NCH + 4) + NCH + c16] = 0.f;              // chunks past N
+#pragma unroll
+      for (int q = 0; q < 4; ++q) dw[k][q] = 0u;
+#pragma unroll
+    for (int bi = 0; bi < 16; ++bi) {
+      float v;
+      if (order == 0) v = xv[bi];
+      else if (order == 1) v = xv[frag_col(4, true, bi)];
+      else v = xv[frag_col(2, true, bi)];
+      int X = (int)rintf(v * inv);                       // |X| <= 127 * 65536
+      const int d0 = (int)(int8_t)(X & 0xFF);
+      X = (X - d0) >> 8;
+      const int d1 = (int)(int8_t)(X & 0xFF);
+      const int d2 = (X - d1) >> 8;
+      dw[0][bi >> 2] |= ((uint32_t)d2 & 0xFFu) << (8 * (bi & 3));
+      dw[1][bi >> 2] |= ((uint32_t)d1 & 0xFFu) << (8 * (bi & 3));
+      dw[2][bi >> 2] |= ((uint32_t)d0 & 0xFFu) << (8 * (bi & 3));
+    }
+#pragma unroll
+    for (int k = 0; k < NDIG; ++k)
+      *(uint4*)(xq + ((size_t)row * NDIG + k) * N + c16 * 16) = make_uint4(dw[k][0], dw[k][1], dw[k][2], dw[k][3]);
+    if ((c16 & 7) == 0) delta[row * (NCH + 4) + (c16 >> 3)] = d;
+    if (c16 < 4) delta[row * (NCH + 4) + NCH + c16] = 0.f;          // chunks past N
   }
 }
 
@@ -365,14 +349,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       }
       first = false;
     }
-    {
-      const int n16 = (b.M * NDIG * N) >> 4;
-      const uint4* src = (const uint4*)gm.xq;
-      uint4* dst = (uint4*)xq;
-      for (int i = tid; i < n16; i += GV_THREADS) dst[i] = src[i];
-      const int nd = b.M * (NCH + 4);
-      for (int i = tid; i < nd; i += GV_THREADS) delta[i] = gm.delta[i];
-    }
+    stage_activations(gm.x, gm.ldx, m.cs, b.xdt, gm.order, b.M, N, xq, delta, tid);
     __syncthreads();
 
     int bars = 0;                                                 // group barriers passed so far
@@ -575,9 +552,7 @@ bool gemv_same_config(const DMat& a, const DMat& b) {
   return da == db && a.bits == b.bits && a.group == b.group && (da || a.keep == b.keep);
 }
 
-size_t gemv_fast_workspace(const DMat& m, int M) {
-  return up256((size_t)M * NDIG * m.N) + up256((size_t)M * (m.N / 128 + 4) * 4);
-}
+size_t gemv_fast_workspace(const DMat&, int) { return 0; }   // activations are staged in LDS
 
 struct GvCall {           // one matrix of a batched call, host side
   DMat m;
@@ -632,25 +607,16 @@ static int launch_keep(const GvBatch& b, size_t lds, int blocks, hipStream_t st)
 int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, void* workspace, size_t ws_bytes,
                            hipStream_t st) {
   if (n < 1 || n > GV_MAX_BATCH) return CBK_ERR_SHAPE;
-  PrepBatch pb;
   GvBatch gb;
-  pb.n = gb.n = n; pb.M = gb.M = M; pb.xdt = xdt; gb.ydt = ydt;
-  size_t off = 0;
-  int items = 0, cost = 0, xq_cap = 0, delta_cap = 0, tiles = 0;
+  gb.n = n; gb.M = M; gb.xdt = xdt; gb.ydt = ydt;
+  int cost = 0, xq_cap = 0, delta_cap = 0, tiles = 0;
   for (int i = 0; i < n; ++i) {
     const DMat& m = calls[i].m;
     const bool dense = family_of(m.layout) == FAM_DENSE;
-    PrepMat& p = pb.mat[i];
     GvMat& g = gb.mat[i];
-    p.x = (const uint16_t*)calls[i].x; p.cs = m.cs; p.ldx = calls[i].ldx; p.N = m.N;
-    p.order = !dense ? 0 : (m.bits == 2 ? 2 : 1);
-    p.xq = (int8_t*)workspace + off;
-    off += up256((size_t)M * NDIG * m.N);
-    p.delta = (float*)((uint8_t*)workspace + off);
-    off += up256((size_t)M * (m.N / 128 + 4) * 4);
-    p.item0 = items;
-    items += M * (m.N / 16);
-    g.m = m; g.xq = p.xq; g.delta = p.delta; g.y = calls[i].y; g.bias = calls[i].bias; g.ldy = calls[i].ldy;
+    g.m = m; g.x = (const uint16_t*)calls[i].x; g.ldx = calls[i].ldx;
+    g.order = !dense ? 0 : (m.bits == 2 ? 2 : 1);
+    g.y = calls[i].y; g.bias = calls[i].bias; g.ldy = calls[i].ldy;
     g.ntiles = (m.K + 15) / 16; g.nS = (m.N / 128 + 3) / 4; g.cost0 = cost;
     g.rsh = m.tiled ? 4 : 0; g.rmask = m.tiled ? 15 : 0;
     g.row_a = m.tiled ? m.stride * 16u : m.stride; g.ustride = m.tiled ? 256u : 16u;
@@ -659,8 +625,7 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
     xq_cap = xq_cap > M * NDIG * m.N ? xq_cap : M * NDIG * m.N;
     delta_cap = delta_cap > M * (m.N / 128 + 4) ? delta_cap : M * (m.N / 128 + 4);
   }
-  if (off > ws_bytes || !workspace) return CBK_ERR_WORKSPACE;
-  pb.items = items;
+  (void)workspace; (void)ws_bytes;
   gb.total_cost = cost; gb.xq_cap = xq_cap; gb.delta_cap = delta_cap;
   int blocks = tiles < 256 ? tiles : 256;                       // one persistent workgroup per CU
   if (const char* e = getenv("CBK_GV_BLOCKS")) blocks = atoi(e) < tiles ? atoi(e) : tiles;
@@ -683,7 +648,6 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
   int nslot = 64;
   while (nslot > 2 && (size_t)nslot * slot_floats * 4 > 24 * 1024) nslot >>= 1;
   gb.sk_cap = sk_cap; gb.nslot = nslot; gb.red_floats = nslot * slot_floats;
-  hipLaunchKernelGGL(gemv_prep_kernel, dim3((items + 255) / 256), dim3(256), 0, st, pb);
   const size_t lds = (size_t)LUT_BYTES + ZERO_BYTES + xq_cap + (size_t)delta_cap * 4 +
                      (size_t)gb.red_floats * 4 + (size_t)nslot * 4;
   const int bits = gb.mat[0].m.bits;
