@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libcbk_hip.so")
-SOURCES = ["cbk_api.hip", "cbk_dequant.hip", "cbk_gemv_generic.hip", "cbk_gemv.hip", "cbk_gemm.hip"]
+SOURCES = ["cbk_api.hip", "cbk_dequant.hip", "cbk_gemv_generic.hip", "cbk_gemv.hip", "cbk_gemm.hip", "cbk_gemm_big.hip"]
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-shared", "-std=c++17",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-command-line-argument"]

@@ -15,6 +15,13 @@ size_t gemv_fast_workspace(const DMat&, int M);
 constexpr int kMaxBatch = 8;
 int launch_gemm(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*,
                 hipStream_t);
+int launch_gemm_big(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*, void*, size_t,
+                    hipStream_t);
+size_t gemm_big_workspace(const DMat&, int M);
+// the 256 x 256 tile kernel pays off once a call fills at least one token tile halfway
+static inline bool gemm_big_takes(const DMat& m, int M) {
+  return M > 128 && family_of(m.layout) != FAM_SPARSE && m.cs_rows <= 1;
+}
 
 static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
@@ -139,6 +146,7 @@ size_t cbk_workspace_bytes(const cbk_desc* in, int M) {
   if (to_dmat(in, &m, false)) return 0;
   const int mc = M > 4 ? 4 : M;
   if (M >= 1 && M <= 16 && gemv_fast_takes(m, mc)) return gemv_fast_workspace(m, mc);
+  if (gemm_big_takes(m, M)) return gemm_big_workspace(m, M);
   return 0;
 }
 
@@ -224,12 +232,14 @@ int cbk_gemv(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ldx,
 
 int cbk_gemm(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ldx, void* y, int y_dtype,
              int64_t ldy, const void* bias, void* workspace, size_t workspace_bytes, void* stream) {
-  (void)workspace; (void)workspace_bytes;
   DMat m;
   int rc = to_dmat(in, &m, true);
   if (rc) return rc;
   rc = check_io(x, x_dtype, M, ldx, y, y_dtype, ldy, m.N, m.K);
   if (rc) return rc;
+  if (gemm_big_takes(m, M))
+    return launch_gemm_big(m, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, workspace, workspace_bytes,
+                           (hipStream_t)stream);
   return launch_gemm(m, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, (hipStream_t)stream);
 }
 
