@@ -1,10 +1,24 @@
-"""Headline benchmark: decode GEMV over a Mistral-7B-shaped layer set in CBK1 form.
+"""Headline benchmark of the CBK1 sparse low-bit linear layer on one MI355X.
 
-One "step" is one pass of the hot path over one layer set: the seven M=1 GEMVs of a decoder
-layer (q, k, v, o, gate, up, down) at sparsity 0.5, 4-bit codes, group 128 (layout BLK1632_4,
-3.1875 bits per weight).  The packed weights of several distinct layer sets are resident in
-HBM before the timed region; successive steps rotate through them so that the streamed set
-exceeds twice the 256 MB Infinity Cache.  `value` is packed bytes streamed per second.
+Decode (the `value` of the JSON line).  One "step" is one pass of the hot path over one
+decoder-layer set: the seven M-row GEMVs of a layer (q, k, v, o, gate, up, down) at sparsity
+0.5, 4-bit codes, group 128 (layout BLK1632_4, 3.1875 bits per weight), launched as the four
+dependency phases of a decoder layer (q,k,v | o | gate,up | down), one batched kernel launch
+per phase, replayed from HIP graphs.  The packed weights of several distinct layer sets are
+resident in HBM before the timed region; successive steps rotate through them so that the
+streamed set exceeds twice the 256 MB Infinity Cache.  `value` is algorithmic bytes (packed
+rows + scales + zeros + col_scale + activations in + outputs out) streamed per second.
+
+`roofline` describes the decode kernel: algorithmic bytes per launch over the average launch
+duration, which is the timed region (HIP events recorded on the launch stream) divided by
+the number of launches in it; the gaps between launches are therefore counted as kernel time.
+
+`prefill_gemm` reports the prefill kernel at the Gemma-3-27B MLP shapes (M=2048, bf16) in
+TFLOP/s against the 2.5 PFLOP/s dense bf16/f16 MFMA peak.
+
+`cpu_baseline` is the C oracle (dequantise-then-matmul, OpenMP over rows) timed on the host
+cores on the SAME packed bytes as the first layer set, and doubles as a last parity check of
+the GPU outputs.
 
 python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mistral7b|gemma27b] [--m M]
 """
@@ -24,6 +38,12 @@ SHAPES = {
                  ("gate", 21504, 5376), ("up", 21504, 5376), ("down", 5376, 21504)],
 }
 HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = 2500.0          # dense bf16 / f16 MFMA peak of MI355X
+
+# HBM bytes per launch of the decode kernel (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, scaled by
+# the same counters read for a device-to-device copy of known size), keyed by
+# (workload, launch grouping, M); filled from the runs summarised under profiles/.
+MEASURED_TRAFFIC = {("mistral7b", "phase", 1): 22254182}
 
 
 def algorithmic_bytes(pm, M, e_x=2, e_y=2):
@@ -31,27 +51,65 @@ def algorithmic_bytes(pm, M, e_x=2, e_y=2):
     return pm.stream_bytes() + pm.cs_rows * pm.N * 2 + M * pm.N * e_x + M * pm.K * e_y
 
 
-def cpu_baseline(shape, layout, bits, group, keep, M, seed=0, budget_s=20.0):
-    """The oracle's dequantise-then-matmul forward on the host cores, on ONE matrix of the layer set."""
+def cpu_baseline(pms, shapes, xs, ys, M, budget_s=20.0):
+    """C oracle forward over the layer set on the host cores, on the bytes the GPU used."""
     import numpy as np
-    from oracle import cbk_ref as R
-    name, K, N = shape
-    raw = R.synth_raw_matrix(K, N, 1.0 - keep / 32.0, bits, seed=seed, block=32, group=group)
-    kw = {} if layout == R.BLK1632_4 else dict(bits=bits, group=group, keep_per_block=keep)
-    pk = R.pack_matrix(raw["mask"], raw["q"], raw["scale"], raw["zero"], layout, **kw)
-    x = np.random.default_rng(1).standard_normal((M, N)).astype(np.float16).astype(np.float32)
-    times = []
-    t_end = time.time() + budget_s
-    while len(times) < 5 and (time.time() < t_end or len(times) < 2):
+    from oracle import cbk_ref_c as C
+    nthreads = min(16, os.cpu_count() or 1)
+    C.set_threads(nthreads)
+    total_bytes, total_t, worst, done = 0, 0.0, 0.0, []
+    t_stop = time.time() + budget_s
+    for pm, (name, K, N) in zip(pms, shapes):
+        if done and time.time() > t_stop:
+            break
+        # one pass per matrix: the C decoder does ~15 ns of work per weight per thread
+        pk = dict(data=pm.array("data").cpu().numpy(), scale=pm.array("scale").cpu().numpy().reshape(K, -1),
+                  zero=pm.array("zero").cpu().numpy().reshape(K, -1))
+        cs = pm.array("col_scale").cpu().numpy().reshape(pm.cs_rows, N) if pm.cs_rows else None
+        x = xs[N].float().cpu().numpy()
         t0 = time.perf_counter()
-        W = R.dequant(pk, K, N, layout, col_scale=raw["col_scale"], **kw)
-        y = x @ W.T
-        times.append(time.perf_counter() - t0)
-    t = sorted(times)[len(times) // 2]
-    nbytes = R.stream_bytes(pk) + N * 2 + M * N * 2 + M * K * 2
-    return dict(value=nbytes / t / 1e9, unit="GB/s", cores=os.cpu_count(), kind="port",
-                sample=f"{name}_proj {K}x{N} only (1 of 7 matrices), numpy dequant+matmul per call, "
-                       f"median of {len(times)} runs, {t * 1e3:.0f} ms per call")
+        y = C.forward(pk, K, N, pm.layout, x, col_scale=cs, bits=pm.bits, group=pm.group, keep_per_block=pm.keep or None)
+        total_t += time.perf_counter() - t0
+        total_bytes += algorithmic_bytes(pm, M)
+        got = ys[name].float().cpu().numpy()
+        worst = max(worst, float(np.linalg.norm(got - y) / np.linalg.norm(y)))
+        done.append(name)
+    return dict(value=round(total_bytes / total_t / 1e9, 3), unit="GB/s", cores=nthreads, kind="port",
+                sample=f"C oracle dequantise-then-matmul (OpenMP, {nthreads} threads) over {'+'.join(done)} of the first "
+                       f"layer set, one pass, {total_t:.2f} s; same packed bytes as the GPU run",
+                gpu_vs_oracle_rel_fro=worst)
+
+
+def prefill_gemm(torch, F, ops, dev, reps=10):
+    """Prefill kernel at the Gemma-3-27B MLP shapes, M=2048, bf16 activations."""
+    M = 2048
+    rows = []
+    tot_flop, tot_ms = 0.0, 0.0
+    for name, K, N in (("gate", 21504, 5376), ("down", 5376, 21504)):
+        pm = F.synth_packed(K, N, F.BLK1632_4, seed=7, device=dev).to_tiled()
+        x = torch.randn(M, N, device=dev, generator=torch.Generator(device=dev).manual_seed(N)).to(torch.bfloat16)
+        for _ in range(2):
+            y = ops.gemm(pm, x)
+        torch.cuda.synchronize()
+        st = torch.cuda.current_stream()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(st)
+        for _ in range(reps):
+            y = ops.gemm(pm, x)
+        e1.record(st)
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        flop = 2.0 * M * K * N
+        tot_flop += flop * (2 if name == "gate" else 1)         # gate and up have the same shape
+        tot_ms += ms * (2 if name == "gate" else 1)
+        rows.append({"matrix": f"{name} {K}x{N}", "ms": round(ms, 4), "tflops": round(flop / ms / 1e9, 1)})
+        del pm, x, y
+    ach = tot_flop / tot_ms / 1e9
+    return {"workload": "gemma27b MLP (gate, up, down), M=2048, bf16 activations, BLK1632_4 3.1875 bpw, "
+                        "time includes the activation pre-scaling kernel",
+            "tflops": round(ach, 1), "per_matrix": rows,
+            "roofline": {"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(ach / MFMA_PEAK_TFLOPS, 4), "traffic": None}}
 
 
 def main():
@@ -65,10 +123,13 @@ def main():
     ap.add_argument("--bits", type=int, default=4)
     ap.add_argument("--keep", type=int, default=16)
     ap.add_argument("--group", type=int, default=128)
-    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host-core baseline")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM measurement")
     ap.add_argument("--launch", default="phase", choices=["matrix", "phase", "layer"],
                     help="GEMVs per launch: one matrix, one dependency phase (qkv | o | gate,up | down), or the layer set")
     ap.add_argument("--no-graph", action="store_true", help="launch from the host instead of replaying HIP graphs")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a 1 GiB device-to-device copy (reference reading for the HBM traffic counters)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -85,10 +146,14 @@ def main():
 
     set_bytes = sum(K * F.row_stride(layout, N, a.bits, a.group, a.keep) + K * (N // a.group) * 3 for _, K, N in shapes)
     n_copies = max(2, -(-2 * 256 * 2**20 // set_bytes))
-    sets = []
+    sets, first_rowmajor = [], None
     for c in range(n_copies):
-        sets.append([F.synth_packed(K, N, layout, a.bits, a.group, a.keep, seed=1000 * c + i, device=dev).to_tiled()
-                     for i, (_, K, N) in enumerate(shapes)])
+        rm = [F.synth_packed(K, N, layout, a.bits, a.group, a.keep, seed=1000 * c + i, device=dev)
+              for i, (_, K, N) in enumerate(shapes)]
+        if c == 0 and not a.no_cpu:
+            first_rowmajor = [p.to("cpu") for p in rm]
+        sets.append([p.to_tiled() for p in rm])
+        del rm
     xs = {N: torch.randn(M, N, device=dev, generator=torch.Generator(device=dev).manual_seed(N)).to(dt)
           for _, _, N in shapes}
     ys = [torch.empty(M, K, dtype=dt, device=dev) for _, K, _ in shapes]
@@ -121,15 +186,23 @@ def main():
             cs.append((n, descs, xp, ldx, yp, ldy, w.data_ptr(), w.numel()))
         calls.append(cs)
 
+    def launch(c):
+        n, descs, xp, ldx, yp, ldy, wp, wn = c
+        rc = L.cbk_gemv_batch(n, descs, xp, ldx, xdt, M, yp, ldy, xdt, None, wp, wn, sp)
+        if rc:
+            raise RuntimeError(L.cbk_strerror(rc).decode())
+
     def step(i):
-        for n, descs, xp, ldx, yp, ldy, wp, wn in calls[i % n_copies]:
-            rc = L.cbk_gemv_batch(n, descs, xp, ldx, xdt, M, yp, ldy, xdt, None, wp, wn, sp)
-            if rc:
-                raise RuntimeError(L.cbk_strerror(rc).decode())
+        for c in calls[i % n_copies]:
+            launch(c)
 
     launches = len(groups)
+    torch.cuda.synchronize()                                    # the weights were made on the default stream
     with torch.cuda.stream(stream):
-        for i in range(n_copies):
+        step(0)
+        stream.synchronize()
+        y_first = {name: y.clone() for (name, _, _), y in zip(shapes, ys)}   # outputs of layer set 0, for the parity check
+        for i in range(1, n_copies):
             step(i)
         stream.synchronize()
         graphs = None
@@ -150,34 +223,49 @@ def main():
             run(a.warmup + i)
         e1.record(stream)
         stream.synchronize()
-    ms = e0.elapsed_time(e1)
-    ms_per_step = ms / a.steps
+        ms_per_step = e0.elapsed_time(e1) / a.steps
+
+        if a.copy_calibration:
+            src = torch.empty(2**30, dtype=torch.uint8, device=dev)
+            dst = torch.empty_like(src)
+            for _ in range(3):
+                dst.copy_(src)
+            stream.synchronize()
+            del src, dst
+
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    # average launch of the decode kernel over the timed region (HIP events on the launch stream);
+    # it contains the gap between consecutive launches, so it is an upper bound of the kernel time
     us_per_launch = ms_per_step * 1e3 / launches
     bytes_per_launch = step_bytes / launches
     achieved = bytes_per_launch / (us_per_launch * 1e-6) / 1e9
     bpw = sets[0][0].bpw()
     out = {
-        "metric": "decode GEMV HBM GB/s at M=1 (packed CBK1 bytes streamed per second)" if M == 1
-                  else f"decode GEMV HBM GB/s at M={M}",
+        "metric": "decode GEMV HBM GB/s (% of 8 TB/s) at M=1; prefill GEMM TFLOP/s at M=2048",
         "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "i8xi8->i32 mfma, f32 scale" if False else ("f16" if a.dtype == "f16" else "bf16"),
+        "dtype": "i8 (int8 MFMA on integer codes and 3-digit block-fixed-point activations, f32 scales)",
         "data": "synthetic",
-        "config": {"workload": f"{a.workload} decode layer set, 7 GEMVs, M={M}, sparsity {1 - a.keep / 32:.4g}, "
-                               f"{a.bits}-bit, group {a.group}, layout {F.LAYOUT_NAME[layout]}, {bpw:.4f} bpw",
+        "config": {"workload": f"{a.workload} decode layer set, 7 GEMVs, M={M}, {a.dtype} activations, sparsity "
+                               f"{1 - a.keep / 32:.4g}, {a.bits}-bit, group {a.group}, layout {F.LAYOUT_NAME[layout]}, "
+                               f"{bpw:.4f} bpw",
                    "layer_set_bytes": step_bytes, "distinct_layer_sets": n_copies,
                    "launches_per_step": launches, "launch_grouping": a.launch,
-                   "hip_graph": not a.no_graph},
+                   "hip_graph": not a.no_graph, "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "decode GEMV", "avg_launch_us": round(us_per_launch, 3),
-                     "bytes_per_launch": int(bytes_per_launch)},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC.get((a.workload, a.launch, M)),
+                     "kernel": "cbk::gemv_mfma_kernel", "avg_launch_us": round(us_per_launch, 3),
+                     "launches_timed": a.steps * launches, "bytes_per_launch": int(bytes_per_launch)},
     }
+    del graphs, sets, calls, keep_alive
+    torch.cuda.empty_cache()
+    if not a.no_prefill:
+        out["prefill_gemm"] = prefill_gemm(torch, F, ops, dev)
     if not a.no_cpu:
-        from oracle import cbk_ref as R
-        out["cpu_baseline"] = cpu_baseline(shapes[0], layout if layout == F.BLK1632_4 else R.BLKC, a.bits, a.group,
-                                           a.keep, M)
+        out["cpu_baseline"] = cpu_baseline(first_rowmajor, shapes, xs, y_first, M)
+        # outputs are rounded to the activation dtype (2^-11 relative) on top of the kernel's own error
+        assert out["cpu_baseline"]["gpu_vs_oracle_rel_fro"] < 1e-3, "GPU outputs disagree with the oracle"
     print(json.dumps(out))
 
 
