@@ -22,14 +22,18 @@ class CobaltLinear(nn.Module):
         super().__init__()
         self.in_features, self.out_features = packed.N, packed.K
         self.register_buffer("blob", packed.blob)
-        o = packed.offs
-        self.register_buffer("cbk_meta", torch.tensor(
-            [packed.K, packed.N, packed.layout, packed.bits, packed.group, packed.keep, packed.cs_rows,
-             packed.cs_splits[0], packed.cs_splits[1], packed.data_bytes, o["data"], o.get("row_off", -1),
-             o["scale"], o["zero"], o.get("col_scale", -1), packed.n_survivors, packed.flags], dtype=torch.int64))
+        self.register_buffer("cbk_meta", self._meta_of(packed))
         self.bias = nn.Parameter(bias.detach().clone(), requires_grad=False) if bias is not None else None
         self.meta = dict(meta or {})
         self._backend = "hip"
+
+    @staticmethod
+    def _meta_of(packed: F.PackedMatrix) -> torch.Tensor:
+        o = packed.offs
+        return torch.tensor(
+            [packed.K, packed.N, packed.layout, packed.bits, packed.group, packed.keep, packed.cs_rows,
+             packed.cs_splits[0], packed.cs_splits[1], packed.data_bytes, o["data"], o.get("row_off", -1),
+             o["scale"], o["zero"], o.get("col_scale", -1), packed.n_survivors, packed.flags], dtype=torch.int64)
 
     # ---- construction ------------------------------------------------------------------
     @classmethod
@@ -96,6 +100,19 @@ class CobaltLinear(nn.Module):
         if self._pm_cache is None or self._pm_cache.blob.data_ptr() != self.blob.data_ptr():
             self._pm_cache = self.packed()
         return self._pm_cache
+
+    def to_device_order(self) -> "CobaltLinear":
+        """Reorder the packed image, once, into the 16-row tile-interleaved byte order the decode
+        kernel streams with fully coalesced loads (a permutation of the same bytes; fixed-stride
+        layouts only, a no-op otherwise).  Call it after the module is on its GPU."""
+        pm = self._pm()
+        if pm.tiled or "row_off" in pm.offs:
+            return self
+        t = pm.to_tiled()
+        self._buffers["blob"] = t.blob
+        self._buffers["cbk_meta"] = self._meta_of(t)
+        self._pm_cache = None
+        return self
 
     # ---- forward --------------------------------------------------------------------------
     def set_forward_backend(self, backend: str):

@@ -115,7 +115,9 @@ size_t cbk_row_stride(const cbk_desc* d);
  * (pack_cobalt.write_matrix :431-433 `stream_bytes`); SPARSE layouts need data_bytes. */
 size_t cbk_stream_bytes(const cbk_desc* d, size_t sparse_data_bytes);
 
-/* Device scratch needed by cbk_gemv / cbk_gemm / cbk_linear for M activation rows. */
+/* Device scratch needed by cbk_gemv / cbk_gemm / cbk_linear for M activation rows (0 for the
+ * decode kernels; the prefill kernel for M > 128 keeps its pre-scaled fp16 activations there:
+ * ceil(M/256)*256*N*2 bytes).  The workspace must be 256-byte aligned. */
 size_t cbk_workspace_bytes(const cbk_desc* d, int M);
 
 /* Rows [row0, row0+nrows) of W_hat -> out[nrows, ld_out] in out_dtype, bit-exact float32
@@ -133,7 +135,7 @@ int cbk_gemv(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
              void* y, int y_dtype, int64_t ldy, const void* bias,
              void* workspace, size_t workspace_bytes, void* stream);
 
-/* Several independent decode GEMVs in one launch pair (activation prep + decode): the matrices
+/* Several independent decode GEMVs in one kernel launch: the matrices
  * a decoder layer multiplies by the same hidden state (q, k, v; gate, up), or any other set
  * with no data dependence.  n <= 8.  Entry i computes ys[i] = xs[i] . W_hat_i^T (+ biases[i]).
  * Matrices that share (family, bits, group, keep) and qualify for the matrix-core kernel run
@@ -146,7 +148,8 @@ int cbk_gemv_batch(int n, const cbk_desc* descs, const void* const* xs, const in
                    int x_dtype, int M, void* const* ys, const int64_t* ldys, int y_dtype,
                    const void* const* biases, void* workspace, size_t workspace_bytes, void* stream);
 
-/* Prefill path, any M >= 1 (built for M >= 256).  Same contract as cbk_gemv.  Replaces the
+/* Prefill path, any M >= 1 (built for M >= 256).  Same contract as cbk_gemv; bf16 activations
+ * are carried as fp16 inside (magnitudes above 65504 saturate).  Replaces the
  * harness entry `gemm` (test_gemm.cu:151-165) and cbk::gemm_tile (cobalt_gemm.cuh:243-609). */
 int cbk_gemm(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
              void* y, int y_dtype, int64_t ldy, const void* bias,

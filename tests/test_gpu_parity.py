@@ -274,12 +274,16 @@ def test_cobalt_linear_forward_matches_reference_module_math():
     pk = R.pack_matrix(raw["mask"], raw["q"], raw["scale"], raw["zero"], R.BLK1632_4)
     W = R.dequant(pk, K, N, R.BLK1632_4, col_scale=raw["col_scale"])
     assert np.array_equal(_np(lin.dequantize()), W)
-    for shape in ((1, N), (3, 5, N), (2, 200, N)):
-        x = (torch.randn(*shape) * 1.0).half()
-        y = lin(x.to(DEV))
-        assert y.shape == shape[:-1] + (K,) and y.dtype == torch.float16
-        ref = R.forward_ref(W, _np(x).reshape(-1, N), bias=_np(bias)).reshape(y.shape)
-        assert rel_fro(_np(y), ref) < 6e-4
+    for tiled in (False, True):
+        if tiled:
+            lin.to_device_order()
+            assert lin.packed().tiled and np.array_equal(_np(lin.dequantize()), W)
+        for shape in ((1, N), (3, 5, N), (2, 200, N)):
+            x = (torch.randn(*shape) * 1.0).half()
+            y = lin(x.to(DEV))
+            assert y.shape == shape[:-1] + (K,) and y.dtype == torch.float16
+            ref = R.forward_ref(W, _np(x).reshape(-1, N), bias=_np(bias)).reshape(y.shape)
+            assert rel_fro(_np(y), ref) < 6e-4
 
 
 # ------------------------------------------------------------------ full-size properties
