@@ -174,58 +174,65 @@ __host__ __device__ constexpr int frag_col(int bits, bool dense, int bi) {
 // converts the activations it needs into its own LDS (a few hundred instructions per thread,
 // overlapped with the first weight loads).  One thread converts 16 columns at a time; the
 // eight threads of a chunk agree on its maximum with three lane exchanges.
-__device__ inline void stage_activations(const uint16_t* x, int64_t ldx, const uint16_t* cs, int xdt, int order,
-                                         int M, int N, int8_t* xq, float* delta, int tid) {
-  const int n16 = N >> 4, NCH = N >> 7, items = M * n16;          // a multiple of 8
-  for (int it = tid; it < items; it += GV_THREADS) {
-    const int row = it / n16, c16 = it - row * n16;
-    const uint16_t* xp = x + (size_t)row * ldx + c16 * 16;
-    const uint4 xr[2] = {((const uint4*)xp)[0], ((const uint4*)xp)[1]};
-    uint4 cr[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
-    if (cs) { cr[0] = ((const uint4*)(cs + c16 * 16))[0]; cr[1] = ((const uint4*)(cs + c16 * 16))[1]; }
-    const uint32_t* xw = (const uint32_t*)xr;
-    const uint32_t* cw = (const uint32_t*)cr;
-    float xv[16];
-    float mx = 0.f;
+struct XLoad { uint4 x[2], c[2]; };
+
+// global loads of staging item `it` (activation row it / (N/16), columns 16 * (it % (N/16)) ...)
+__device__ inline void stage_load(const uint16_t* x, int64_t ldx, const uint16_t* cs, int n16, int it, XLoad& r) {
+  const int row = it / n16, c16 = it - row * n16;
+  const uint16_t* xp = x + (size_t)row * ldx + c16 * 16;
+  r.x[0] = ((const uint4*)xp)[0]; r.x[1] = ((const uint4*)xp)[1];
+  r.c[0] = make_uint4(0, 0, 0, 0); r.c[1] = make_uint4(0, 0, 0, 0);
+  if (cs) { r.c[0] = ((const uint4*)(cs + c16 * 16))[0]; r.c[1] = ((const uint4*)(cs + c16 * 16))[1]; }
+}
+
+// conversion of one loaded item into digits and delta in LDS; the eight consecutive lanes of a
+// chunk are always active together (the item count is a multiple of 8)
+__device__ inline void stage_convert(const XLoad& r, bool has_cs, int xdt, int order, int N, int n16, int it,
+                                     int8_t* xq, float* delta) {
+  const int NCH = N >> 7;
+  const int row = it / n16, c16 = it - row * n16;
+  const uint32_t* xw = (const uint32_t*)r.x;
+  const uint32_t* cw = (const uint32_t*)r.c;
+  float xv[16];
+  float mx = 0.f;
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const uint16_t xb = (uint16_t)(xw[e >> 1] >> (16 * (e & 1)));
-      float v = xdt == CBK_F16 ? h2f(xb) : bf2f(xb);
-      if (cs) v *= h2f((uint16_t)(cw[e >> 1] >> (16 * (e & 1))));
-      xv[e] = v;
-      mx = fmaxf(mx, fabsf(v));
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 4, 64));
-    const float d = mx > 0.f ? mx / 8323072.f : 1.f;
-    const float inv = 1.f / d;
-    uint32_t dw[NDIG][4];
-#pragma unroll
-    for (int k = 0; k < NDIG; ++k)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) dw[k][q] = 0u;
-#pragma unroll
-    for (int bi = 0; bi < 16; ++bi) {
-      float v;
-      if (order == 0) v = xv[bi];
-      else if (order == 1) v = xv[frag_col(4, true, bi)];
-      else v = xv[frag_col(2, true, bi)];
-      int X = (int)rintf(v * inv);                       // |X| <= 127 * 65536
-      const int d0 = (int)(int8_t)(X & 0xFF);
-      X = (X - d0) >> 8;
-      const int d1 = (int)(int8_t)(X & 0xFF);
-      const int d2 = (X - d1) >> 8;
-      dw[0][bi >> 2] |= ((uint32_t)d2 & 0xFFu) << (8 * (bi & 3));
-      dw[1][bi >> 2] |= ((uint32_t)d1 & 0xFFu) << (8 * (bi & 3));
-      dw[2][bi >> 2] |= ((uint32_t)d0 & 0xFFu) << (8 * (bi & 3));
-    }
-#pragma unroll
-    for (int k = 0; k < NDIG; ++k)
-      *(uint4*)(xq + ((size_t)row * NDIG + k) * N + c16 * 16) = make_uint4(dw[k][0], dw[k][1], dw[k][2], dw[k][3]);
-    if ((c16 & 7) == 0) delta[row * (NCH + 4) + (c16 >> 3)] = d;
-    if (c16 < 4) delta[row * (NCH + 4) + NCH + c16] = 0.f;          // chunks past N
+  for (int e = 0; e < 16; ++e) {
+    const uint16_t xb = (uint16_t)(xw[e >> 1] >> (16 * (e & 1)));
+    float v = xdt == CBK_F16 ? h2f(xb) : bf2f(xb);
+    if (has_cs) v *= h2f((uint16_t)(cw[e >> 1] >> (16 * (e & 1))));
+    xv[e] = v;
+    mx = fmaxf(mx, fabsf(v));
   }
+  mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
+  mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
+  mx = fmaxf(mx, __shfl_xor(mx, 4, 64));
+  const float d = mx > 0.f ? mx / 8323072.f : 1.f;
+  const float inv = 1.f / d;
+  uint32_t dw[NDIG][4];
+#pragma unroll
+  for (int k = 0; k < NDIG; ++k)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) dw[k][q] = 0u;
+#pragma unroll
+  for (int bi = 0; bi < 16; ++bi) {
+    float v;
+    if (order == 0) v = xv[bi];
+    else if (order == 1) v = xv[frag_col(4, true, bi)];
+    else v = xv[frag_col(2, true, bi)];
+    int X = (int)rintf(v * inv);                       // |X| <= 127 * 65536
+    const int d0 = (int)(int8_t)(X & 0xFF);
+    X = (X - d0) >> 8;
+    const int d1 = (int)(int8_t)(X & 0xFF);
+    const int d2 = (X - d1) >> 8;
+    dw[0][bi >> 2] |= ((uint32_t)d2 & 0xFFu) << (8 * (bi & 3));
+    dw[1][bi >> 2] |= ((uint32_t)d1 & 0xFFu) << (8 * (bi & 3));
+    dw[2][bi >> 2] |= ((uint32_t)d0 & 0xFFu) << (8 * (bi & 3));
+  }
+#pragma unroll
+  for (int k = 0; k < NDIG; ++k)
+    *(uint4*)(xq + ((size_t)row * NDIG + k) * N + c16 * 16) = make_uint4(dw[k][0], dw[k][1], dw[k][2], dw[k][3]);
+  if ((c16 & 7) == 0) delta[row * (NCH + 4) + (c16 >> 3)] = d;
+  if (c16 < 4) delta[row * (NCH + 4) + NCH + c16] = 0.f;          // chunks past N
 }
 
 // ------------------------------------------------------------------ the decode kernel
@@ -331,12 +338,18 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     bool v0 = p0.tl < ntl;
     Pos p1 = p0; bool v1 = v0 && advance(p1);
     Pos p2 = p1; bool v2 = v1 && advance(p2);
+    // The activation loads go out before the first weight loads: the weight prefetch of a whole
+    // launch is tens of megabytes, and a request queued behind it would keep every wavefront
+    // from decoding until that burst has drained.
+    const int n16 = N >> 4, xitems = b.M * n16;                   // a multiple of 8
+    int xit = tid;
+    XLoad xl;
+    if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, xl);
     Loads<C> cur, nx1, nx2;                                       // two steps of loads stay in flight
     issue(t_lo + p0.tl, p0.S, cur);
-    issue(t_lo + p1.tl, p1.S, nx1);
 
     // ---- stage: selector table and counters (once), activation digits and deltas of this matrix
-    __syncthreads();                                              // previous matrix fully consumed
+    if (!first) __syncthreads();                                  // previous matrix fully consumed
     if (first) {
       if (tid < 256) {
         const uint2 e = make_selectors((uint32_t)tid, C::SEL_KIND);
@@ -349,7 +362,14 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       }
       first = false;
     }
-    stage_activations(gm.x, gm.ldx, m.cs, b.xdt, gm.order, b.M, N, xq, delta, tid);
+    while (xit < xitems) {
+      stage_convert(xl, m.cs != nullptr, b.xdt, gm.order, N, n16, xit, xq, delta);
+      xit += GV_THREADS;
+      if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, xl);
+    }
+    // the second step of loads goes out only now: issued together with the first, the two
+    // bursts of all wavefronts interleave in the memory system and every first step lands late
+    issue(t_lo + p1.tl, p1.S, nx1);
     __syncthreads();
 
     int bars = 0;                                                 // group barriers passed so far
