@@ -35,6 +35,20 @@ constexpr int GB_R = 256;       // weight rows per workgroup tile
 constexpr int GB_K = 64;        // input columns per stage
 constexpr int GB_P = GB_K + 8;  // LDS row pitch in halfs (144 B): conflict-free 16-byte reads
 constexpr int GB_LUT = 256 * 8 * 8;   // selector table, 8 lane-private copies of 256 x 8 B
+constexpr int GB_XBUF = GB_T * GB_K * 2;   // one activation stage in LDS: 256 rows x 128 B, unpadded, swizzled
+
+// One wavefront-wide copy of 64 x 16 bytes from global memory straight into LDS (no VGPRs, no
+// ds_write): lane l reads sbase + voff and its 16 bytes land at LDS byte lds + 16 * l.  The
+// compiler does not know that this instruction counts on vmcnt or that it writes LDS; the
+// kernel waits for it by hand before the barrier that publishes the stage.
+__device__ inline void dma_x16(const void* base, uint32_t voff, uint32_t lds) {
+  // base and lds are the same in every lane; say so, or they may arrive in vector registers
+  const uint64_t b64 = (uint64_t)base;
+  const uint64_t sbase = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b64) |
+                         ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b64 >> 32)) << 32);
+  lds = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds) : "memory");
+}
 
 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
 
@@ -51,14 +65,14 @@ __device__ inline uint2 gb_selectors(uint32_t mb) {
   return make_uint2(lo, hi);
 }
 
-// ---- X' = fp16(x * col_scale), [Mpad, N] row-major, rows M..Mpad-1 zero
+// ---- X' = fp16(x * col_scale), [Mpad, Npad] row-major; rows M..Mpad-1 and columns N..Npad-1 zero
 __global__ __launch_bounds__(256) void gemm_prep_kernel(const uint16_t* x, int64_t ldx, const uint16_t* cs, int xdt,
-                                                        int M, int Mpad, int N, uint16_t* out) {
+                                                        int M, int Mpad, int N, int Npad, uint16_t* out) {
   const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;     // one thread = 8 columns
-  const int n8 = N >> 3;
+  const int n8 = Npad >> 3;
   if (id >= (int64_t)Mpad * n8) return;
   const int row = (int)(id / n8), c8 = (int)(id % n8);
-  if (row >= M) { *(uint4*)(out + (size_t)row * N + c8 * 8) = make_uint4(0, 0, 0, 0); return; }
+  if (row >= M || c8 * 8 >= N) { *(uint4*)(out + (size_t)row * Npad + c8 * 8) = make_uint4(0, 0, 0, 0); return; }
   const uint4 v = *(const uint4*)(x + (size_t)row * ldx + c8 * 8);
   uint4 c = make_uint4(0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u);
   if (cs) c = *(const uint4*)(cs + c8 * 8);
@@ -73,13 +87,13 @@ __global__ __launch_bounds__(256) void gemm_prep_kernel(const uint16_t* x, int64
     a0 = fminf(fmaxf(a0, -65504.f), 65504.f); a1 = fminf(fmaxf(a1, -65504.f), 65504.f);
     o[e] = (uint32_t)f2h(a0) | ((uint32_t)f2h(a1) << 16);
   }
-  *(uint4*)(out + (size_t)row * N + c8 * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+  *(uint4*)(out + (size_t)row * Npad + c8 * 8) = make_uint4(o[0], o[1], o[2], o[3]);
 }
 
 struct GbArgs {
   DMat m;
-  const uint16_t* xp;      // X' fp16 [M, N]
-  int M;
+  const uint16_t* xp;      // X' fp16 [Mpad, Npad]
+  int M, Npad;
   void* y;
   int ydt;
   int64_t ldy;
@@ -105,11 +119,13 @@ __device__ inline uint4 bytes_to_halfs(uint32_t b0, uint32_t b1, h2_t s2) {
 }
 
 // FAST: 0 generic reader, 1 bitmap 16-of-32 4-bit, 2 dense 4-bit  (group 128 in both fast modes)
-template <int FAST>
+template <int FAST, int YDT>
 __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  _Float16* Xs = (_Float16*)smem;                                 // [2][GB_T][GB_P]
-  _Float16* Ws = Xs + 2 * GB_T * GB_P;                            // [2][GB_R][GB_P]
+  // Xs [2][GB_T][64 halfs]: row r, logical 16-byte piece c at physical piece c ^ ((r >> 1) & 7)
+  // (conflict-free 16-byte fragment reads without padding, which the direct copies cannot make)
+  _Float16* Xs = (_Float16*)smem;
+  _Float16* Ws = (_Float16*)(smem + 2 * GB_XBUF);                 // [2][GB_R][GB_P]
   uint2* lut = (uint2*)(Ws + 2 * GB_R * GB_P);                    // [256][8]
   const DMat& m = a.m;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -122,7 +138,9 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   if (lin >= nb) return;
   const int tt = lin / a.tiles_r, tr = lin % a.tiles_r;
   const int t0 = tt * GB_T, r0 = tr * GB_R;
-  const int N = m.N, nst = N / GB_K;
+  const int N = m.N, Npad = a.Npad;
+  const int nst = Npad / GB_K;                                    // a multiple of 4; stages past N see X' = 0
+  const int nch = N >> 7;                                         // 128-column chunks of the weight rows
 
   if (FAST == 1) {
     const uint2 e = gb_selectors((uint32_t)tid);
@@ -145,61 +163,74 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   const int wrc = wok ? wrow : m.K - 1;
   const RowView rv = row_view(m, wrc);
   const size_t meta0 = meta_index(m, wrc, 0), meta_step = m.tiled ? 16 : 1;
-  // activation rows this thread copies: 8 x 16 B per stage, rows tid/8 + 32 i (X' is padded
-  // to whole token tiles, so no bounds checks)
-  const uint16_t* xsrc = a.xp + (size_t)(t0 + (tid >> 3)) * N + (tid & 7) * 8;
-  const size_t xstep = (size_t)32 * N;
-  const uint32_t xdst = (uint32_t)((tid >> 3) * GB_P + (tid & 7) * 8);
-
-  uint4 xr0, xr1, xr2, xr3, xr4, xr5, xr6, xr7;                   // named: an array here ends up on the stack
-  struct WReg { uint32_t m[2]; uint32_t c[8]; uint32_t z; float s; };
-  WReg w0, w1;                                                    // stages of even / odd parity
-
-  auto load_x = [&](int s) {
-    const uint16_t* p = xsrc + s * GB_K;
-    xr0 = *(const uint4*)(p);             xr1 = *(const uint4*)(p + xstep);
-    xr2 = *(const uint4*)(p + 2 * xstep); xr3 = *(const uint4*)(p + 3 * xstep);
-    xr4 = *(const uint4*)(p + 4 * xstep); xr5 = *(const uint4*)(p + 5 * xstep);
-    xr6 = *(const uint4*)(p + 6 * xstep); xr7 = *(const uint4*)(p + 7 * xstep);
+  // Activation tile: wavefront w copies rows 64w .. 64w+63 of every stage with eight direct
+  // copies of eight rows each; lane l of copy q takes row 64w + 8q + l/8 and fills physical
+  // piece l%8 of it, i.e. fetches logical piece (l%8) ^ ((4q + l/16) & 7).  That is one of two
+  // values per lane (q even / odd), so two lane offsets and a scalar base per copy suffice.
+  const int wv = __builtin_amdgcn_readfirstlane(wave);
+  const uint32_t xvo_e = (uint32_t)((lane >> 3) * Npad * 2 + (((lane & 7) ^ (lane >> 4)) * 16));
+  const uint32_t xvo_o = (uint32_t)((lane >> 3) * Npad * 2 + (((lane & 7) ^ (4 + (lane >> 4))) * 16));
+  const uint8_t* xsb = (const uint8_t*)(a.xp + (size_t)(t0 + 64 * wv) * Npad);
+  const uint32_t xlds0 = (uint32_t)(uintptr_t)Xs + (uint32_t)wv * 8192u;
+  auto dma_x = [&](int s, int buf) {                              // stage s -> Xs[buf]
+    const uint8_t* sb = xsb + (size_t)s * (GB_K * 2);
+    const uint32_t ld = xlds0 + (uint32_t)buf * GB_XBUF;
+#pragma unroll
+    for (int q = 0; q < 8; ++q)
+      dma_x16(sb + (size_t)q * 8 * Npad * 2, (q & 1) ? xvo_o : xvo_e, ld + q * 1024);
   };
-  auto load_w = [&](int s, WReg& w) {
-    const int c0 = s * GB_K;
+  // fragment reads: this lane's row inside a 32-row block and its four swizzled piece offsets
+  const uint32_t xsw = ((lane & 31) >> 1) & 7;
+  uint32_t xpc[4];
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) xpc[kk] = (((2 * kk + (lane >> 5)) ^ xsw) * 16);
+
+  // one 128-column chunk of this thread's weight row: two stages' worth
+  struct WChunk { uint32_t m[4]; uint32_t c[FAST == 2 ? 16 : 8]; uint32_t z; float s; };
+  WChunk wA, wB;
+
+  auto load_chunk = [&](int c, WChunk& w) {
+    c = c < nch ? c : nch - 1;
     if (FAST == 1) {
-      // mask: 8 bytes at byte c0/8 of the row; codes: 16 bytes at code plane + c0/4
-      const uint32_t md = (uint32_t)c0 >> 5;
-      w.m[0] = rv.dword(md); w.m[1] = rv.dword(md + 1);
-      const uint4 v = *(const uint4*)rv.unit((m.code_off >> 4) + ((uint32_t)c0 >> 6));
-      w.c[0] = v.x; w.c[1] = v.y; w.c[2] = v.z; w.c[3] = v.w;
-    } else if (FAST == 2) {
-      const uint4 v0 = *(const uint4*)rv.unit((uint32_t)c0 >> 5), v1 = *(const uint4*)rv.unit(((uint32_t)c0 >> 5) + 1);
+      const uint4 mk = *(const uint4*)rv.unit((uint32_t)c);                         // 16 B of bitmap
+      w.m[0] = mk.x; w.m[1] = mk.y; w.m[2] = mk.z; w.m[3] = mk.w;
+      const uint32_t u = (m.code_off >> 4) + 2u * (uint32_t)c;                     // 32 B of survivor codes
+      const uint4 v0 = *(const uint4*)rv.unit(u), v1 = *(const uint4*)rv.unit(u + 1);
       w.c[0] = v0.x; w.c[1] = v0.y; w.c[2] = v0.z; w.c[3] = v0.w; w.c[4] = v1.x; w.c[5] = v1.y; w.c[6] = v1.z; w.c[7] = v1.w;
+    } else if (FAST == 2) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint4 v = *(const uint4*)rv.unit(4u * (uint32_t)c + i);              // 64 B of codes
+        w.c[4 * i] = v.x; w.c[4 * i + 1] = v.y; w.c[4 * i + 2] = v.z; w.c[4 * i + 3] = v.w;
+      }
     }
     if (FAST != 0) {
-      const size_t mi = meta0 + (size_t)(c0 >> 7) * meta_step;
+      const size_t mi = meta0 + (size_t)c * meta_step;
       w.z = m.zero[mi];
       w.s = h2f(m.scale[mi]);
     }
   };
 
-  // decode the staged weights of stage s into Ws[buf], quarter qq (16 columns) at a time
-  // selectors of the two mask bytes of quarter qq (bitmap layout only)
-  auto fetch_sel = [&](const WReg& w, int qq, uint2 (&sel)[2]) {
+  // selectors of the two mask bytes of quarter qq of half h of a chunk (bitmap layout only)
+  auto fetch_sel = [&](const WChunk& w, int h, int qq, uint2 (&sel)[2]) {
     if (FAST != 1) return;
 #pragma unroll
     for (int hb = 0; hb < 2; ++hb) {
-      const int jb8 = qq * 2 + hb;
-      const uint32_t mb = (w.m[jb8 >> 2] >> (8 * (jb8 & 3))) & 0xFFu;
+      const int jb = 8 * h + qq * 2 + hb;                          // mask byte of the chunk, 0..15
+      const uint32_t mb = (w.m[jb >> 2] >> (8 * (jb & 3))) & 0xFFu;
       sel[hb] = lut[mb * 8 + l8];
     }
   };
-  auto store_w_quarter = [&](int s, const WReg& w, int buf, int qq, const uint2 (&selq)[2]) {
+  // decode quarter qq (16 columns) of stage s = half h of chunk w into Ws[buf]
+  auto store_w_quarter = [&](int s, const WChunk& w, int h, int buf, int qq, const uint2 (&selq)[2]) {
     _Float16* dst = Ws + (size_t)buf * GB_R * GB_P + tid * GB_P + qq * 16;
     if (FAST == 0) {
       if (qq & 1) return;                                         // the generic reader works on 32 columns
       uint32_t packed[16];
       if (wok) {
         int q[32];
-        const int t = (s * GB_K >> 5) + (qq >> 1);
+        int t = (s * GB_K >> 5) + (qq >> 1);
+        t = t < (N >> 5) ? t : (N >> 5) - 1;
         const uint32_t keep = decode_block32(m, rv, t, q);
         const int g = (t * BLOCK) / m.group;
         const float sc = h2f(m.scale[meta_index(m, wrc, g)]);
@@ -228,17 +259,18 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
       const int jb8 = qq * 2 + hb;                                // mask byte of the stage, 0..7
       uint32_t b0, b1;
       if (FAST == 1) {
-        const uint32_t mw = w.m[jb8 >> 2];
+        const int blk = 2 * h + (jb8 >> 2);                       // 32-column block of the chunk
+        const uint32_t mw = w.m[blk];
         const int jj = jb8 & 3;
         const uint32_t r = jj == 0 ? 0u : (uint32_t)__builtin_popcount(mw & ((1u << (8 * jj)) - 1u));
-        const uint64_t st = ((uint64_t)w.c[2 * (jb8 >> 2) + 1] << 32) | w.c[2 * (jb8 >> 2)];
+        const uint64_t st = ((uint64_t)w.c[2 * blk + 1] << 32) | w.c[2 * blk];
         const uint32_t cw = (uint32_t)(st >> ((r * 4u) & 63u));
         const uint32_t p0 = ((cw & 0x0F0F0F0Fu) + nz) ^ 0x80808080u;
         const uint32_t p1 = (((cw >> 4) & 0x0F0F0F0Fu) + nz) ^ 0x80808080u;
         b0 = __builtin_amdgcn_perm(p1, p0, selq[hb].x);
         b1 = __builtin_amdgcn_perm(p1, p0, selq[hb].y);
       } else {
-        const uint32_t cw = w.c[jb8];
+        const uint32_t cw = w.c[8 * h + jb8];
         const uint32_t p0 = ((cw & 0x0F0F0F0Fu) + nz) ^ 0x80808080u;          // even columns
         const uint32_t p1 = (((cw >> 4) & 0x0F0F0F0Fu) + nz) ^ 0x80808080u;   // odd columns
         b0 = __builtin_amdgcn_perm(p1, p0, 0x05010400u);
@@ -247,73 +279,55 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
       ((uint4*)dst)[hb] = bytes_to_halfs(b0, b1, s2);
     }
   };
-  auto store_x = [&](int buf) {
-    _Float16* base = Xs + (size_t)buf * GB_T * GB_P + xdst;
-    *(uint4*)(base) = xr0;                 *(uint4*)(base + 32 * GB_P) = xr1;
-    *(uint4*)(base + 64 * GB_P) = xr2;     *(uint4*)(base + 96 * GB_P) = xr3;
-    *(uint4*)(base + 128 * GB_P) = xr4;    *(uint4*)(base + 160 * GB_P) = xr5;
-    *(uint4*)(base + 192 * GB_P) = xr6;    *(uint4*)(base + 224 * GB_P) = xr7;
-  };
-
-  // ---- prologue: stage 0 into buffer 0; stage 1 into registers (X in xr, W in w1)
-  load_x(0); load_w(0, w0);
+  // ---- prologue: chunks 0 and 1 into registers; stage 0 into buffer 0
+  dma_x(0, 0);
+  load_chunk(0, wA); load_chunk(1, wB);
   __syncthreads();                                                // selector table visible
-  store_x(0);
 #pragma unroll
   for (int qq = 0; qq < 4; ++qq) {
     uint2 sel[2];
-    fetch_sel(w0, qq, sel);
-    store_w_quarter(0, w0, 0, qq, sel);
+    fetch_sel(wA, 0, qq, sel);
+    store_w_quarter(0, wA, 0, 0, qq, sel);
   }
-  load_w(1, w1); load_x(1);
   uint2 selq[2];                                                  // selectors of the next quarter to decode
-  fetch_sel(w1, 0, selq);
+  fetch_sel(wA, 1, 0, selq);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
-  // One stage: matrix-core work on buffer s % 2.  With MORE, the registers holding stage
-  // s + 1 are written to the other buffer (X as is, W decoded a quarter at a time between the
-  // MFMAs) and stage s + 2 (clamped to the last) is fetched into the registers just freed,
-  // so every global load has a whole stage in which to land.  wd: registers of stage s + 1,
-  // wl: registers that receive stage s + 2.  No branches inside.
-  auto stage = [&](int s, auto more_tag, const WReg& wd, WReg& wl) {
-    constexpr bool MORE = decltype(more_tag)::value;
+  // One stage: matrix-core work on buffer s % 2 while stage s + 1 moves into the other buffer:
+  // its activations by direct copies issued at the top, its weights (half HD of chunk wd)
+  // decoded a quarter per phase between the MFMAs.  The selectors of the following quarter
+  // (after the last one: of quarter 0 of half HN of chunk wn) are fetched a phase early.  With
+  // LOADW the 128-column weight chunk `cl` is loaded into wl, first touched seven phases later;
+  // these loads are issued after the direct copies, so the wait before the barrier can leave
+  // them in flight.  No branches inside.
+  constexpr int NWL = FAST == 1 ? 5 : FAST == 2 ? 6 : 0;          // vector loads of one load_chunk
+  auto stage = [&](int s, auto loadw_tag, const WChunk& wd, auto hd_tag, const WChunk& wn, auto hn_tag, WChunk& wl, int cl) {
+    constexpr bool LOADW = decltype(loadw_tag)::value;
+    constexpr int HD = decltype(hd_tag)::value, HN = decltype(hn_tag)::value;
     const int buf = s & 1;
-    const _Float16* xb = Xs + (size_t)buf * GB_T * GB_P + (128 * wt + (lane & 31)) * GB_P + 8 * (lane >> 5);
+    const uint8_t* xb = (const uint8_t*)Xs + (size_t)buf * GB_XBUF + (128 * wt + (lane & 31)) * 128;
     const _Float16* wb = Ws + (size_t)buf * GB_R * GB_P + (128 * wr + (lane & 31)) * GB_P + 8 * (lane >> 5);
     v8h af[2][4], bf[2][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) af[0][i] = *(const v8h*)(xb + 32 * i * GB_P);
+    for (int i = 0; i < 4; ++i) af[0][i] = *(const v8h*)(xb + 4096 * i + xpc[0]);
 #pragma unroll
     for (int j = 0; j < 4; ++j) bf[0][j] = *(const v8h*)(wb + 32 * j * GB_P);
-    // the X registers of stage s + 1 go to LDS two per phase; the loads of stage s + 2 below
-    // land in fresh registers (the old ones stay live until their store)
-    const uint4 xo0 = xr0, xo1 = xr1, xo2 = xr2, xo3 = xr3, xo4 = xr4, xo5 = xr5, xo6 = xr6, xo7 = xr7;
-    _Float16* xw = Xs + (size_t)(buf ^ 1) * GB_T * GB_P + xdst;
-    if (MORE) {
-      const int s2 = s + 2 < nst ? s + 2 : nst - 1;
-      load_w(s2, wl);                                             // first: its data is wanted first
-      load_x(s2);
-    }
+    dma_x(s + 1 < nst ? s + 1 : nst - 1, buf ^ 1);
+    if (LOADW) load_chunk(cl, wl);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int kk = 0; kk < GB_K / 16; ++kk) {
       const int c = kk & 1, n = c ^ 1;
       if (kk + 1 < GB_K / 16) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) af[n][i] = *(const v8h*)(xb + 32 * i * GB_P + 16 * (kk + 1));
+        for (int i = 0; i < 4; ++i) af[n][i] = *(const v8h*)(xb + 4096 * i + xpc[kk + 1 < 4 ? kk + 1 : 3]);
 #pragma unroll
         for (int j = 0; j < 4; ++j) bf[n][j] = *(const v8h*)(wb + 32 * j * GB_P + 16 * (kk + 1));
       }
-      // selectors one quarter ahead, so that their LDS latency is never waited for
       uint2 seln[2];
-      if (kk + 1 < GB_K / 16) fetch_sel(wd, kk + 1, seln); else fetch_sel(wl, 0, seln);
-      if (MORE) {
-        if (kk == 0) { *(uint4*)(xw) = xo0;              *(uint4*)(xw + 32 * GB_P) = xo1; }
-        if (kk == 1) { *(uint4*)(xw + 64 * GB_P) = xo2;  *(uint4*)(xw + 96 * GB_P) = xo3; }
-        if (kk == 2) { *(uint4*)(xw + 128 * GB_P) = xo4; *(uint4*)(xw + 160 * GB_P) = xo5; }
-        if (kk == 3) { *(uint4*)(xw + 192 * GB_P) = xo6; *(uint4*)(xw + 224 * GB_P) = xo7; }
-        store_w_quarter(s + 1, wd, buf ^ 1, kk, selq);
-      }
+      if (kk + 1 < GB_K / 16) fetch_sel(wd, HD, kk + 1, seln); else fetch_sel(wn, HN, 0, seln);
+      store_w_quarter(s + 1, wd, HD, buf ^ 1, kk, selq);
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -327,48 +341,91 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
       }
       __builtin_amdgcn_sched_barrier(0);
     }
+    // the direct copies of stage s + 1 must have landed before the barrier publishes them
+    if (LOADW && NWL == 5) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+    else if (LOADW && NWL == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   };
-  // N is a multiple of 128, so the number of stages is even.  The last stage also decodes
-  // (the clamped, already consumed) registers into the idle buffer: one loop body, no tail.
-  for (int s = 0; s < nst; s += 2) {
-    stage(s, std::true_type{}, w1, w0);
-    stage(s + 1, std::true_type{}, w0, w1);
+  // Four stages per trip (two chunks): stage 2p decodes the upper half of chunk p, stage 2p+1
+  // the lower half of chunk p+1 and loads chunk p+2 into the registers chunk p has left.
+  using T = std::true_type; using Fl = std::false_type;
+  using H0 = std::integral_constant<int, 0>; using H1 = std::integral_constant<int, 1>;
+  for (int s = 0; s < nst; s += 4) {
+    const int p = s >> 1;
+    stage(s,     Fl{}, wA, H1{}, wB, H0{}, wA, 0);
+    stage(s + 1, T{},  wB, H0{}, wB, H1{}, wA, p + 2);
+    stage(s + 2, Fl{}, wB, H1{}, wA, H0{}, wB, 0);
+    stage(s + 3, T{},  wA, H0{}, wA, H1{}, wB, p + 3);
   }
 
-  // ---- epilogue: D[i][j] with j = lane%32 (weight row), i = 8*(r/4) + 4*(lane/32) + r%4 (token)
+  // ---- epilogue.  D[i][j] holds, in lane l and register r, token 8*(r/4) + 4*(l/32) + r%4 and
+  // weight row l%32 of its 32 x 32 block.  Each wavefront turns its 128 x 128 sub-tile around
+  // through LDS (the operand buffers are free now), 32 tokens at a time, so that global stores
+  // are whole 16-byte pieces of consecutive output columns: 256 B (f16) or 512 B (f32) per token.
+  // Everything is compile-time indexed and branch-free per element: the 256 accumulators make
+  // this straight-line code, and it has to stay small enough for the instruction cache.
+  {
+    constexpr int ESZ = YDT == CBK_F32 ? 4 : 2;
+    constexpr int PITCH = 128 * ESZ + 16;                          // bytes per token row in LDS
+    constexpr int EPP = 16 / ESZ, PPR = 128 / EPP;                 // elements per 16-byte piece, pieces per row
+    uint8_t* ep = smem + (size_t)wave * (32 * (128 * 4 + 16));
+    uint8_t* epl = ep + 4 * (lane >> 5) * PITCH + (lane & 31) * ESZ;
+    float bv[4];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int k = r0 + 128 * wr + 32 * j + (lane & 31);
-    if (k >= m.K) continue;
-    float bv = 0.f;
-    if (a.bias) bv = (a.ydt == CBK_F32) ? ((const float*)a.bias)[k]
-                   : (a.ydt == CBK_F16) ? h2f(((const uint16_t*)a.bias)[k]) : bf2f(((const uint16_t*)a.bias)[k]);
+    for (int j = 0; j < 4; ++j) {
+      const int k = r0 + 128 * wr + 32 * j + (lane & 31);
+      bv[j] = 0.f;
+      if (a.bias && k < m.K) bv[j] = load_act<YDT>(a.bias, k);
+    }
+    const bool vec_ok = ((a.ldy * ESZ) & 15) == 0 && (((uintptr_t)a.y) & 15) == 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 4; ++i) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int tok = t0 + 128 * wt + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (tok >= a.M) continue;
-        const float v = acc[i][j][r] + bv;
-        const size_t o = (size_t)tok * a.ldy + k;
-        if (a.ydt == CBK_F32) ((float*)a.y)[o] = v;
-        else if (a.ydt == CBK_F16) ((uint16_t*)a.y)[o] = f2h(v);
-        else ((uint16_t*)a.y)[o] = f2bf(v);
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float v = acc[i][j][r] + bv[j];
+          uint8_t* d = epl + (8 * (r >> 2) + (r & 3)) * PITCH + 32 * j * ESZ;
+          if (YDT == CBK_F32) *(float*)d = v;
+          else if (YDT == CBK_F16) *(uint16_t*)d = f2h(v);
+          else {
+            const uint32_t u = __float_as_uint(v);
+            const uint32_t rn = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+            *(uint16_t*)d = (uint16_t)(((u & 0x7fffffffu) > 0x7f800000u) ? ((u >> 16) | 0x40u) : rn);
+          }
+        }
+#pragma unroll
+      for (int t = 0; t < 32 * PPR / 64; ++t) {
+        const int pc = t * 64 + lane;
+        const int row = pc / PPR, c = pc % PPR;
+        const int tok = t0 + 128 * wt + 32 * i + row, k = r0 + 128 * wr + c * EPP;
+        if (tok >= a.M || k >= m.K) continue;
+        const uint8_t* src = ep + row * PITCH + c * 16;
+        uint8_t* dst = (uint8_t*)a.y + ((size_t)tok * a.ldy + k) * ESZ;
+        if (vec_ok && k + EPP <= m.K) *(uint4*)dst = *(const uint4*)src;
+        else
+          for (int e = 0; e < EPP && k + e < m.K; ++e) {
+            if (ESZ == 4) ((float*)dst)[e] = ((const float*)src)[e];
+            else ((uint16_t*)dst)[e] = ((const uint16_t*)src)[e];
+          }
       }
+    }
   }
 }
+
+static inline int gb_npad(int N) { return (N + 255) / 256 * 256; }
 
 size_t gemm_big_workspace(const DMat& m, int M) {
   const size_t mpad = (size_t)(M + GB_T - 1) / GB_T * GB_T;
-  return (mpad * m.N * 2 + 255) & ~(size_t)255;
+  return (mpad * gb_npad(m.N) * 2 + 255) & ~(size_t)255;
 }
 
-template <int FAST>
-static int launch_big(const GbArgs& a, int blocks, hipStream_t st) {
-  auto kern = gemm_big_kernel<FAST>;
+template <int FAST, int YDT>
+static int launch_big_y(const GbArgs& a, int blocks, hipStream_t st) {
+  auto kern = gemm_big_kernel<FAST, YDT>;
   static std::atomic<int> configured{0};
-  const size_t lds = (size_t)2 * (GB_T + GB_R) * GB_P * 2 + GB_LUT;
+  const size_t lds = (size_t)2 * GB_XBUF + (size_t)2 * GB_R * GB_P * 2 + GB_LUT;
   if (!configured.load(std::memory_order_acquire)) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
       return CBK_ERR_HIP;
@@ -378,6 +435,14 @@ static int launch_big(const GbArgs& a, int blocks, hipStream_t st) {
   return hipGetLastError() == hipSuccess ? CBK_OK : CBK_ERR_HIP;
 }
 
+template <int FAST>
+static int launch_big(const GbArgs& a, int blocks, hipStream_t st) {
+  if (a.ydt == CBK_F32) return launch_big_y<FAST, CBK_F32>(a, blocks, st);
+  if (a.ydt == CBK_F16) return launch_big_y<FAST, CBK_F16>(a, blocks, st);
+  if (a.ydt == CBK_BF16T) return launch_big_y<FAST, CBK_BF16T>(a, blocks, st);
+  return CBK_ERR_DTYPE;
+}
+
 int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
                     const void* bias, void* ws, size_t ws_bytes, hipStream_t st) {
   if (family_of(m.layout) == FAM_SPARSE) return CBK_ERR_UNSUPPORTED;
@@ -385,11 +450,12 @@ int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, v
   if (!ws || ws_bytes < gemm_big_workspace(m, M)) return CBK_ERR_WORKSPACE;
   if ((uintptr_t)ws & 255) return CBK_ERR_ALIGN;
   const int Mpad = (M + GB_T - 1) / GB_T * GB_T;
-  const int64_t items = (int64_t)Mpad * (m.N / 8);
+  const int Npad = gb_npad(m.N);
+  const int64_t items = (int64_t)Mpad * (Npad / 8);
   hipLaunchKernelGGL(gemm_prep_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st,
-                     (const uint16_t*)x, ldx, m.cs, xdt, M, Mpad, m.N, (uint16_t*)ws);
+                     (const uint16_t*)x, ldx, m.cs, xdt, M, Mpad, m.N, Npad, (uint16_t*)ws);
   GbArgs a;
-  a.m = m; a.xp = (const uint16_t*)ws; a.M = M; a.y = y; a.ydt = ydt; a.ldy = ldy; a.bias = bias;
+  a.m = m; a.xp = (const uint16_t*)ws; a.M = M; a.Npad = Npad; a.y = y; a.ydt = ydt; a.ldy = ldy; a.bias = bias;
   a.tiles_t = (M + GB_T - 1) / GB_T; a.tiles_r = (m.K + GB_R - 1) / GB_R;
   const int nb = a.tiles_t * a.tiles_r;
   const int blocks = ((nb + 7) / 8) * 8;
