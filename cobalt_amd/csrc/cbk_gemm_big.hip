@@ -1,69 +1,13 @@
-// Prefill GEMM for M > 128:  Y[M, K] = X[M, N] . W_hat[K, N]^T on the gfx950 matrix cores.
-//
-// Workgroup tile 256 tokens x 256 weight rows, 64 input columns per stage, four wavefronts
-// each owning a 128 x 128 sub-tile (4 x 4 blocks of v_mfma_f32_32x32x16_f16, 256 accumulator
-// registers), one wavefront per SIMD.  Both operands are double-buffered in LDS (147 KB):
-// while the matrix cores work on stage s, the same wavefronts dequantise the weights of
-// stage s + 1 into the other buffer and copy the activation tile there.
-//
-// Operands.  The activation side is X' = fp16(x * col_scale), written once per call into the
-// caller's workspace by a small elementwise kernel (bf16 inputs are widened exactly; the
-// product is rounded once to fp16, magnitudes above 65504 saturate).  The weight side is
-// fp16((q - zero) * scale) for a kept column and exactly 0 for a pruned one, so
-// Y = sum_j X'[m,j] * W'[k,j] carries two roundings of relative size 2^-12.  Feeding bf16
-// operands instead would round to 2^-9, which alone exceeds the 1e-3 relative-Frobenius
-// budget of this layer; the f16 and bf16 MFMA rates are identical.
-//
-// Weight decode.  Each of the 256 threads owns one weight row of the tile and decodes its
-// 64 columns of the stage.  For 4-bit codes with 16 of 32 kept, and for the dense 4-bit
-// layout, this is the byte-permute decoder of the decode kernel (selector table in LDS)
-// followed by two packed-half operations per column pair; other configurations go through
-// the generic 32-column reader.
-//
-// Workgroups are ordered so that those running at the same time on one XCD (blockIdx % 8)
-// share their token tile, which then stays in that XCD's L2.
-//
-// Reference semantics: cbk::gemm_tile (src/cobaltkernel/csrc/cobalt_gemm.cuh:243-609).
-#include <atomic>
-#include <type_traits>
-#include "cbk_device.h"
+// Prefill GEMM for M > 128: activation pre-scaling kernel, the generic-reader instantiation
+// and the dispatch over the per-code-width instantiations (cbk_gemm_big_b2/3/4.hip).  The
+// kernel itself is in cbk_gemm_big.h.
+#include "cbk_gemm_big.h"
 
 namespace cbk {
 
-constexpr int GB_T = 256;       // tokens per workgroup tile
-constexpr int GB_R = 256;       // weight rows per workgroup tile
-constexpr int GB_K = 64;        // input columns per stage
-constexpr int GB_P = GB_K + 8;  // LDS row pitch in halfs (144 B): conflict-free 16-byte reads
-constexpr int GB_LUT = 256 * 8 * 8;   // selector table, 8 lane-private copies of 256 x 8 B
-constexpr int GB_XBUF = GB_T * GB_K * 2;   // one activation stage in LDS: 256 rows x 128 B, unpadded, swizzled
-
-// One wavefront-wide copy of 64 x 16 bytes from global memory straight into LDS (no VGPRs, no
-// ds_write): lane l reads sbase + voff and its 16 bytes land at LDS byte lds + 16 * l.  The
-// compiler does not know that this instruction counts on vmcnt or that it writes LDS; the
-// kernel waits for it by hand before the barrier that publishes the stage.
-__device__ inline void dma_x16(const void* base, uint32_t voff, uint32_t lds) {
-  // base and lds are the same in every lane; say so, or they may arrive in vector registers
-  const uint64_t b64 = (uint64_t)base;
-  const uint64_t sbase = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b64) |
-                         ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b64 >> 32)) << 32);
-  lds = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds);
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds) : "memory");
-}
-
-typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
-
-__device__ inline uint2 gb_selectors(uint32_t mb) {
-  uint32_t lo = 0, hi = 0, r = 0;
-#pragma unroll
-  for (int p = 0; p < 8; ++p) {
-    const uint32_t idx = (r >> 1) + 4u * (r & 1u);
-    const bool kp = (mb >> p) & 1u;
-    const uint32_t sel = kp ? idx : 0x0Cu;
-    if (p < 4) lo |= sel << (8 * p); else hi |= sel << (8 * (p - 4));
-    r += kp ? 1u : 0u;
-  }
-  return make_uint2(lo, hi);
-}
+int launch_gemm_big_b2(const GbArgs&, int keep, int group, int blocks, hipStream_t);
+int launch_gemm_big_b3(const GbArgs&, int keep, int group, int blocks, hipStream_t);
+int launch_gemm_big_b4(const GbArgs&, int keep, int group, int blocks, hipStream_t);
 
 // ---- X' = fp16(x * col_scale), [Mpad, Npad] row-major; rows M..Mpad-1 and columns N..Npad-1 zero
 __global__ __launch_bounds__(256) void gemm_prep_kernel(const uint16_t* x, int64_t ldx, const uint16_t* cs, int xdt,
@@ -90,330 +34,6 @@ __global__ __launch_bounds__(256) void gemm_prep_kernel(const uint16_t* x, int64
   *(uint4*)(out + (size_t)row * Npad + c8 * 8) = make_uint4(o[0], o[1], o[2], o[3]);
 }
 
-struct GbArgs {
-  DMat m;
-  const uint16_t* xp;      // X' fp16 [Mpad, Npad]
-  int M, Npad;
-  void* y;
-  int ydt;
-  int64_t ldy;
-  const void* bias;
-  int tiles_t, tiles_r;
-};
-
-// eight signed bytes (q - z for a kept column, 0 for a pruned one) -> eight halfs times scale
-__device__ inline uint4 bytes_to_halfs(uint32_t b0, uint32_t b1, h2_t s2) {
-  // byte b (two's complement) -> u = b ^ 0x80 = b + 128 -> half bits 0x6400 | u = 1024 + 128 + b
-  const uint32_t u0 = b0 ^ 0x80808080u, u1 = b1 ^ 0x80808080u;
-  const uint32_t k = 0x64646464u;
-  uint32_t w[4] = {__builtin_amdgcn_perm(k, u0, 0x04010400u), __builtin_amdgcn_perm(k, u0, 0x04030402u),
-                   __builtin_amdgcn_perm(k, u1, 0x04010400u), __builtin_amdgcn_perm(k, u1, 0x04030402u)};
-  const h2_t off = {(_Float16)-1152.0f, (_Float16)-1152.0f};
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    h2_t v = __builtin_bit_cast(h2_t, w[i]);
-    v = (v + off) * s2;
-    w[i] = __builtin_bit_cast(uint32_t, v);
-  }
-  return make_uint4(w[0], w[1], w[2], w[3]);
-}
-
-// FAST: 0 generic reader, 1 bitmap 16-of-32 4-bit, 2 dense 4-bit  (group 128 in both fast modes)
-template <int FAST, int YDT>
-__global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
-  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  // Xs [2][GB_T][64 halfs]: row r, logical 16-byte piece c at physical piece c ^ ((r >> 1) & 7)
-  // (conflict-free 16-byte fragment reads without padding, which the direct copies cannot make)
-  _Float16* Xs = (_Float16*)smem;
-  _Float16* Ws = (_Float16*)(smem + 2 * GB_XBUF);                 // [2][GB_R][GB_P]
-  uint2* lut = (uint2*)(Ws + 2 * GB_R * GB_P);                    // [256][8]
-  const DMat& m = a.m;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wt = wave >> 1, wr = wave & 1;
-  // XCD-aware order: blockIdx % 8 picks the XCD; give each XCD whole token tiles
-  const int nb = a.tiles_t * a.tiles_r;
-  const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-  const int per = (nb + 7) >> 3;
-  const int lin = xcd * per + idx;                                 // token-tile-major linear id
-  if (lin >= nb) return;
-  const int tt = lin / a.tiles_r, tr = lin % a.tiles_r;
-  const int t0 = tt * GB_T, r0 = tr * GB_R;
-  const int N = m.N, Npad = a.Npad;
-  const int nst = Npad / GB_K;                                    // a multiple of 4; stages past N see X' = 0
-  const int nch = N >> 7;                                         // 128-column chunks of the weight rows
-
-  if (FAST == 1) {
-    const uint2 e = gb_selectors((uint32_t)tid);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) lut[tid * 8 + j] = e;
-  }
-  const uint32_t l8 = lane & 7;
-
-  v16f acc[4][4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-
-  // this thread's weight row
-  const int wrow = r0 + tid;
-  const bool wok = wrow < m.K;
-  const int wrc = wok ? wrow : m.K - 1;
-  const RowView rv = row_view(m, wrc);
-  const size_t meta0 = meta_index(m, wrc, 0), meta_step = m.tiled ? 16 : 1;
-  // Activation tile: wavefront w copies rows 64w .. 64w+63 of every stage with eight direct
-  // copies of eight rows each; lane l of copy q takes row 64w + 8q + l/8 and fills physical
-  // piece l%8 of it, i.e. fetches logical piece (l%8) ^ ((4q + l/16) & 7).  That is one of two
-  // values per lane (q even / odd), so two lane offsets and a scalar base per copy suffice.
-  const int wv = __builtin_amdgcn_readfirstlane(wave);
-  const uint32_t xvo_e = (uint32_t)((lane >> 3) * Npad * 2 + (((lane & 7) ^ (lane >> 4)) * 16));
-  const uint32_t xvo_o = (uint32_t)((lane >> 3) * Npad * 2 + (((lane & 7) ^ (4 + (lane >> 4))) * 16));
-  const uint8_t* xsb = (const uint8_t*)(a.xp + (size_t)(t0 + 64 * wv) * Npad);
-  const uint32_t xlds0 = (uint32_t)(uintptr_t)Xs + (uint32_t)wv * 8192u;
-  auto dma_x = [&](int s, int buf) {                              // stage s -> Xs[buf]
-    const uint8_t* sb = xsb + (size_t)s * (GB_K * 2);
-    const uint32_t ld = xlds0 + (uint32_t)buf * GB_XBUF;
-#pragma unroll
-    for (int q = 0; q < 8; ++q)
-      dma_x16(sb + (size_t)q * 8 * Npad * 2, (q & 1) ? xvo_o : xvo_e, ld + q * 1024);
-  };
-  // fragment reads: this lane's row inside a 32-row block and its four swizzled piece offsets
-  const uint32_t xsw = ((lane & 31) >> 1) & 7;
-  uint32_t xpc[4];
-#pragma unroll
-  for (int kk = 0; kk < 4; ++kk) xpc[kk] = (((2 * kk + (lane >> 5)) ^ xsw) * 16);
-
-  // one 128-column chunk of this thread's weight row: two stages' worth
-  struct WChunk { uint32_t m[4]; uint32_t c[FAST == 2 ? 16 : 8]; uint32_t z; float s; };
-  WChunk wA, wB;
-
-  auto load_chunk = [&](int c, WChunk& w) {
-    c = c < nch ? c : nch - 1;
-    if (FAST == 1) {
-      const uint4 mk = *(const uint4*)rv.unit((uint32_t)c);                         // 16 B of bitmap
-      w.m[0] = mk.x; w.m[1] = mk.y; w.m[2] = mk.z; w.m[3] = mk.w;
-      const uint32_t u = (m.code_off >> 4) + 2u * (uint32_t)c;                     // 32 B of survivor codes
-      const uint4 v0 = *(const uint4*)rv.unit(u), v1 = *(const uint4*)rv.unit(u + 1);
-      w.c[0] = v0.x; w.c[1] = v0.y; w.c[2] = v0.z; w.c[3] = v0.w; w.c[4] = v1.x; w.c[5] = v1.y; w.c[6] = v1.z; w.c[7] = v1.w;
-    } else if (FAST == 2) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const uint4 v = *(const uint4*)rv.unit(4u * (uint32_t)c + i);              // 64 B of codes
-        w.c[4 * i] = v.x; w.c[4 * i + 1] = v.y; w.c[4 * i + 2] = v.z; w.c[4 * i + 3] = v.w;
-      }
-    }
-    if (FAST != 0) {
-      const size_t mi = meta0 + (size_t)c * meta_step;
-      w.z = m.zero[mi];
-      w.s = h2f(m.scale[mi]);
-    }
-  };
-
-  // selectors of the two mask bytes of quarter qq of half h of a chunk (bitmap layout only)
-  auto fetch_sel = [&](const WChunk& w, int h, int qq, uint2 (&sel)[2]) {
-    if (FAST != 1) return;
-#pragma unroll
-    for (int hb = 0; hb < 2; ++hb) {
-      const int jb = 8 * h + qq * 2 + hb;                          // mask byte of the chunk, 0..15
-      const uint32_t mb = (w.m[jb >> 2] >> (8 * (jb & 3))) & 0xFFu;
-      sel[hb] = lut[mb * 8 + l8];
-    }
-  };
-  // decode quarter qq (16 columns) of stage s = half h of chunk w into Ws[buf]
-  auto store_w_quarter = [&](int s, const WChunk& w, int h, int buf, int qq, const uint2 (&selq)[2]) {
-    _Float16* dst = Ws + (size_t)buf * GB_R * GB_P + tid * GB_P + qq * 16;
-    if (FAST == 0) {
-      if (qq & 1) return;                                         // the generic reader works on 32 columns
-      uint32_t packed[16];
-      if (wok) {
-        int q[32];
-        int t = (s * GB_K >> 5) + (qq >> 1);
-        t = t < (N >> 5) ? t : (N >> 5) - 1;
-        const uint32_t keep = decode_block32(m, rv, t, q);
-        const int g = (t * BLOCK) / m.group;
-        const float sc = h2f(m.scale[meta_index(m, wrc, g)]);
-        const float z = (float)m.zero[meta_index(m, wrc, g)];
-        const bool dense = family_of(m.layout) == FAM_DENSE;
-#pragma unroll
-        for (int p = 0; p < 32; p += 2) {
-          float v0 = __fmul_rn((float)q[p] - z, sc), v1 = __fmul_rn((float)q[p + 1] - z, sc);
-          if (!dense) { v0 = ((keep >> p) & 1u) ? v0 : 0.f; v1 = ((keep >> (p + 1)) & 1u) ? v1 : 0.f; }
-          packed[p >> 1] = (uint32_t)f2h(v0) | ((uint32_t)f2h(v1) << 16);
-        }
-      } else {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) packed[e] = 0;
-      }
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-        ((uint4*)dst)[e] = make_uint4(packed[4 * e], packed[4 * e + 1], packed[4 * e + 2], packed[4 * e + 3]);
-      return;
-    }
-    const _Float16 sh = (_Float16)(wok ? w.s : 0.f);
-    const h2_t s2 = {sh, sh};
-    const uint32_t nz = 0x80808080u - w.z * 0x01010101u;
-#pragma unroll
-    for (int hb = 0; hb < 2; ++hb) {                              // two mask bytes = 16 columns
-      const int jb8 = qq * 2 + hb;                                // mask byte of the stage, 0..7
-      uint32_t b0, b1;
-      if (FAST == 1) {
-        const int blk = 2 * h + (jb8 >> 2);                       // 32-column block of the chunk
-        const uint32_t mw = w.m[blk];
-        const int jj = jb8 & 3;
-        const uint32_t r = jj == 0 ? 0u : (uint32_t)__builtin_popcount(mw & ((1u << (8 * jj)) - 1u));
-        const uint64_t st = ((uint64_t)w.c[2 * blk + 1] << 32) | w.c[2 * blk];
-        const uint32_t cw = (uint32_t)(st >> ((r * 4u) & 63u));
-        const uint32_t p0 = ((cw & 0x0F0F0F0Fu) + nz) ^ 0x80808080u;
-        const uint32_t p1 = (((cw >> 4) & 0x0F0F0F0Fu) + nz) ^ 0x80808080u;
-        b0 = __builtin_amdgcn_perm(p1, p0, selq[hb].x);
-        b1 = __builtin_amdgcn_perm(p1, p0, selq[hb].y);
-      } else {
-        const uint32_t cw = w.c[8 * h + jb8];
-        const uint32_t p0 = ((cw & 0x0F0F0F0Fu) + nz) ^ 0x80808080u;          // even columns
-        const uint32_t p1 = (((cw >> 4) & 0x0F0F0F0Fu) + nz) ^ 0x80808080u;   // odd columns
-        b0 = __builtin_amdgcn_perm(p1, p0, 0x05010400u);
-        b1 = __builtin_amdgcn_perm(p1, p0, 0x07030602u);
-      }
-      ((uint4*)dst)[hb] = bytes_to_halfs(b0, b1, s2);
-    }
-  };
-  // ---- prologue: chunks 0 and 1 into registers; stage 0 into buffer 0
-  dma_x(0, 0);
-  load_chunk(0, wA); load_chunk(1, wB);
-  __syncthreads();                                                // selector table visible
-#pragma unroll
-  for (int qq = 0; qq < 4; ++qq) {
-    uint2 sel[2];
-    fetch_sel(wA, 0, qq, sel);
-    store_w_quarter(0, wA, 0, 0, qq, sel);
-  }
-  uint2 selq[2];                                                  // selectors of the next quarter to decode
-  fetch_sel(wA, 1, 0, selq);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-
-  // One stage: matrix-core work on buffer s % 2 while stage s + 1 moves into the other buffer:
-  // its activations by direct copies issued at the top, its weights (half HD of chunk wd)
-  // decoded a quarter per phase between the MFMAs.  The selectors of the following quarter
-  // (after the last one: of quarter 0 of half HN of chunk wn) are fetched a phase early.  With
-  // LOADW the 128-column weight chunk `cl` is loaded into wl, first touched seven phases later;
-  // these loads are issued after the direct copies, so the wait before the barrier can leave
-  // them in flight.  No branches inside.
-  constexpr int NWL = FAST == 1 ? 5 : FAST == 2 ? 6 : 0;          // vector loads of one load_chunk
-  auto stage = [&](int s, auto loadw_tag, const WChunk& wd, auto hd_tag, const WChunk& wn, auto hn_tag, WChunk& wl, int cl) {
-    constexpr bool LOADW = decltype(loadw_tag)::value;
-    constexpr int HD = decltype(hd_tag)::value, HN = decltype(hn_tag)::value;
-    const int buf = s & 1;
-    const uint8_t* xb = (const uint8_t*)Xs + (size_t)buf * GB_XBUF + (128 * wt + (lane & 31)) * 128;
-    const _Float16* wb = Ws + (size_t)buf * GB_R * GB_P + (128 * wr + (lane & 31)) * GB_P + 8 * (lane >> 5);
-    v8h af[2][4], bf[2][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) af[0][i] = *(const v8h*)(xb + 4096 * i + xpc[0]);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) bf[0][j] = *(const v8h*)(wb + 32 * j * GB_P);
-    dma_x(s + 1 < nst ? s + 1 : nst - 1, buf ^ 1);
-    if (LOADW) load_chunk(cl, wl);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int kk = 0; kk < GB_K / 16; ++kk) {
-      const int c = kk & 1, n = c ^ 1;
-      if (kk + 1 < GB_K / 16) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) af[n][i] = *(const v8h*)(xb + 4096 * i + xpc[kk + 1 < 4 ? kk + 1 : 3]);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) bf[n][j] = *(const v8h*)(wb + 32 * j * GB_P + 16 * (kk + 1));
-      }
-      uint2 seln[2];
-      if (kk + 1 < GB_K / 16) fetch_sel(wd, HD, kk + 1, seln); else fetch_sel(wn, HN, 0, seln);
-      store_w_quarter(s + 1, wd, HD, buf ^ 1, kk, selq);
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[c][i], bf[c][j], acc[i][j], 0, 0, 0);
-      selq[0] = seln[0]; selq[1] = seln[1];
-#pragma unroll
-      for (int g = 0; g < 16; ++g) {                              // one MFMA, then a slice of the decode
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    // the direct copies of stage s + 1 must have landed before the barrier publishes them
-    if (LOADW && NWL == 5) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
-    else if (LOADW && NWL == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-  };
-  // Four stages per trip (two chunks): stage 2p decodes the upper half of chunk p, stage 2p+1
-  // the lower half of chunk p+1 and loads chunk p+2 into the registers chunk p has left.
-  using T = std::true_type; using Fl = std::false_type;
-  using H0 = std::integral_constant<int, 0>; using H1 = std::integral_constant<int, 1>;
-  for (int s = 0; s < nst; s += 4) {
-    const int p = s >> 1;
-    stage(s,     Fl{}, wA, H1{}, wB, H0{}, wA, 0);
-    stage(s + 1, T{},  wB, H0{}, wB, H1{}, wA, p + 2);
-    stage(s + 2, Fl{}, wB, H1{}, wA, H0{}, wB, 0);
-    stage(s + 3, T{},  wA, H0{}, wA, H1{}, wB, p + 3);
-  }
-
-  // ---- epilogue.  D[i][j] holds, in lane l and register r, token 8*(r/4) + 4*(l/32) + r%4 and
-  // weight row l%32 of its 32 x 32 block.  Each wavefront turns its 128 x 128 sub-tile around
-  // through LDS (the operand buffers are free now), 32 tokens at a time, so that global stores
-  // are whole 16-byte pieces of consecutive output columns: 256 B (f16) or 512 B (f32) per token.
-  // Everything is compile-time indexed and branch-free per element: the 256 accumulators make
-  // this straight-line code, and it has to stay small enough for the instruction cache.
-  {
-    constexpr int ESZ = YDT == CBK_F32 ? 4 : 2;
-    constexpr int PITCH = 128 * ESZ + 16;                          // bytes per token row in LDS
-    constexpr int EPP = 16 / ESZ, PPR = 128 / EPP;                 // elements per 16-byte piece, pieces per row
-    uint8_t* ep = smem + (size_t)wave * (32 * (128 * 4 + 16));
-    uint8_t* epl = ep + 4 * (lane >> 5) * PITCH + (lane & 31) * ESZ;
-    float bv[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int k = r0 + 128 * wr + 32 * j + (lane & 31);
-      bv[j] = 0.f;
-      if (a.bias && k < m.K) bv[j] = load_act<YDT>(a.bias, k);
-    }
-    const bool vec_ok = ((a.ldy * ESZ) & 15) == 0 && (((uintptr_t)a.y) & 15) == 0;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float v = acc[i][j][r] + bv[j];
-          uint8_t* d = epl + (8 * (r >> 2) + (r & 3)) * PITCH + 32 * j * ESZ;
-          if (YDT == CBK_F32) *(float*)d = v;
-          else if (YDT == CBK_F16) *(uint16_t*)d = f2h(v);
-          else {
-            const uint32_t u = __float_as_uint(v);
-            const uint32_t rn = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-            *(uint16_t*)d = (uint16_t)(((u & 0x7fffffffu) > 0x7f800000u) ? ((u >> 16) | 0x40u) : rn);
-          }
-        }
-#pragma unroll
-      for (int t = 0; t < 32 * PPR / 64; ++t) {
-        const int pc = t * 64 + lane;
-        const int row = pc / PPR, c = pc % PPR;
-        const int tok = t0 + 128 * wt + 32 * i + row, k = r0 + 128 * wr + c * EPP;
-        if (tok >= a.M || k >= m.K) continue;
-        const uint8_t* src = ep + row * PITCH + c * 16;
-        uint8_t* dst = (uint8_t*)a.y + ((size_t)tok * a.ldy + k) * ESZ;
-        if (vec_ok && k + EPP <= m.K) *(uint4*)dst = *(const uint4*)src;
-        else
-          for (int e = 0; e < EPP && k + e < m.K; ++e) {
-            if (ESZ == 4) ((float*)dst)[e] = ((const float*)src)[e];
-            else ((uint16_t*)dst)[e] = ((const uint16_t*)src)[e];
-          }
-      }
-    }
-  }
-}
-
 static inline int gb_npad(int N) { return (N + 255) / 256 * 256; }
 
 size_t gemm_big_workspace(const DMat& m, int M) {
@@ -421,32 +41,11 @@ size_t gemm_big_workspace(const DMat& m, int M) {
   return (mpad * gb_npad(m.N) * 2 + 255) & ~(size_t)255;
 }
 
-template <int FAST, int YDT>
-static int launch_big_y(const GbArgs& a, int blocks, hipStream_t st) {
-  auto kern = gemm_big_kernel<FAST, YDT>;
-  static std::atomic<int> configured{0};
-  const size_t lds = (size_t)2 * GB_XBUF + (size_t)2 * GB_R * GB_P * 2 + GB_LUT;
-  if (!configured.load(std::memory_order_acquire)) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
-      return CBK_ERR_HIP;
-    configured.store(1, std::memory_order_release);
-  }
-  hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), lds, st, a);
-  return hipGetLastError() == hipSuccess ? CBK_OK : CBK_ERR_HIP;
-}
-
-template <int FAST>
-static int launch_big(const GbArgs& a, int blocks, hipStream_t st) {
-  if (a.ydt == CBK_F32) return launch_big_y<FAST, CBK_F32>(a, blocks, st);
-  if (a.ydt == CBK_F16) return launch_big_y<FAST, CBK_F16>(a, blocks, st);
-  if (a.ydt == CBK_BF16T) return launch_big_y<FAST, CBK_BF16T>(a, blocks, st);
-  return CBK_ERR_DTYPE;
-}
-
 int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
                     const void* bias, void* ws, size_t ws_bytes, hipStream_t st) {
   if (family_of(m.layout) == FAM_SPARSE) return CBK_ERR_UNSUPPORTED;
   if (m.cs_rows > 1) return CBK_ERR_UNSUPPORTED;
+  if (ydt != CBK_F32 && ydt != CBK_F16 && ydt != CBK_BF16T) return CBK_ERR_DTYPE;
   if (!ws || ws_bytes < gemm_big_workspace(m, M)) return CBK_ERR_WORKSPACE;
   if ((uintptr_t)ws & 255) return CBK_ERR_ALIGN;
   const int Mpad = (M + GB_T - 1) / GB_T * GB_T;
@@ -461,9 +60,15 @@ int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, v
   const int blocks = ((nb + 7) / 8) * 8;
   const bool le128 = (m.flags & CBK_FLAG_ZERO_LE_128) != 0;
   const int fam = family_of(m.layout);
-  if (le128 && fam == FAM_BLK && m.bits == 4 && m.keep == 16 && m.group == 128) return launch_big<1>(a, blocks, st);
-  if (le128 && fam == FAM_DENSE && m.bits == 4 && m.group == 128) return launch_big<2>(a, blocks, st);
-  return launch_big<0>(a, blocks, st);
+  int rc = CBK_ERR_UNSUPPORTED;
+  if (le128 && (fam == FAM_BLK || fam == FAM_DENSE)) {
+    const int keep = fam == FAM_DENSE ? 0 : m.keep;
+    if (m.bits == 2) rc = launch_gemm_big_b2(a, keep, m.group, blocks, st);
+    else if (m.bits == 3) rc = launch_gemm_big_b3(a, keep, m.group, blocks, st);
+    else if (m.bits == 4) rc = launch_gemm_big_b4(a, keep, m.group, blocks, st);
+  }
+  if (rc == CBK_ERR_UNSUPPORTED) rc = launch_big_cfg<0, 0, 128>(a, blocks, st);   // generic reader
+  return rc;
 }
 
 }  // namespace cbk

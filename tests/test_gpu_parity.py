@@ -240,6 +240,44 @@ def test_gemm_matches_oracle(case, dtype, tiled):
         assert err < TOL, f"{case_id(case)} M={M}: {err}"
 
 
+@pytest.mark.parametrize("case", [(F.BLK1632_4, 4, 128, 16), (F.DENSE4, 4, 128, 0), (F.BLKC, 3, 64, 23)], ids=case_id)
+def test_gemm_odd_chunk_count_and_ragged_tiles(case):
+    """N = 3 chunks of 128 (the kernel works on chunk pairs and pads), K and M not multiples of
+    the 256 x 256 tile, every output dtype, strided activations and outputs."""
+    K, N, M = 264, 384, 300
+    raw = make_raw(case, K, N, seed=31)
+    pk = oracle_pack(case, raw)
+    W = R.dequant(pk, K, N, case[0], col_scale=raw["col_scale"], **kw_of(case))
+    x = acts(M, N, torch.float16, seed=8)
+    ref = R.forward_ref(W, _np(x))
+    for tiled in (False, True):
+        pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV, tiled=tiled)
+        for odt in (torch.float32, torch.float16, torch.bfloat16):
+            y = ops.gemm(pm, x.to(DEV), out_dtype=odt)
+            assert y.dtype == odt and rel_fro(_np(y), ref) < (TOL if odt != torch.bfloat16 else 3e-3)
+        xs = torch.zeros(M, N + 8, dtype=torch.float16); xs[:, :N] = x
+        assert rel_fro(_np(ops.gemm(pm, xs.to(DEV)[:, :N], out_dtype=torch.float32)), ref) < TOL
+
+
+@pytest.mark.parametrize("case", ALL_MFMA_CASES, ids=case_id)
+def test_gemm_every_kernel_configuration(case):
+    """Every instantiation of the prefill kernel's byte-permute decoder (code width x survivors
+    per block x group size, bitmap and dense), both byte orders, five 128-column chunks so that
+    code bits straddle 16-byte units at every skew, run twice."""
+    K, N, M = 272, 640, 260
+    raw = make_raw(case, K, N, seed=5 * case[1] + case[3])
+    pk = oracle_pack(case, raw)
+    W = R.dequant(pk, K, N, case[0], col_scale=raw["col_scale"], **kw_of(case))
+    x = acts(M, N, torch.bfloat16, seed=3)
+    ref = R.forward_ref(W, _np(x))
+    for tiled in (False, True):
+        pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV, tiled=tiled)
+        y = ops.gemm(pm, x.to(DEV), out_dtype=torch.float32)
+        err = rel_fro(_np(y), ref)
+        assert err < TOL, f"{case_id(case)} tiled={tiled}: {err}"
+        assert torch.equal(y, ops.gemm(pm, x.to(DEV), out_dtype=torch.float32))
+
+
 def test_gemm_bias_dtype_and_prune_zero():
     case = (F.BLK1632_4, 4, 128, 16)
     K, N, M = 256, 2048, 300
