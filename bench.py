@@ -13,8 +13,9 @@ rows + scales + zeros + col_scale + activations in + outputs out) streamed per s
 duration, which is the timed region (HIP events recorded on the launch stream) divided by
 the number of launches in it; the gaps between launches are therefore counted as kernel time.
 
-`prefill_gemm` reports the prefill kernel at the Gemma-3-27B MLP shapes (M=2048, bf16) in
-TFLOP/s against the 2.5 PFLOP/s dense bf16/f16 MFMA peak.
+`prefill_gemm` reports the prefill kernel at the Gemma-3-27B MLP shapes (M=2048, bf16 by
+default; --prefill-workload / --prefill-m / --prefill-dtype choose others) in TFLOP/s against
+the 2.5 PFLOP/s dense bf16/f16 MFMA peak.
 
 `cpu_baseline` is the C oracle (dequantise-then-matmul, OpenMP over rows) timed on the host
 cores on the SAME packed bytes as the first layer set, and doubles as a last parity check of
@@ -80,15 +81,16 @@ def cpu_baseline(pms, shapes, xs, ys, M, budget_s=20.0):
                 gpu_vs_oracle_rel_fro=worst)
 
 
-def prefill_gemm(torch, F, ops, dev, reps=10):
-    """Prefill kernel at the Gemma-3-27B MLP shapes, M=2048, bf16 activations."""
-    M = 2048
+def prefill_gemm(torch, F, ops, dev, workload, layout, bits, group, keep, M, dt, reps=10):
+    """Prefill kernel on the MLP matrices (gate, up, down) of a layer set."""
+    shapes = {n: (K, N) for n, K, N in SHAPES[workload]}
     rows = []
     tot_flop, tot_ms = 0.0, 0.0
-    for name, K, N in (("gate", 21504, 5376), ("down", 5376, 21504)):
-        pm = F.synth_packed(K, N, F.BLK1632_4, seed=7, device=dev).to_tiled()
-        x = torch.randn(M, N, device=dev, generator=torch.Generator(device=dev).manual_seed(N)).to(torch.bfloat16)
-        for _ in range(2):
+    for name in ("gate", "down"):
+        K, N = shapes[name]
+        pm = F.synth_packed(K, N, layout, bits, group, keep, seed=7, device=dev).to_tiled()
+        x = torch.randn(M, N, device=dev, generator=torch.Generator(device=dev).manual_seed(N)).to(dt)
+        for _ in range(3):
             y = ops.gemm(pm, x)
         torch.cuda.synchronize()
         st = torch.cuda.current_stream()
@@ -103,13 +105,16 @@ def prefill_gemm(torch, F, ops, dev, reps=10):
         tot_flop += flop * (2 if name == "gate" else 1)         # gate and up have the same shape
         tot_ms += ms * (2 if name == "gate" else 1)
         rows.append({"matrix": f"{name} {K}x{N}", "ms": round(ms, 4), "tflops": round(flop / ms / 1e9, 1)})
+        bpw = pm.bpw()
         del pm, x, y
     ach = tot_flop / tot_ms / 1e9
-    return {"workload": "gemma27b MLP (gate, up, down), M=2048, bf16 activations, BLK1632_4 3.1875 bpw, "
-                        "time includes the activation pre-scaling kernel",
+    return {"workload": f"{workload} MLP (gate, up, down), M={M}, {str(dt)[6:]} activations, {F.LAYOUT_NAME[layout]} "
+                        f"{bits}-bit keep {keep}/32 group {group}, {bpw:.4f} bpw; time includes the activation "
+                        "pre-scaling kernel",
             "tflops": round(ach, 1), "per_matrix": rows,
             "roofline": {"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                         "frac": round(ach / MFMA_PEAK_TFLOPS, 4), "traffic": None}}
+                         "frac": round(ach / MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                         "kernel": "cbk::gemm_big_kernel"}}
 
 
 def main():
@@ -125,6 +130,9 @@ def main():
     ap.add_argument("--group", type=int, default=128)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-core baseline")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM measurement")
+    ap.add_argument("--prefill-workload", default="gemma27b", choices=list(SHAPES))
+    ap.add_argument("--prefill-m", type=int, default=2048)
+    ap.add_argument("--prefill-dtype", default="bf16", choices=["f16", "bf16"])
     ap.add_argument("--launch", default="phase", choices=["matrix", "phase", "layer"],
                     help="GEMVs per launch: one matrix, one dependency phase (qkv | o | gate,up | down), or the layer set")
     ap.add_argument("--no-graph", action="store_true", help="launch from the host instead of replaying HIP graphs")
@@ -261,7 +269,8 @@ def main():
     del graphs, sets, calls, keep_alive
     torch.cuda.empty_cache()
     if not a.no_prefill:
-        out["prefill_gemm"] = prefill_gemm(torch, F, ops, dev)
+        out["prefill_gemm"] = prefill_gemm(torch, F, ops, dev, a.prefill_workload, layout, a.bits, a.group, a.keep,
+                                           a.prefill_m, torch.float16 if a.prefill_dtype == "f16" else torch.bfloat16)
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline(first_rowmajor, shapes, xs, y_first, M)
         # outputs are rounded to the activation dtype (2^-11 relative) on top of the kernel's own error

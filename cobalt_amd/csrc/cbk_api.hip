@@ -144,8 +144,7 @@ size_t cbk_stream_bytes(const cbk_desc* in, size_t sparse_data_bytes) {
 size_t cbk_workspace_bytes(const cbk_desc* in, int M) {
   DMat m;
   if (to_dmat(in, &m, false)) return 0;
-  const int mc = M > 4 ? 4 : M;
-  if (M >= 1 && M <= 16 && gemv_fast_takes(m, mc)) return gemv_fast_workspace(m, mc);
+  if (M >= 1 && M <= 16 && gemv_fast_takes(m, 1)) return gemv_fast_workspace(m, 1);
   if (gemm_big_takes(m, M)) return gemm_big_workspace(m, M);
   return 0;
 }
@@ -174,6 +173,8 @@ int cbk_gemv_batch(int n, const cbk_desc* descs, const void* const* xs, const in
   if (!descs || !xs || !ldxs || !ys || !ldys) return CBK_ERR_NULL;
   if (M > 16) return CBK_ERR_SHAPE;
   GvCall calls[kMaxBatch];
+  // activation rows per pass: as many (4, 2 or 1) as the digits of every matrix fit in LDS with
+  int mc = M >= 4 ? 4 : (M >= 2 ? 2 : 1);
   bool fast = true;
   for (int i = 0; i < n; ++i) {
     int rc = to_dmat(descs + i, &calls[i].m, true);
@@ -182,24 +183,21 @@ int cbk_gemv_batch(int n, const cbk_desc* descs, const void* const* xs, const in
     if (rc) return rc;
     calls[i].x = xs[i]; calls[i].ldx = ldxs[i]; calls[i].y = ys[i]; calls[i].ldy = ldys[i];
     calls[i].bias = biases ? biases[i] : nullptr;
-    fast = fast && gemv_fast_takes(calls[i].m, M > 4 ? 4 : M) && gemv_same_config(calls[0].m, calls[i].m);
+    while (mc > 1 && !gemv_fast_takes(calls[i].m, mc) && gemv_fast_takes(calls[i].m, 1)) mc >>= 1;
+    fast = fast && gemv_fast_takes(calls[i].m, 1) && gemv_same_config(calls[0].m, calls[i].m);
   }
   hipStream_t st = (hipStream_t)stream;
   if (fast) {
-    size_t need = 0;
-    for (int i = 0; i < n; ++i) need += gemv_fast_workspace(calls[i].m, M > 4 ? 4 : M);
-    if (need && (!workspace || workspace_bytes < need)) return CBK_ERR_WORKSPACE;
-    if (need && ((uintptr_t)workspace & 255)) return CBK_ERR_ALIGN;
     const size_t ysz = y_dtype == CBK_F32 ? 4 : 2;
-    for (int m0 = 0; m0 < M; m0 += 4) {                 // at most 4 activation rows per launch
-      const int mc = M - m0 < 4 ? M - m0 : 4;
+    for (int m0 = 0, mp; m0 < M; m0 += mp) {            // the weights are streamed once per pass
+      mp = M - m0 < mc ? M - m0 : mc;
       GvCall part[kMaxBatch];
       for (int i = 0; i < n; ++i) {
         part[i] = calls[i];
         part[i].x = (const uint8_t*)calls[i].x + (size_t)m0 * calls[i].ldx * 2;
         part[i].y = (uint8_t*)calls[i].y + (size_t)m0 * calls[i].ldy * ysz;
       }
-      int rc = launch_gemv_fast_batch(n, part, x_dtype, mc, y_dtype, workspace, workspace_bytes, st);
+      int rc = launch_gemv_fast_batch(n, part, x_dtype, mp, y_dtype, workspace, workspace_bytes, st);
       if (rc) return rc;
     }
     return CBK_OK;
@@ -225,7 +223,7 @@ int cbk_gemv(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ldx,
   rc = check_io(x, x_dtype, M, ldx, y, y_dtype, ldy, m.N, m.K);
   if (rc) return rc;
   if (M > 16) return CBK_ERR_SHAPE;
-  if (gemv_fast_takes(m, M > 4 ? 4 : M))
+  if (gemv_fast_takes(m, 1))
     return cbk_gemv_batch(1, in, &x, &ldx, x_dtype, M, &y, &ldy, y_dtype, &bias, workspace, workspace_bytes, stream);
   return launch_gemv_generic(m, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, (hipStream_t)stream);
 }
