@@ -33,8 +33,6 @@
 // Reference semantics: cbk::gemv_blk1632_multi / gemv_dense4_multi
 // (src/cobaltkernel/csrc/cobalt_gemv.cuh:617-712, :839-1123): same sums, other machinery.
 #include <atomic>
-#include <cstdio>
-#include <cstdlib>
 #include "cbk_decode.h"
 
 namespace cbk {
@@ -77,11 +75,19 @@ struct GvMat {
   uint32_t row_a, ustride;
 };
 
-struct GvBatch {
-  GvMat mat[GV_MAX_BATCH];
-  int n, M, xdt, ydt, total_cost;
+// What every wavefront needs before it can find its work: small, first in the kernel
+// arguments and read in one go (each dependent read of the argument block is a round trip).
+struct GvHead {
+  int n, M, xdt, ydt;
+  int cq, cr;              // cost units per workgroup: cq, and one more for the first cr workgroups
   int xq_cap, delta_cap;   // LDS bytes reserved for digits / floats reserved for delta
   int sk_cap, nslot, red_floats;   // reduction slots: nslot x sk_cap x M x 16 floats
+  int cost_end[GV_MAX_BATCH];      // cost0 + ntiles * nS of every matrix (total cost from entry n on)
+};
+
+struct GvBatch {
+  GvHead h;
+  GvMat mat[GV_MAX_BATCH];
 };
 
 // Column order of the activation digits inside a 16-column fragment: the byte order in which
@@ -177,9 +183,10 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
   uint2* lut = (uint2*)smem;
   uint8_t* zreg = smem + LUT_BYTES;
   int8_t* xq = (int8_t*)(zreg + ZERO_BYTES);
-  float* delta = (float*)(xq + b.xq_cap);
-  float* red = delta + b.delta_cap;                    // [nslot][sk_cap][M][16] partial sums
-  int* cnt = (int*)(red + b.red_floats);               // [nslot] arrival counters
+  const GvHead h = b.h;
+  float* delta = (float*)(xq + h.xq_cap);
+  float* red = delta + h.delta_cap;                    // [nslot][sk_cap][M][16] partial sums
+  int* cnt = (int*)(red + h.red_floats);               // [nslot] arrival counters
 
   const int wr = lane & 15, kq = lane >> 4;            // weight row in tile / lane quarter
   const uint32_t l16 = lane & (LUT_LANES - 1);
@@ -190,12 +197,18 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
   const uint32_t xq_off = (uint32_t)((uint8_t*)xq - smem), z_off = (uint32_t)(zreg - smem);
 
   // the tiles of this workgroup: those whose first cost unit falls in [c0, c1)
-  const int c0 = (int)(((int64_t)b.total_cost * blockIdx.x) / gridDim.x);
-  const int c1 = (int)(((int64_t)b.total_cost * (blockIdx.x + 1)) / gridDim.x);
+  const int bx = (int)blockIdx.x;
+  const int c0 = bx * h.cq + (bx < h.cr ? bx : h.cr);
+  const int c1 = c0 + h.cq + (bx < h.cr ? 1 : 0);
   bool first = true;
+  // first matrix with cost units at or after c0
+  int mi0 = 0;
+#pragma unroll
+  for (int i = 0; i < GV_MAX_BATCH; ++i) mi0 += (i < h.n && h.cost_end[i] <= c0) ? 1 : 0;
 
-  for (int mi = 0; mi < b.n; ++mi) {
-    const GvMat& gm = b.mat[mi];
+  for (int mi = mi0; mi < h.n; ++mi) {
+    const GvMat gm = b.mat[mi];                                   // one read of the whole record
+    if (gm.cost0 >= c1) break;                                    // uniform over the workgroup
     const DMat& m = gm.m;
     const int nS = gm.nS;
     int t_lo = (c0 - gm.cost0 + nS - 1) / nS, t_hi = (c1 - gm.cost0 + nS - 1) / nS;
@@ -206,7 +219,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     // items: tile tl (local), part j of SK; part j covers macro-steps [j*spi, min(nS,(j+1)*spi))
     const int SK = gm.sk, spi = gm.spi;
     const int nitems = (t_hi - t_lo) * SK;
-    const int gt = b.nslot >> 1;                                  // tiles per barrier group
+    const int gt = h.nslot >> 1;                                  // tiles per barrier group
 
     // matrix constants, read from the kernel arguments once
     const uint8_t* const m_data = m.data;
@@ -266,7 +279,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     // The activation loads go out before the first weight loads: the weight prefetch of a whole
     // launch is tens of megabytes, and a request queued behind it would keep every wavefront
     // from decoding until that burst has drained.
-    const int n16 = N >> 4, xitems = b.M * n16;                   // a multiple of 8
+    const int n16 = N >> 4, xitems = h.M * n16;                   // a multiple of 8
     int xit = tid;
     XLoad xl;
     if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, xl);
@@ -282,13 +295,13 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
         for (int j = 0; j < LUT_LANES; ++j) lut[tid * LUT_LANES + j] = e;
       } else if (tid < 256 + ZERO_BYTES / 4) {
         ((uint32_t*)zreg)[tid - 256] = 0u;
-      } else if (tid < 256 + ZERO_BYTES / 4 + b.nslot) {
+      } else if (tid < 256 + ZERO_BYTES / 4 + h.nslot) {
         cnt[tid - 256 - ZERO_BYTES / 4] = 0;
       }
       first = false;
     }
     while (xit < xitems) {
-      stage_convert(xl, m.cs != nullptr, b.xdt, gm.order, N, n16, xit, xq, delta);
+      stage_convert(xl, m.cs != nullptr, h.xdt, gm.order, N, n16, xit, xq, delta);
       xit += GV_THREADS;
       if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, xl);
     }
@@ -316,7 +329,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
         uint32_t aaddr[MP];
 #pragma unroll
         for (int p = 0; p < MP; ++p) {
-          const bool on = valid && a_slice == kq && a_dig < NDIG && p < b.M;
+          const bool on = valid && a_slice == kq && a_dig < NDIG && p < h.M;
           aaddr[p] = on ? xq_off + (uint32_t)((p * NDIG + a_dig) * N + chunk * 128) : z_off;
         }
         // ---- bring the chunk's first code bit to bit 0 of cw[0]
@@ -392,7 +405,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
               const int g = (C::NGC == 2 && t == 7) ? 1 : 0;
 #pragma unroll
               for (int p = 0; p < MP; ++p) {
-                const float dl = delta[(p < b.M ? p : 0) * (NCH + 4) + chunk];      // 0 past the last chunk
+                const float dl = delta[(p < h.M ? p : 0) * (NCH + 4) + chunk];      // 0 past the last chunk
                 const float f = fmaf((float)(acc[p][0] * 256 + acc[p][1]), 256.f, (float)acc[p][2]);
                 ysum[p] = fmaf(f, h2f((uint16_t)cur.sc[g]) * dl, ysum[p]);
                 acc[p] = (v4i){0, 0, 0, 0};
@@ -413,32 +426,32 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       auto store = [&](int om, int r, float v) {
         const int k = tile * 16 + r;
         if (k >= m.K) return;
-        if (gm.bias) v += (b.ydt == CBK_F32) ? ((const float*)gm.bias)[k]
-                        : (b.ydt == CBK_F16) ? h2f(((const uint16_t*)gm.bias)[k]) : bf2f(((const uint16_t*)gm.bias)[k]);
+        if (gm.bias) v += (h.ydt == CBK_F32) ? ((const float*)gm.bias)[k]
+                        : (h.ydt == CBK_F16) ? h2f(((const uint16_t*)gm.bias)[k]) : bf2f(((const uint16_t*)gm.bias)[k]);
         const size_t o = (size_t)om * gm.ldy + k;
-        if (b.ydt == CBK_F32) ((float*)gm.y)[o] = v;
-        else if (b.ydt == CBK_F16) ((uint16_t*)gm.y)[o] = f2h(v);
+        if (h.ydt == CBK_F32) ((float*)gm.y)[o] = v;
+        else if (h.ydt == CBK_F16) ((uint16_t*)gm.y)[o] = f2h(v);
         else ((uint16_t*)gm.y)[o] = f2bf(v);
       };
       if (SK == 1) {
 #pragma unroll
         for (int p = 0; p < MP; ++p)
-          if (kq == 0 && p < b.M) store(p, wr, part_sum[p]);
+          if (kq == 0 && p < h.M) store(p, wr, part_sum[p]);
       } else {
         // partial sums of the SK parts of a tile meet in an LDS slot; the wave that arrives last
         // adds them in part order (not arrival order), so the result does not depend on timing
-        const int slot = tl & (b.nslot - 1);
-        float* rs = red + (size_t)slot * b.sk_cap * b.M * 16;
+        const int slot = tl & (h.nslot - 1);
+        float* rs = red + (size_t)slot * h.sk_cap * h.M * 16;
 #pragma unroll
         for (int p = 0; p < MP; ++p)
-          if (kq == 0 && p < b.M) rs[(part * b.M + p) * 16 + wr] = part_sum[p];
+          if (kq == 0 && p < h.M) rs[(part * h.M + p) * 16 + wr] = part_sum[p];
         int old = 0;
         if (lane == 0) old = atomicAdd(&cnt[slot], 1);
         old = __shfl(old, 0, 64);
         if (old == SK - 1) {                                      // uniform over the wave
-          for (int om = kq; om < b.M; om += 4) {
+          for (int om = kq; om < h.M; om += 4) {
             float v = 0.f;
-            for (int j = 0; j < SK; ++j) v += rs[(j * b.M + om) * 16 + wr];
+            for (int j = 0; j < SK; ++j) v += rs[(j * h.M + om) * 16 + wr];
             store(om, wr, v);
           }
           if (lane == 0) cnt[slot] = 0;
@@ -497,15 +510,13 @@ static int launch_cfg(const GvBatch& b, size_t lds, int blocks, hipStream_t st) 
     configured.store(1, std::memory_order_release);
   }
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(GV_THREADS), lds, st, b);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess && getenv("CBK_DEBUG")) fprintf(stderr, "gemv launch failed: %s (lds %zu blocks %d M %d)\n", hipGetErrorString(e), lds, blocks, b.M);
-  return e == hipSuccess ? CBK_OK : CBK_ERR_HIP;
+  return hipGetLastError() == hipSuccess ? CBK_OK : CBK_ERR_HIP;
 }
 
 template <int BITS, int KEEP, int GRP>
 static int launch_mp(const GvBatch& b, size_t lds, int blocks, hipStream_t st) {
-  if (b.M == 1) return launch_cfg<BITS, KEEP, GRP, 1>(b, lds, blocks, st);
-  if (b.M == 2) return launch_cfg<BITS, KEEP, GRP, 2>(b, lds, blocks, st);
+  if (b.h.M == 1) return launch_cfg<BITS, KEEP, GRP, 1>(b, lds, blocks, st);
+  if (b.h.M == 2) return launch_cfg<BITS, KEEP, GRP, 2>(b, lds, blocks, st);
   return launch_cfg<BITS, KEEP, GRP, 4>(b, lds, blocks, st);
 }
 
@@ -532,7 +543,7 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
                            hipStream_t st) {
   if (n < 1 || n > GV_MAX_BATCH) return CBK_ERR_SHAPE;
   GvBatch gb;
-  gb.n = n; gb.M = M; gb.xdt = xdt; gb.ydt = ydt;
+  gb.h.n = n; gb.h.M = M; gb.h.xdt = xdt; gb.h.ydt = ydt;
   int cost = 0, xq_cap = 0, delta_cap = 0, tiles = 0;
   for (int i = 0; i < n; ++i) {
     const DMat& m = calls[i].m;
@@ -545,19 +556,19 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
     g.rsh = m.tiled ? 4 : 0; g.rmask = m.tiled ? 15 : 0;
     g.row_a = m.tiled ? m.stride * 16u : m.stride; g.ustride = m.tiled ? 256u : 16u;
     cost += g.ntiles * g.nS;
+    gb.h.cost_end[i] = cost;
     tiles += g.ntiles;
     xq_cap = xq_cap > M * NDIG * m.N ? xq_cap : M * NDIG * m.N;
     delta_cap = delta_cap > M * (m.N / 128 + 4) ? delta_cap : M * (m.N / 128 + 4);
   }
   (void)workspace; (void)ws_bytes;
-  gb.total_cost = cost; gb.xq_cap = xq_cap; gb.delta_cap = delta_cap;
+  for (int i = n; i < GV_MAX_BATCH; ++i) gb.h.cost_end[i] = cost;
+  gb.h.xq_cap = xq_cap; gb.h.delta_cap = delta_cap;
   int blocks = tiles < 256 ? tiles : 256;                       // one persistent workgroup per CU
-  if (const char* e = getenv("CBK_GV_BLOCKS")) blocks = atoi(e) < tiles ? atoi(e) : tiles;
   // macro-steps per work item: about two items per wavefront over the whole launch, so that
   // the tail is short; a tile is split into at most 16 parts
   int spi = cost / (blocks * GV_WAVES * 2);
   spi = spi < 1 ? 1 : (spi > 8 ? 8 : spi);
-  if (const char* e = getenv("CBK_GV_SPI")) spi = atoi(e);
   int sk_cap = 1;
   for (int i = 0; i < n; ++i) {
     GvMat& g = gb.mat[i];
@@ -571,9 +582,10 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
   const int slot_floats = sk_cap * M * 16;
   int nslot = 64;
   while (nslot > 2 && (size_t)nslot * slot_floats * 4 > 24 * 1024) nslot >>= 1;
-  gb.sk_cap = sk_cap; gb.nslot = nslot; gb.red_floats = nslot * slot_floats;
+  gb.h.sk_cap = sk_cap; gb.h.nslot = nslot; gb.h.red_floats = nslot * slot_floats;
+  gb.h.cq = cost / blocks; gb.h.cr = cost % blocks;
   const size_t lds = (size_t)LUT_BYTES + ZERO_BYTES + xq_cap + (size_t)delta_cap * 4 +
-                     (size_t)gb.red_floats * 4 + (size_t)nslot * 4;
+                     (size_t)gb.h.red_floats * 4 + (size_t)nslot * 4;
   const int bits = gb.mat[0].m.bits;
   return bits == 2 ? launch_keep<2>(gb, lds, blocks, st) : bits == 3 ? launch_keep<3>(gb, lds, blocks, st)
        : bits == 4 ? launch_keep<4>(gb, lds, blocks, st) : CBK_ERR_UNSUPPORTED;
