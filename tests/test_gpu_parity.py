@@ -324,6 +324,38 @@ def test_cobalt_linear_forward_matches_reference_module_math():
             assert rel_fro(_np(y), ref) < 6e-4
 
 
+def test_from_linear_single_layer_configuration():
+    """The reference's single-layer case: W 4096x4096 ~ N(0, 0.02) with 1 % of the columns
+    scaled by 10, calibration activations 128x4096 ~ N(0, 1), column-balanced mask at sparsity
+    0.5, OBS, 4-bit RTN group 128, x 1x4096 fp16.  Compressed on the GPU by the product, then
+    the HIP forward is compared with the C oracle's forward over the packed bytes."""
+    from oracle import cbk_ref_c as RC
+    g = torch.Generator().manual_seed(0)
+    K = N = 4096
+    W = torch.randn(K, N, generator=g) * 0.02
+    W[:, torch.randperm(N, generator=g)[:41]] *= 10
+    X = torch.randn(128, N, generator=g)
+    lin = torch.nn.Linear(N, K, bias=False)
+    lin.weight.data.copy_(W)
+    m = CobaltLinear.from_linear(lin.to(DEV), X_cal=X.to(DEV), sparsity=0.5, bits=4, group=128)
+    pm = m.packed()
+    assert pm.layout == F.BLK1632_4 and abs(pm.bpw() - 3.1875) < 1e-9
+    cpu = pm.to("cpu")
+    pk = dict(data=cpu.array("data").numpy(), scale=cpu.array("scale").numpy().reshape(K, -1),
+              zero=cpu.array("zero").numpy().reshape(K, -1))
+    cs = cpu.array("col_scale").numpy().reshape(1, N)
+    x = torch.randn(1, N, generator=g).half()
+    ref = RC.forward(pk, K, N, pm.layout, x.float().numpy(), col_scale=cs)
+    for tiled in (False, True):
+        if tiled:
+            m.to_device_order()
+        y = ops.linear(m._pm(), x.to(DEV), out_dtype=torch.float32)
+        assert rel_fro(_np(y), ref) < TOL
+    # the compressed layer still computes roughly what the dense one did on calibration-like inputs
+    dense = (x.float() @ W.T).numpy()
+    assert rel_fro(ref, dense) < 0.35
+
+
 # ------------------------------------------------------------------ full-size properties
 @pytest.mark.parametrize("K,N,case", [(14336, 4096, (F.BLK1632_4, 4, 128, 16)), (4096, 14336, (F.BLKC, 3, 128, 10)),
                                       (5376, 21504, (F.BLKC, 2, 64, 23))], ids=["mistral-gate", "mistral-down-b3", "gemma-down-b2g64"])
