@@ -118,22 +118,28 @@ __device__ inline void stage_load(const uint16_t* x, int64_t ldx, const uint16_t
 
 // conversion of one loaded item into digits and delta in LDS; the eight consecutive lanes of a
 // chunk are always active together (the item count is a multiple of 8)
-__device__ inline void stage_convert(const XLoad& r, bool has_cs, int xdt, int order, int N, int n16, int it,
+template <int ORDER>
+__device__ inline void stage_convert(const XLoad& r, bool has_cs, int xdt, int N, int n16, int it,
                                      int8_t* xq, float* delta) {
   const int NCH = N >> 7;
   const int row = it / n16, c16 = it - row * n16;
   const uint32_t* xw = (const uint32_t*)r.x;
   const uint32_t* cw = (const uint32_t*)r.c;
   float xv[16];
+  if (xdt == CBK_F16) {                                            // one uniform branch, not one per element
+#pragma unroll
+    for (int e = 0; e < 16; ++e) xv[e] = h2f((uint16_t)(xw[e >> 1] >> (16 * (e & 1))));
+  } else {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) xv[e] = bf2f((uint16_t)(xw[e >> 1] >> (16 * (e & 1))));
+  }
+  if (has_cs) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) xv[e] *= h2f((uint16_t)(cw[e >> 1] >> (16 * (e & 1))));
+  }
   float mx = 0.f;
 #pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    const uint16_t xb = (uint16_t)(xw[e >> 1] >> (16 * (e & 1)));
-    float v = xdt == CBK_F16 ? h2f(xb) : bf2f(xb);
-    if (has_cs) v *= h2f((uint16_t)(cw[e >> 1] >> (16 * (e & 1))));
-    xv[e] = v;
-    mx = fmaxf(mx, fabsf(v));
-  }
+  for (int e = 0; e < 16; ++e) mx = fmaxf(mx, fabsf(xv[e]));
   mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
   mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
   mx = fmaxf(mx, __shfl_xor(mx, 4, 64));
@@ -146,10 +152,7 @@ __device__ inline void stage_convert(const XLoad& r, bool has_cs, int xdt, int o
     for (int q = 0; q < 4; ++q) dw[k][q] = 0u;
 #pragma unroll
   for (int bi = 0; bi < 16; ++bi) {
-    float v;
-    if (order == 0) v = xv[bi];
-    else if (order == 1) v = xv[frag_col(4, true, bi)];
-    else v = xv[frag_col(2, true, bi)];
+    const float v = ORDER == 0 ? xv[bi] : ORDER == 1 ? xv[frag_col(4, true, bi)] : xv[frag_col(2, true, bi)];
     int X = (int)rintf(v * inv);                       // |X| <= 127 * 65536
     const int d0 = (int)(int8_t)(X & 0xFF);
     X = (X - d0) >> 8;
@@ -301,7 +304,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       first = false;
     }
     while (xit < xitems) {
-      stage_convert(xl, m.cs != nullptr, h.xdt, gm.order, N, n16, xit, xq, delta);
+      stage_convert<(!C::DENSE ? 0 : (BITS == 2 ? 2 : 1))>(xl, m.cs != nullptr, h.xdt, N, n16, xit, xq, delta);
       xit += GV_THREADS;
       if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, xl);
     }
