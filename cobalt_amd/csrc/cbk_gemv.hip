@@ -286,8 +286,10 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     int xit = tid;
     XLoad xl;
     if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, xl);
-    Loads<C> cur, nx1, nx2;                                       // two steps of loads stay in flight
-    issue(t_lo + p0.tl, p0.S, cur);
+    // Three load buffers rotate through the roles (being decoded, next, being loaded) by name:
+    // copying a buffer would wait for the loads that are still filling it.
+    Loads<C> LA, LB, LC;
+    issue(t_lo + p0.tl, p0.S, LA);
 
     // ---- stage: selector table and counters (once), activation digits and deltas of this matrix
     if (!first) __syncthreads();                                  // previous matrix fully consumed
@@ -310,12 +312,12 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     }
     // the second step of loads goes out only now: issued together with the first, the two
     // bursts of all wavefronts interleave in the memory system and every first step lands late
-    issue(t_lo + p1.tl, p1.S, nx1);
+    issue(t_lo + p1.tl, p1.S, LB);
     __syncthreads();
 
     int bars = 0;                                                 // group barriers passed so far
     float ysum[MP];
-    while (v0) {
+    auto do_step = [&](Loads<C>& cur, Loads<C>& tgt) {             // decode `cur`, load two steps ahead into `tgt`
       const int tl = p0.tl, part = p0.part, S = p0.S;
       const int tile = t_lo + tl;
       const int s_end = (part * spi + spi < nS) ? part * spi + spi : nS;
@@ -325,7 +327,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 #pragma unroll
         for (int p = 0; p < MP; ++p) ysum[p] = 0.f;
       }
-      issue(t_lo + p2.tl, p2.S, nx2);
+      issue(t_lo + p2.tl, p2.S, tgt);
       {
         const int chunk = 4 * S + kq;
         const bool valid = chunk < NCH;
@@ -417,7 +419,6 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
           }
         }
       }
-      cur = nx1; nx1 = nx2;
       if (S + 1 == s_end) {
       // ---- the item is done: add the four lane quarters (the four chunks of every macro-step)
       float part_sum[MP];
@@ -463,6 +464,14 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       }
       p0 = p1; v0 = v1; p1 = p2; v1 = v2;
       if (v2) v2 = advance(p2);
+    };
+    while (true) {
+      if (!v0) break;
+      do_step(LA, LC);
+      if (!v0) break;
+      do_step(LB, LA);
+      if (!v0) break;
+      do_step(LC, LB);
     }
     // every wave passes the same number of group barriers
     const int ngroups = ((t_hi - t_lo) + gt - 1) / gt;
