@@ -288,6 +288,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, xl);
     // Three load buffers rotate through the roles (being decoded, next, being loaded) by name:
     // copying a buffer would wait for the loads that are still filling it.
+    // Configurations with long code streams or four activation rows keep one step in flight
+    // instead of two: three buffers would not fit the 128 registers of a 16-wavefront workgroup.
+    constexpr bool DEEP = C::NL <= 8 && MP < 4;
     Loads<C> LA, LB, LC;
     issue(t_lo + p0.tl, p0.S, LA);
 
@@ -312,7 +315,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     }
     // the second step of loads goes out only now: issued together with the first, the two
     // bursts of all wavefronts interleave in the memory system and every first step lands late
-    issue(t_lo + p1.tl, p1.S, LB);
+    if (DEEP) issue(t_lo + p1.tl, p1.S, LB);
     __syncthreads();
 
     int bars = 0;                                                 // group barriers passed so far
@@ -327,7 +330,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 #pragma unroll
         for (int p = 0; p < MP; ++p) ysum[p] = 0.f;
       }
-      issue(t_lo + p2.tl, p2.S, tgt);
+      if (DEEP) issue(t_lo + p2.tl, p2.S, tgt); else issue(t_lo + p1.tl, p1.S, tgt);
       {
         const int chunk = 4 * S + kq;
         const bool valid = chunk < NCH;
@@ -467,11 +470,13 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     };
     while (true) {
       if (!v0) break;
-      do_step(LA, LC);
+      do_step(LA, DEEP ? LC : LB);
       if (!v0) break;
       do_step(LB, LA);
-      if (!v0) break;
-      do_step(LC, LB);
+      if (DEEP) {
+        if (!v0) break;
+        do_step(LC, LB);
+      }
     }
     // every wave passes the same number of group barriers
     const int ngroups = ((t_hi - t_lo) + gt - 1) / gt;
