@@ -108,8 +108,9 @@ __host__ __device__ constexpr int frag_col(int bits, bool dense, int bi) {
 struct XLoad { uint4 x[2], c[2]; };
 
 // global loads of staging item `it` (activation row it / (N/16), columns 16 * (it % (N/16)) ...)
-__device__ inline void stage_load(const uint16_t* x, int64_t ldx, const uint16_t* cs, int n16, int it, XLoad& r) {
-  const int row = it / n16, c16 = it - row * n16;
+__device__ inline void stage_load(const uint16_t* x, int64_t ldx, const uint16_t* cs, int n16, int it, bool one_row,
+                                  XLoad& r) {
+  const int row = one_row ? 0 : it / n16, c16 = it - row * n16;
   const uint16_t* xp = x + (size_t)row * ldx + c16 * 16;
   r.x[0] = ((const uint4*)xp)[0]; r.x[1] = ((const uint4*)xp)[1];
   r.c[0] = make_uint4(0, 0, 0, 0); r.c[1] = make_uint4(0, 0, 0, 0);
@@ -119,10 +120,10 @@ __device__ inline void stage_load(const uint16_t* x, int64_t ldx, const uint16_t
 // conversion of one loaded item into digits and delta in LDS; the eight consecutive lanes of a
 // chunk are always active together (the item count is a multiple of 8)
 template <int ORDER>
-__device__ inline void stage_convert(const XLoad& r, bool has_cs, int xdt, int N, int n16, int it,
+__device__ inline void stage_convert(const XLoad& r, bool has_cs, int xdt, int N, int n16, int it, bool one_row,
                                      int8_t* xq, float* delta) {
   const int NCH = N >> 7;
-  const int row = it / n16, c16 = it - row * n16;
+  const int row = one_row ? 0 : it / n16, c16 = it - row * n16;
   const uint32_t* xw = (const uint32_t*)r.x;
   const uint32_t* cw = (const uint32_t*)r.c;
   float xv[16];
@@ -140,9 +141,12 @@ __device__ inline void stage_convert(const XLoad& r, bool has_cs, int xdt, int N
   float mx = 0.f;
 #pragma unroll
   for (int e = 0; e < 16; ++e) mx = fmaxf(mx, fabsf(xv[e]));
-  mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
-  mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
-  mx = fmaxf(mx, __shfl_xor(mx, 4, 64));
+  // maximum over the eight lanes of the chunk with register-to-register lane moves: swap
+  // neighbours, swap pairs, mirror the eight-lane half row (every lane of a quad holds the
+  // quad's maximum by then, so the mirror image is the other quad's)
+  mx = fmaxf(mx, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, mx), 0xB1, 0xF, 0xF, true)));
+  mx = fmaxf(mx, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, mx), 0x4E, 0xF, 0xF, true)));
+  mx = fmaxf(mx, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, mx), 0x141, 0xF, 0xF, true)));
   const float d = mx > 0.f ? mx / 8323072.f : 1.f;
   const float inv = 1.f / d;
   uint32_t dw[NDIG][4];
@@ -285,7 +289,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     const int n16 = N >> 4, xitems = h.M * n16;                   // a multiple of 8
     int xit = tid;
     XLoad xl;
-    if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, xl);
+    if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, MP == 1, xl);
     // Three load buffers rotate through the roles (being decoded, next, being loaded) by name:
     // copying a buffer would wait for the loads that are still filling it.
     // Configurations with long code streams or four activation rows keep one step in flight
@@ -309,9 +313,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       first = false;
     }
     while (xit < xitems) {
-      stage_convert<(!C::DENSE ? 0 : (BITS == 2 ? 2 : 1))>(xl, m.cs != nullptr, h.xdt, N, n16, xit, xq, delta);
+      stage_convert<(!C::DENSE ? 0 : (BITS == 2 ? 2 : 1))>(xl, m.cs != nullptr, h.xdt, N, n16, xit, MP == 1, xq, delta);
       xit += GV_THREADS;
-      if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, xl);
+      if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, MP == 1, xl);
     }
     // the second step of loads goes out only now: issued together with the first, the two
     // bursts of all wavefronts interleave in the memory system and every first step lands late
