@@ -246,25 +246,22 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   };
   constexpr int NWL = FASTD ? (BITMAP ? 1 : 0) + C::NL / 4 + 2 * C::NGC : 0;   // vector loads of one load_chunk
 
-  // selectors of the two mask bytes of quarter qq of half h of a chunk (bitmap layouts only)
-  auto fetch_sel = [&](const WChunk& w, int h, int qq, uint2 (&sel)[2]) {
-    if (!BITMAP) return;
-#pragma unroll
-    for (int hb = 0; hb < 2; ++hb) {
-      const int jb = 8 * h + qq * 2 + hb;                          // mask byte of the chunk, 0..15
-      const uint32_t mb = (w.m[jb >> 2] >> (8 * (jb & 3))) & 0xFFu;
-      sel[hb] = lut[mb * 8 + l8];
-    }
+  // selectors of mask byte b8 (0..7) of half h of a chunk (bitmap layouts only)
+  auto fetch_sel = [&](const WChunk& w, int h, int b8) -> uint2 {
+    if (!BITMAP) return make_uint2(0, 0);
+    const int jb = 8 * h + b8;                                     // mask byte of the chunk, 0..15
+    const uint32_t mb = (w.m[jb >> 2] >> (8 * (jb & 3))) & 0xFFu;
+    return lut[mb * 8 + l8];
   };
-  // decode quarter qq (16 columns) of stage s = half h of chunk w into Ws[buf]
-  auto store_w_quarter = [&](int s, WChunk& w, int h, int buf, int qq, const uint2 (&selq)[2]) {
-    _Float16* dst = Ws + (size_t)buf * GB_R * GB_P + tid * GB_P + qq * 16;
+  // decode mask byte b8 (8 columns) of stage s = half h of chunk w into Ws[buf]
+  auto store_w_byte = [&](int s, WChunk& w, int h, int buf, int b8, uint2 sel) {
+    _Float16* dst = Ws + (size_t)buf * GB_R * GB_P + tid * GB_P + b8 * 8;
     if (!FASTD) {
-      if (qq & 1) return;                                         // the generic reader works on 32 columns
+      if (b8 & 3) return;                                         // the generic reader works on 32 columns
       uint32_t packed[16];
       if (wok) {
         int q[32];
-        int t = (s * GB_K >> 5) + (qq >> 1);
+        int t = (s * GB_K >> 5) + (b8 >> 2);
         t = t < (N >> 5) ? t : (N >> 5) - 1;
         const uint32_t keep = decode_block32(m, rv, t, q);
         const int g = (t * BLOCK) / m.group;
@@ -286,115 +283,137 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
         ((uint4*)dst)[e] = make_uint4(packed[4 * e], packed[4 * e + 1], packed[4 * e + 2], packed[4 * e + 3]);
       return;
     }
-    if (h == 0 && qq == 0) align_chunk_codes<C>(w.raw, w.ci, w.c);  // once per chunk, at its first use
-    const int blk = 2 * h + (qq >> 1);                              // 32-column block of the chunk
-    if ((qq & 1) == 0) block_stream<C, BITS>(w.c, blk, st);          // once per block
+    if (h == 0 && b8 == 0) align_chunk_codes<C>(w.raw, w.ci, w.c);  // once per chunk, at its first use
+    const int blk = 2 * h + (b8 >> 2);                              // 32-column block of the chunk
+    const int jj = b8 & 3;                                          // mask byte inside the block
+    if (jj == 0) block_stream<C, BITS>(w.c, blk, st);               // once per block
     const int gi = C::NGC == 2 ? h : 0;                             // quantisation group of this stage
     const _Float16 sh = (_Float16)(wok ? w.s[gi] : 0.f);
     const h2_t s2 = {sh, sh};
     const uint32_t nz = 0x80808080u - ((w.z >> (8 * gi)) & 0xFFu) * 0x01010101u;
-#pragma unroll
-    for (int hb = 0; hb < 2; ++hb) {                              // two mask bytes = 16 columns
-      const int jj = (qq & 1) * 2 + hb;                           // mask byte inside the block, 0..3
-      uint32_t p0, p1, b0, b1;
-      if (BITMAP) {
-        const uint32_t mw = w.m[blk];
-        const uint32_t r = jj == 0 ? 0u : (uint32_t)__builtin_popcount(mw & ((1u << (8 * jj)) - 1u));
-        const uint32_t cwin = jj == 0 ? st[0] : window<C::NW>(st, r * C::SB);
-        if (C::SB == 4) {
-          p0 = bias_pool(cwin & 0x0F0F0F0Fu, nz);
-          p1 = bias_pool((cwin >> 4) & 0x0F0F0F0Fu, nz);
-        } else {
-          const uint32_t lo16 = cwin & 0xFFFFu;
-          const uint32_t t2 = (lo16 << 14) | lo16;
-          p0 = bias_pool(t2 & 0x03030303u, nz);
-          p1 = bias_pool((t2 >> 4) & 0x03030303u, nz);
-        }
-        b0 = perm(p1, p0, selq[hb].x);
-        b1 = perm(p1, p0, selq[hb].y);
-      } else if (C::SB == 4) {                                     // dense 4-bit, or 3-bit widened to nibbles
-        const uint32_t cwin = st[jj];
-        p0 = bias_pool(cwin & 0x0F0F0F0Fu, nz);                    // even columns
-        p1 = bias_pool((cwin >> 4) & 0x0F0F0F0Fu, nz);             // odd columns
-        b0 = perm(p1, p0, 0x05010400u);
-        b1 = perm(p1, p0, 0x07030602u);
-      } else {                                                     // dense 2-bit: 16 codes per dword
-        const uint32_t lo16 = (st[jj >> 1] >> (16 * (jj & 1))) & 0xFFFFu;
+    uint32_t p0, p1, b0, b1;
+    if (BITMAP) {
+      const uint32_t mw = w.m[blk];
+      const uint32_t r = jj == 0 ? 0u : (uint32_t)__builtin_popcount(mw & ((1u << (8 * jj)) - 1u));
+      const uint32_t cwin = jj == 0 ? st[0] : window<C::NW>(st, r * C::SB);
+      if (C::SB == 4) {
+        p0 = bias_pool(cwin & 0x0F0F0F0Fu, nz);
+        p1 = bias_pool((cwin >> 4) & 0x0F0F0F0Fu, nz);
+      } else {
+        const uint32_t lo16 = cwin & 0xFFFFu;
         const uint32_t t2 = (lo16 << 14) | lo16;
-        p0 = bias_pool(t2 & 0x03030303u, nz);                      // c0 c4 c1 c5
-        p1 = bias_pool((t2 >> 4) & 0x03030303u, nz);               // c2 c6 c3 c7
-        b0 = perm(p1, p0, 0x06040200u);
-        b1 = perm(p1, p0, 0x07050301u);
+        p0 = bias_pool(t2 & 0x03030303u, nz);
+        p1 = bias_pool((t2 >> 4) & 0x03030303u, nz);
       }
-      ((uint4*)dst)[hb] = bytes_to_halfs(b0, b1, s2);
+      b0 = perm(p1, p0, sel.x);
+      b1 = perm(p1, p0, sel.y);
+    } else if (C::SB == 4) {                                       // dense 4-bit, or 3-bit widened to nibbles
+      const uint32_t cwin = st[jj];
+      p0 = bias_pool(cwin & 0x0F0F0F0Fu, nz);                      // even columns
+      p1 = bias_pool((cwin >> 4) & 0x0F0F0F0Fu, nz);               // odd columns
+      b0 = perm(p1, p0, 0x05010400u);
+      b1 = perm(p1, p0, 0x07030602u);
+    } else {                                                       // dense 2-bit: 16 codes per dword
+      const uint32_t lo16 = (st[jj >> 1] >> (16 * (jj & 1))) & 0xFFFFu;
+      const uint32_t t2 = (lo16 << 14) | lo16;
+      p0 = bias_pool(t2 & 0x03030303u, nz);                        // c0 c4 c1 c5
+      p1 = bias_pool((t2 >> 4) & 0x03030303u, nz);                 // c2 c6 c3 c7
+      b0 = perm(p1, p0, 0x06040200u);
+      b1 = perm(p1, p0, 0x07050301u);
     }
+    *(uint4*)dst = bytes_to_halfs(b0, b1, s2);
   };
 
-  // ---- prologue: chunks 0 and 1 into registers; stage 0 into buffer 0
-  dma_x(0, 0);
-  load_chunk(0, wA); load_chunk(1, wB);
-  __syncthreads();                                                // selector table visible
-#pragma unroll
-  for (int qq = 0; qq < 4; ++qq) {
-    uint2 sel[2];
-    fetch_sel(wA, 0, qq, sel);
-    store_w_quarter(0, wA, 0, 0, qq, sel);
-  }
-  uint2 selq[2];                                                  // selectors of the next quarter to decode
-  fetch_sel(wA, 1, 0, selq);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-
-  // One stage: matrix-core work on buffer s % 2 while stage s + 1 moves into the other buffer:
-  // its activations by direct copies issued at the top, its weights (half HD of chunk wd)
-  // decoded a quarter per phase between the MFMAs.  The selectors of the following quarter
-  // (after the last one: of quarter 0 of half HN of chunk wn) are fetched a phase early.  With
-  // LOADW the 128-column weight chunk `cl` is loaded into wl, first touched seven phases later;
-  // these loads are issued after the direct copies, so the wait before the barrier can leave
-  // them in flight.  No branches inside.
-  auto stage = [&](int s, auto loadw_tag, WChunk& wd, auto hd_tag, const WChunk& wn, auto hn_tag, WChunk& wl, int cl) {
-    constexpr bool LOADW = decltype(loadw_tag)::value;
-    constexpr int HD = decltype(hd_tag)::value, HN = decltype(hn_tag)::value;
-    const int buf = s & 1;
+  // fragment registers, two sets; set 0 of the next stage is loaded at the end of the current one
+  v8h af[2][4], bf[2][4];
+  auto read_frags = [&](int buf, int kk, int set) {
     const uint8_t* xb = (const uint8_t*)Xs + (size_t)buf * GB_XBUF + (128 * wt + (lane & 31)) * 128;
     const _Float16* wb = Ws + (size_t)buf * GB_R * GB_P + (128 * wr + (lane & 31)) * GB_P + 8 * (lane >> 5);
-    v8h af[2][4], bf[2][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) af[0][i] = *(const v8h*)(xb + 4096 * i + xpc[0]);
+    for (int i = 0; i < 4; ++i) af[set][i] = *(const v8h*)(xb + 4096 * i + xpc[kk]);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) bf[0][j] = *(const v8h*)(wb + 32 * j * GB_P);
-    dma_x(s + 1 < nst ? s + 1 : nst - 1, buf ^ 1);
-    if (LOADW) load_chunk(cl, wl);
-    __builtin_amdgcn_sched_barrier(0);
+    for (int j = 0; j < 4; ++j) bf[set][j] = *(const v8h*)(wb + 32 * j * GB_P + 16 * kk);
+  };
+
+  // ---- prologue: chunk 0 into registers and stage 0 into buffer 0; then, in the order every
+  // stage leaves them, the copies of stage 1 and the loads of chunk 1
+  dma_x(0, 0);
+  load_chunk(0, wA);
+  __syncthreads();                                                // selector table visible
+#pragma unroll
+  for (int b8 = 0; b8 < 8; ++b8) store_w_byte(0, wA, 0, 0, b8, fetch_sel(wA, 0, b8));
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  read_frags(0, 0, 0);
+  dma_x(nst > 1 ? 1 : 0, 1);
+  load_chunk(1, wB);
+  uint2 selc[3];                                                  // selectors of the mask bytes decoded next
+#pragma unroll
+  for (int i = 0; i < 3; ++i) selc[i] = fetch_sel(wA, 1, i);
+
+  // One stage = four phases of 16 MFMAs on buffer s % 2.  Phases 0-2 also decode the weights of
+  // stage s + 1 (half HD of chunk wd; mask bytes 0-2, 3-5, 6-7) into the other buffer between
+  // their MFMAs, fetching the selectors of the following phase (at the end: of bytes 0-2 of half
+  // HN of chunk wn) a phase early.  Phase 3 first waits for the direct copies of stage s + 1
+  // (issued a stage ago) and passes the barrier, then starts the fragment reads of stage s + 1,
+  // the direct copies of stage s + 2 and, with LOADW, the loads of weight chunk `cl`, and only
+  // then issues its 16 MFMAs from registers: the LDS latency of the next stage hides under them.
+  // PREVW says whether the previous stage loaded a chunk (its loads follow the copies being
+  // waited for and may stay in flight).  No branches inside.
+  constexpr int NB0 = 3, NB1 = 3;                                 // mask bytes decoded in phases 0 and 1
+  auto stage = [&](int s, auto loadw_tag, auto prevw_tag, WChunk& wd, auto hd_tag, const WChunk& wn, auto hn_tag,
+                   WChunk& wl, int cl) {
+    constexpr bool LOADW = decltype(loadw_tag)::value, PREVW = decltype(prevw_tag)::value;
+    constexpr int HD = decltype(hd_tag)::value, HN = decltype(hn_tag)::value;
+    const int buf = s & 1;
 #pragma unroll
     for (int kk = 0; kk < GB_K / 16; ++kk) {
       const int c = kk & 1, n = c ^ 1;
-      if (kk + 1 < GB_K / 16) {
+      if (kk < 3) {
+        read_frags(buf, kk + 1, n);
+        uint2 seln[3];
+        if (kk == 0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) af[n][i] = *(const v8h*)(xb + 4096 * i + xpc[kk + 1 < 4 ? kk + 1 : 3]);
+          for (int i = 0; i < NB1; ++i) seln[i] = fetch_sel(wd, HD, NB0 + i);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) bf[n][j] = *(const v8h*)(wb + 32 * j * GB_P + 16 * (kk + 1));
+          for (int i = 0; i < NB0; ++i) store_w_byte(s + 1, wd, HD, buf ^ 1, i, selc[i]);
+        } else if (kk == 1) {
+#pragma unroll
+          for (int i = 0; i < 8 - NB0 - NB1; ++i) seln[i] = fetch_sel(wd, HD, NB0 + NB1 + i);
+#pragma unroll
+          for (int i = 0; i < NB1; ++i) store_w_byte(s + 1, wd, HD, buf ^ 1, NB0 + i, selc[i]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < NB0; ++i) seln[i] = fetch_sel(wn, HN, i);
+#pragma unroll
+          for (int i = 0; i < 8 - NB0 - NB1; ++i) store_w_byte(s + 1, wd, HD, buf ^ 1, NB0 + NB1 + i, selc[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < 3; ++i) selc[i] = seln[i];
+      } else {
+        // the direct copies of stage s + 1 must have landed before the barrier publishes them
+        if (PREVW) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NWL) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        read_frags(buf ^ 1, 0, 0);
+        dma_x(s + 2 < nst ? s + 2 : nst - 1, buf);
+        if (LOADW) load_chunk(cl, wl);
       }
-      uint2 seln[2];
-      if (kk + 1 < GB_K / 16) fetch_sel(wd, HD, kk + 1, seln); else fetch_sel(wn, HN, 0, seln);
-      store_w_quarter(s + 1, wd, HD, buf ^ 1, kk, selq);
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[c][i], bf[c][j], acc[i][j], 0, 0, 0);
-      selq[0] = seln[0]; selq[1] = seln[1];
+      if (kk < 3) {
 #pragma unroll
-      for (int g = 0; g < 16; ++g) {                              // one MFMA, then a slice of the decode
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+        for (int g = 0; g < 16; ++g) {                            // one MFMA, then a slice of the decode
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (kk == 2) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+          else __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    // the direct copies of stage s + 1 must have landed before the barrier publishes them
-    if (LOADW) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NWL) : "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
   };
   // Four stages per trip (two chunks): stage 2p decodes the upper half of chunk p, stage 2p+1
   // the lower half of chunk p+1 and loads chunk p+2 into the registers chunk p has left.
@@ -402,11 +421,15 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   using H0 = std::integral_constant<int, 0>; using H1 = std::integral_constant<int, 1>;
   for (int s = 0; s < nst; s += 4) {
     const int p = s >> 1;
-    stage(s,     Fl{}, wA, H1{}, wB, H0{}, wA, 0);
-    stage(s + 1, T{},  wB, H0{}, wB, H1{}, wA, p + 2);
-    stage(s + 2, Fl{}, wB, H1{}, wA, H0{}, wB, 0);
-    stage(s + 3, T{},  wA, H0{}, wA, H1{}, wB, p + 3);
+    stage(s,     Fl{}, T{},  wA, H1{}, wB, H0{}, wA, 0);
+    stage(s + 1, T{},  Fl{}, wB, H0{}, wB, H1{}, wA, p + 2);
+    stage(s + 2, Fl{}, T{},  wB, H1{}, wA, H0{}, wB, 0);
+    stage(s + 3, T{},  Fl{}, wA, H0{}, wA, H1{}, wB, p + 3);
   }
+  // the last stage issued copies of a stage that does not exist: let them land before the
+  // epilogue reuses LDS
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
 
   const int tok0 = t0 + 128 * wt, row0 = r0 + 128 * wr;
   if (a.ydt == CBK_F32) gb_epilogue<CBK_F32>(a, acc, smem, lane, wave, tok0, row0);
