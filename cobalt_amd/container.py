@@ -1,0 +1,114 @@
+"""CBK1 directories: `manifest.json` plus one `.bin` per decoder layer, each a concatenation of
+256-byte aligned arrays that are, byte for byte, what the kernels read (reference:
+docs/FORMAT.md:1-37 container, :126-151 fused matrices and `alias_of`; writer
+src/cobaltkernel/pack_cobalt.py:390-505; loader src/cobaltkernel/runner.py:413-484).
+
+Reading is offset-driven: every matrix entry of the manifest names its blob and the offset and
+length of each of its arrays, so row-fused matrices and the `alias_of` entries that point into
+them need no special case.  A layer's blob is loaded once; the PackedMatrix of every matrix in
+it is a view (offset table) onto that one tensor.  On disk the rows are in the reference's
+row-major order; `to_tiled()` reorders them for the decode kernel after the move to the GPU.
+"""
+from __future__ import annotations
+
+import json
+import os
+from typing import Dict, List, Optional, Tuple
+
+import numpy as np
+import torch
+
+from . import format as F
+
+FORMAT_NAME = "CBK1"
+FORMAT_VERSION = 1
+
+
+def _entry(pm: F.PackedMatrix, blob_name: str, base: Dict[str, int]) -> dict:
+    arrays = {}
+    for name in ("data", "row_off", "scale", "zero", "col_scale"):
+        if name in pm.offs and (name != "col_scale" or pm.cs_rows):
+            arrays[name] = {"off": base[name], "bytes": int(pm.array(name).numel() * pm.array(name).element_size())}
+    e = {"K": pm.K, "N": pm.N, "G": pm.G, "layout": pm.layout, "layout_name": F.LAYOUT_NAME[pm.layout],
+         "cs_rows": pm.cs_rows, "n_survivors": pm.n_survivors, "stream_bytes": pm.stream_bytes(),
+         "bpw": pm.bpw(), "blob": blob_name, "arrays": arrays}
+    if pm.layout in (F.BLKC, F.DENSEB) or pm.group != 128:
+        e.update(bits=pm.bits, group=pm.group, keep=pm.keep)       # the extension layouts carry their parameters
+    if pm.cs_rows == 3:
+        e["cs_splits"] = list(pm.cs_splits)
+    return e
+
+
+def write_container(path: str, layers: List[Dict[str, F.PackedMatrix]], config: Optional[dict] = None) -> dict:
+    """Write `layers[i][name]` (row-major PackedMatrix objects) as layer_%02d.bin + manifest.json.
+    Returns the manifest."""
+    os.makedirs(path, exist_ok=True)
+    manifest = {"format": FORMAT_NAME, "version": FORMAT_VERSION, "config": dict(config or {}), "layers": []}
+    for li, mats in enumerate(layers):
+        blob_name = f"layer_{li:02d}.bin"
+        pos = 0
+        entries = {}
+        with open(os.path.join(path, blob_name), "wb") as f:
+            for name, pm in mats.items():
+                if pm.tiled:
+                    raise ValueError(f"{name}: write the row-major order; the tiled order is a load-time transform")
+                base = {}
+                for an in ("data", "row_off", "scale", "zero", "col_scale"):
+                    if an not in pm.offs or (an == "col_scale" and not pm.cs_rows):
+                        continue
+                    pad = F._align(pos, F.ARR_ALIGN) - pos
+                    f.write(b"\0" * pad)
+                    pos += pad
+                    raw = pm.array(an).contiguous().view(torch.uint8).cpu().numpy().tobytes()
+                    base[an] = pos
+                    f.write(raw)
+                    pos += len(raw)
+                entries[name] = _entry(pm, blob_name, base)
+            f.write(b"\0" * (F._align(pos, F.ARR_ALIGN) - pos))
+        manifest["layers"].append(entries)
+    with open(os.path.join(path, "manifest.json"), "w") as f:
+        json.dump(manifest, f, indent=1)
+    return manifest
+
+
+def matrix_from_entry(e: dict, blob: torch.Tensor) -> F.PackedMatrix:
+    """PackedMatrix view of one manifest entry onto its (already loaded) blob."""
+    layout = int(e["layout"])
+    bits, group, keep = F.canon(layout, e.get("bits"), e.get("group"), e.get("keep"))
+    a = e["arrays"]
+    offs = {k: int(v["off"]) for k, v in a.items()}
+    K, N = int(e["K"]), int(e["N"])
+    data_bytes = int(a["data"]["bytes"]) - F.BLOB_TAIL
+    zero = blob[offs["zero"]: offs["zero"] + int(a["zero"]["bytes"])]
+    flags = F.FLAG_ZERO_LE_128 if int(zero.max()) <= 128 else 0
+    return F.PackedMatrix(blob, offs, K, N, layout, bits, group, keep, int(e.get("cs_rows", 0)),
+                          tuple(e.get("cs_splits", (0, 0))), data_bytes, int(e.get("n_survivors", 0)), flags=flags)
+
+
+def read_container(path: str, device="cpu", include_aliases: bool = True) -> Tuple[dict, List[Dict[str, F.PackedMatrix]]]:
+    """(manifest, layers) with every blob read once and placed on `device`."""
+    with open(os.path.join(path, "manifest.json")) as f:
+        manifest = json.load(f)
+    if manifest.get("format") != FORMAT_NAME:
+        raise ValueError(f"{path}: not a {FORMAT_NAME} directory")
+    blobs: Dict[str, torch.Tensor] = {}
+    layers = []
+    for entries in manifest["layers"]:
+        mats = {}
+        for name, e in entries.items():
+            if e.get("alias_of") and not include_aliases:
+                continue
+            bn = e["blob"]
+            if bn not in blobs:
+                raw = np.fromfile(os.path.join(path, bn), dtype=np.uint8)
+                blobs[bn] = torch.from_numpy(raw).to(device)
+            mats[name] = matrix_from_entry(e, blobs[bn])
+        layers.append(mats)
+    return manifest, layers
+
+
+def total_stream_bytes(manifest: dict) -> int:
+    """Weight bytes one pass over the model streams; entries with `alias_of` are views into a
+    fused matrix and are not counted twice (docs/FORMAT.md:146-151)."""
+    return sum(int(e["stream_bytes"]) for entries in manifest["layers"] for e in entries.values()
+               if not e.get("alias_of"))
