@@ -244,7 +244,6 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
       w.s[1] = h2f(m.scale[mi + meta_step]);
     }
   };
-  constexpr int NWL = FASTD ? (BITMAP ? 1 : 0) + C::NL / 4 + 2 * C::NGC : 0;   // vector loads of one load_chunk
 
   // selectors of mask byte b8 (0..7) of half h of a chunk (bitmap layouts only)
   auto fetch_sel = [&](const WChunk& w, int h, int b8) -> uint2 {
@@ -358,12 +357,10 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   // (issued a stage ago) and passes the barrier, then starts the fragment reads of stage s + 1,
   // the direct copies of stage s + 2 and, with LOADW, the loads of weight chunk `cl`, and only
   // then issues its 16 MFMAs from registers: the LDS latency of the next stage hides under them.
-  // PREVW says whether the previous stage loaded a chunk (its loads follow the copies being
-  // waited for and may stay in flight).  No branches inside.
+  // No branches inside.
   constexpr int NB0 = 3, NB1 = 3;                                 // mask bytes decoded in phases 0 and 1
-  auto stage = [&](int s, auto loadw_tag, auto prevw_tag, WChunk& wd, auto hd_tag, const WChunk& wn, auto hn_tag,
-                   WChunk& wl, int cl) {
-    constexpr bool LOADW = decltype(loadw_tag)::value, PREVW = decltype(prevw_tag)::value;
+  auto stage = [&](int s, auto loadw_tag, WChunk& wd, auto hd_tag, const WChunk& wn, auto hn_tag, WChunk& wl, int cl) {
+    constexpr bool LOADW = decltype(loadw_tag)::value;
     constexpr int HD = decltype(hd_tag)::value, HN = decltype(hn_tag)::value;
     const int buf = s & 1;
 #pragma unroll
@@ -392,8 +389,10 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
         for (int i = 0; i < 3; ++i) selc[i] = seln[i];
       } else {
         // the direct copies of stage s + 1 must have landed before the barrier publishes them
-        if (PREVW) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NWL) : "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // (the weight chunk loads of the previous stage wait here as well: they were issued a
+        // whole stage ago, and counting them out of the wait would rest on how many load
+        // instructions the compiler keeps)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         read_frags(buf ^ 1, 0, 0);
         dma_x(s + 2 < nst ? s + 2 : nst - 1, buf);
@@ -421,10 +420,10 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   using H0 = std::integral_constant<int, 0>; using H1 = std::integral_constant<int, 1>;
   for (int s = 0; s < nst; s += 4) {
     const int p = s >> 1;
-    stage(s,     Fl{}, T{},  wA, H1{}, wB, H0{}, wA, 0);
-    stage(s + 1, T{},  Fl{}, wB, H0{}, wB, H1{}, wA, p + 2);
-    stage(s + 2, Fl{}, T{},  wB, H1{}, wA, H0{}, wB, 0);
-    stage(s + 3, T{},  Fl{}, wA, H0{}, wA, H1{}, wB, p + 3);
+    stage(s,     Fl{}, wA, H1{}, wB, H0{}, wA, 0);
+    stage(s + 1, T{},  wB, H0{}, wB, H1{}, wA, p + 2);
+    stage(s + 2, Fl{}, wB, H1{}, wA, H0{}, wB, 0);
+    stage(s + 3, T{},  wA, H0{}, wA, H1{}, wB, p + 3);
   }
   // the last stage issued copies of a stage that does not exist: let them land before the
   // epilogue reuses LDS
