@@ -2,9 +2,10 @@
 //
 // Workgroup tile 256 tokens x 256 weight rows, 64 input columns per stage, four wavefronts
 // each owning a 128 x 128 sub-tile (4 x 4 blocks of v_mfma_f32_32x32x16_f16, 256 accumulator
-// registers), one wavefront per SIMD.  Both operands are double-buffered in LDS (147 KB):
-// while the matrix cores work on stage s, the same wavefronts dequantise the weights of
-// stage s + 1 into the other buffer and copy the activation tile there.
+// registers), one wavefront per SIMD.  Both operands are double-buffered in LDS (64 KB of
+// activations, 72 KB of weights): while the matrix cores work on stage s, the same wavefronts
+// dequantise the weights of stage s + 1 into the other buffer, and the activation tile is
+// copied there from global memory without passing through registers.
 //
 // Operands.  The activation side is X' = fp16(x * col_scale), written once per call into the
 // caller's workspace by a small elementwise kernel (bf16 inputs are widened exactly; the
