@@ -44,7 +44,7 @@ MFMA_PEAK_TFLOPS = 2500.0          # dense bf16 / f16 MFMA peak of MI355X
 # HBM bytes per launch of the decode kernel (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, scaled by
 # the same counters read for a device-to-device copy of known size), keyed by
 # (workload, launch grouping, M); filled from the runs summarised under profiles/.
-MEASURED_TRAFFIC = {("mistral7b", "phase", 1): 22291866}
+MEASURED_TRAFFIC = {("mistral7b", "phase", 1): 22333466}
 
 
 def algorithmic_bytes(pm, M, e_x=2, e_y=2):
@@ -58,26 +58,42 @@ def cpu_baseline(pms, shapes, xs, ys, M, budget_s=20.0):
     from oracle import cbk_ref_c as C
     nthreads = min(16, os.cpu_count() or 1)
     C.set_threads(nthreads)
-    total_bytes, total_t, worst, done = 0, 0.0, 0.0, []
+    total_bytes, total_t, worst, done, calls = 0, 0.0, 0.0, [], []
     t_stop = time.time() + budget_s
     for pm, (name, K, N) in zip(pms, shapes):
         if done and time.time() > t_stop:
             break
-        # one pass per matrix: the C decoder does ~15 ns of work per weight per thread
         pk = dict(data=pm.array("data").cpu().numpy(), scale=pm.array("scale").cpu().numpy().reshape(K, -1),
                   zero=pm.array("zero").cpu().numpy().reshape(K, -1))
         cs = pm.array("col_scale").cpu().numpy().reshape(pm.cs_rows, N) if pm.cs_rows else None
         x = xs[N].float().cpu().numpy()
+        call = lambda pk=pk, K=K, N=N, pm=pm, x=x, cs=cs: C.forward(
+            pk, K, N, pm.layout, x, col_scale=cs, bits=pm.bits, group=pm.group, keep_per_block=pm.keep or None)
         t0 = time.perf_counter()
-        y = C.forward(pk, K, N, pm.layout, x, col_scale=cs, bits=pm.bits, group=pm.group, keep_per_block=pm.keep or None)
+        y = call()
         total_t += time.perf_counter() - t0
         total_bytes += algorithmic_bytes(pm, M)
         got = ys[name].float().cpu().numpy()
         worst = max(worst, float(np.linalg.norm(got - y) / np.linalg.norm(y)))
         done.append(name)
+        calls.append((call, algorithmic_bytes(pm, M)))
+    # further passes over the same matrices until about one second of wall time on all threads
+    # (10-30 s of CPU work); the first, checked pass counts too
+    passes = 1
+    more = max(0, min(40, int(1.0 / max(total_t, 1e-3))))
+    for _ in range(more):
+        if time.time() > t_stop:
+            break
+        for call, nbytes in calls:
+            t0 = time.perf_counter()
+            call()
+            total_t += time.perf_counter() - t0
+            total_bytes += nbytes
+        passes += 1
     return dict(value=round(total_bytes / total_t / 1e9, 3), unit="GB/s", cores=nthreads, kind="port",
                 sample=f"C oracle dequantise-then-matmul (OpenMP, {nthreads} threads) over {'+'.join(done)} of the first "
-                       f"layer set, one pass, {total_t:.2f} s; same packed bytes as the GPU run",
+                       f"layer set, {passes} passes, {total_t:.2f} s wall = {total_t * nthreads:.0f} core-seconds; "
+                       f"same packed bytes as the GPU run",
                 gpu_vs_oracle_rel_fro=worst)
 
 
