@@ -19,9 +19,14 @@
 // the A operand therefore carry (activation row, quarter, digit) variants that are non-zero
 // in one quarter only, and the 16x16 result keeps the groups apart.  One persistent workgroup
 // of sixteen wavefronts per CU owns a contiguous range of row tiles; a tile is cut into up
-// to 16 column parts and the (tile, part) items are dealt round-robin to the wavefronts, which
-// run without a barrier per tile: the partial sums of a tile meet in an LDS slot and the
-// wavefront that arrives last adds them in part order, so results are run-to-run identical.
+// to 16 column parts; a wavefront's first three (tile, part) items are fixed, the later ones it
+// takes from a counter in LDS.  There is no barrier per tile: the partial sums of a tile meet
+// in an LDS slot and the wavefront that arrives last adds them in part order, so results are
+// run-to-run identical and do not depend on which wavefront summed which item.
+// For 2 <= M <= 4 the headline configurations put the lane quarters on the four 32-column
+// blocks of one chunk instead of on four chunks (see block_split_capable below), so that
+// every MFMA serves all activation rows; sums are formed in the same order as for M = 1, so
+// a row's result does not depend on M.
 // The activation digits and the byte-permute selector table live in LDS for the whole launch.
 //
 // Expansion of the bitmap.  For one mask byte (8 columns, r survivors before it in its
@@ -68,11 +73,11 @@ struct GvMat {
   int nS;                  // macro-steps per tile = ceil(N / 512)
   int cost0;               // sum of ntiles * nS over the matrices before this one
   int spi, sk;             // macro-steps per work item, work items per tile
-  // branch-free addressing of either byte order: row k starts at data + (k >> rsh) * row_a +
-  // (k & rmask) * 16 and its 16-byte units are ustride apart; the scale / zero entry of
-  // (k, g) has index ((k >> rsh) * G + g) * (rmask + 1) + (k & rmask)
-  int rsh, rmask;
-  uint32_t row_a, ustride;
+  // branch-free addressing of either byte order.  Row r of tile t starts at
+  // data + t * tile_a + r * lane_mul and its 16-byte units are 1 << ush bytes apart; the scale /
+  // zero entry of (row, group g) has index t * 16 * G + r * sz_mul + (g << csh).
+  uint32_t tile_a, lane_mul, sz_mul;
+  int ush, csh;
 };
 
 // What every wavefront needs before it can find its work: small, first in the kernel
@@ -97,6 +102,19 @@ __host__ __device__ constexpr int frag_col(int bits, bool dense, int bi) {
   if (!dense) return bi;
   if (bits == 2) return (bi >> 2) + 4 * (bi & 3);                                 // byte 4k+j <- column k+4j
   return ((bi >> 3) << 3) + 2 * (bi & 3) + ((bi >> 2) & 1);                       // even | odd per 8
+}
+
+// Two ways to lay a macro-step (16 rows x 512 columns) on the 16x16x64 MFMA.
+//  * quarter-per-chunk: lane quarter kq decodes chunk 4S + kq; one MFMA adds four different
+//    quantisation groups, so the A rows are (quarter, digit) and one activation row needs one
+//    pass.  Used for M = 1 and for every configuration below that cannot use the other way.
+//  * quarter-per-block: lane quarter kq decodes block kq (32 columns) of each of the four
+//    chunks; one MFMA covers 64 columns of a single group, the A rows are (activation row,
+//    digit), and up to four activation rows share every MFMA.  Needs group 128 and a block's
+//    code bits to be 4, 8 or 16 whole bytes.
+__host__ __device__ constexpr bool block_split_capable(int bits, int keep, int grp) {
+  const int cb = (keep == 0 ? 32 : keep) * bits;
+  return grp == 128 && bits != 3 && (cb == 32 || cb == 64 || cb == 128);
 }
 
 // ------------------------------------------------------------------ activation prep
@@ -173,6 +191,70 @@ __device__ inline void stage_convert(const XLoad& r, bool has_cs, int xdt, int N
   if (c16 < 4) delta[row * (NCH + 4) + NCH + c16] = 0.f;          // chunks past N
 }
 
+// ------------------------------------------------------------------ one 32-column block
+// mask bytes of a block and the number of survivors before each of them
+template <class C>
+__device__ inline void split_mask(uint32_t mw, uint32_t (&mb)[4], uint32_t (&rk)[4]) {
+  if (!C::DENSE) {
+    mb[0] = mw & 0xFFu; mb[1] = __builtin_amdgcn_ubfe(mw, 8, 8); mb[2] = __builtin_amdgcn_ubfe(mw, 16, 8); mb[3] = mw >> 24;
+    rk[0] = 0; rk[1] = (uint32_t)__builtin_popcount(mb[0]);
+    rk[2] = rk[1] + (uint32_t)__builtin_popcount(mb[1]); rk[3] = rk[2] + (uint32_t)__builtin_popcount(mb[2]);
+  }
+}
+
+// ranks and table reads of one block
+template <class C>
+__device__ inline void fetch_selectors(uint32_t mw, const uint2* lut, uint32_t l16, uint32_t (&rk)[4], uint2 (&sel4)[4]) {
+  uint32_t mb[4];
+  split_mask<C>(mw, mb, rk);
+  if (!C::DENSE) {
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) sel4[jj] = lut[mb[jj] * LUT_LANES + l16];
+  }
+}
+
+// Sixteen columns (half `half` of the block whose code stream is st) as signed bytes q - zero,
+// pruned columns 0: the B operand of one MFMA.
+// The selectors of the block's four mask bytes (sel) were read from the table earlier, so that
+// the LDS latency is not waited for here.
+template <class C, int BITS>
+__device__ inline void decode_half(const uint32_t (&st)[C::NW], const uint32_t (&rk)[4], const uint2 (&sel4)[4],
+                                   uint32_t nz, int half, uint32_t (&bfrag)[4]) {
+#pragma unroll
+  for (int jj2 = 0; jj2 < 2; ++jj2) {
+    const int jj = 2 * half + jj2;                       // mask byte inside the block
+    uint32_t p0, p1;
+    if (C::DENSE) {
+      if (C::SB == 4) {
+        const uint32_t w = st[jj];
+        p0 = bias_pool(w & 0x0F0F0F0Fu, nz);
+        p1 = bias_pool((w >> 4) & 0x0F0F0F0Fu, nz);
+      } else {                                           // 2-bit: 16 codes per dword
+        const uint32_t w = st[half] >> (4 * jj2);
+        p0 = bias_pool(w & 0x03030303u, nz);
+        p1 = bias_pool((w >> 2) & 0x03030303u, nz);
+      }
+      bfrag[2 * jj2] = p0; bfrag[2 * jj2 + 1] = p1;
+    } else {
+      uint32_t w;
+      if (jj == 0) w = st[0];
+      else w = window<C::NW>(st, rk[jj] * C::SB);
+      if (C::SB == 4) {
+        p0 = bias_pool(w & 0x0F0F0F0Fu, nz);
+        p1 = bias_pool((w >> 4) & 0x0F0F0F0Fu, nz);
+      } else {
+        const uint32_t lo16 = w & 0xFFFFu;
+        const uint32_t t2 = (lo16 << 14) | lo16;
+        p0 = bias_pool(t2 & 0x03030303u, nz);
+        p1 = bias_pool((t2 >> 4) & 0x03030303u, nz);
+      }
+      const uint2 sel = sel4[jj];
+      bfrag[2 * jj2] = perm(p1, p0, sel.x);
+      bfrag[2 * jj2 + 1] = perm(p1, p0, sel.y);
+    }
+  }
+}
+
 // ------------------------------------------------------------------ the decode kernel
 template <class C>
 struct Loads {
@@ -185,8 +267,10 @@ struct Loads {
 template <int BITS, int KEEP, int GRP, int MP>
 __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
   using C = Cfg<BITS, KEEP, GRP, MP>;
+  constexpr bool QB = MP == 4 && block_split_capable(BITS, KEEP, GRP);
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // in a scalar register: positions are scalar work
   uint2* lut = (uint2*)smem;
   uint8_t* zreg = smem + LUT_BYTES;
   int8_t* xq = (int8_t*)(zreg + ZERO_BYTES);
@@ -232,55 +316,117 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     const uint8_t* const m_data = m.data;
     const uint16_t* const m_scale = m.scale;
     const uint8_t* const m_zero = m.zero;
-    const int m_K = m.K, m_G = m.G, rsh = gm.rsh, rmask = gm.rmask, mmul = gm.rmask + 1;
-    const uint32_t row_a = gm.row_a, ustride = gm.ustride, code_u0 = m.code_off >> 4;
+    const int m_K = m.K, m_G = m.G, ush = gm.ush, csh = gm.csh;
+    const uint32_t tile_a = gm.tile_a, lane_mul = gm.lane_mul, sz_mul = gm.sz_mul, code_u0 = m.code_off >> 4;
     const int last_tile = t_hi - 1, last_S = nS - 1;
 
     // ---- issue the loads of one (tile, macro-step) position; out-of-range positions are clamped
+    // Everything that depends only on (tile, S) is scalar work; a lane adds a 32-bit offset.
     auto issue = [&](int tile, int S, Loads<C>& L) {
       tile = tile < last_tile ? tile : last_tile;
       S = S < last_S ? S : last_S;
-      int row = tile * 16 + wr;
-      row = row < m_K ? row : m_K - 1;
-      const uint8_t* rb = m_data + (size_t)(row >> rsh) * row_a + (size_t)(row & rmask) * 16;
-      int ch = 4 * S + kq;
-      ch = ch < NCH ? ch : NCH - 1;
+      const int S4 = 4 * S;
+      const int rlim = m_K - 1 - tile * 16;                         // rows past K repeat row K - 1
+      const uint32_t wrc = (uint32_t)(wr < rlim ? wr : rlim);
+      const uint32_t lane_off = __umul24(wrc, lane_mul);
+      const uint8_t* const tb = m_data + (size_t)tile * tile_a;
+      const size_t sz_t = (size_t)tile * (size_t)(16 * m_G);
+      const int klim = NCH - 1 - S4;                                // chunks past N repeat chunk NCH - 1
+      const uint32_t chl = (uint32_t)(kq < klim ? kq : klim);
+      if constexpr (QB) {
+        // block kq of the chunks 4S .. 4S+3: one mask dword and CB / 8 code bytes each
+        constexpr uint32_t BB = C::CB / 8;
+        const uint32_t voff_m = lane_off + (uint32_t)kq * 4u;
+        const uint32_t voff_c = lane_off + ((((uint32_t)kq * BB) >> 4) << ush) + (((uint32_t)kq * BB) & 15u);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          int chc = S4 + c;
+          chc = chc < NCH ? chc : NCH - 1;
+          if (!C::DENSE) L.mk[c] = *(const uint32_t*)(tb + ((size_t)chc << ush) + voff_m);
+          const uint8_t* cp = tb + ((size_t)(code_u0 + (uint32_t)chc * (C::CHB / 128)) << ush) + voff_c;
+          if (C::CB == 32) {
+            L.raw[c] = *(const uint32_t*)cp;
+          } else if (C::CB == 64) {
+            const uint2 v = *(const uint2*)cp;
+            L.raw[2 * c] = v.x; L.raw[2 * c + 1] = v.y;
+          } else {
+            const uint4 v = *(const uint4*)cp;
+            L.raw[4 * c] = v.x; L.raw[4 * c + 1] = v.y; L.raw[4 * c + 2] = v.z; L.raw[4 * c + 3] = v.w;
+          }
+        }
+        // zero point and scale of group 4S + kq; the other quarters fetch them from this lane
+        const size_t gs = sz_t + ((size_t)S4 << csh);
+        const uint32_t gv = __umul24(wrc, sz_mul) + (chl << csh);
+        L.zraw = (uint32_t)(m_zero + gs)[gv] | ((uint32_t)(m_scale + gs)[gv] << 8);
+        return;
+      }
+      const uint8_t* const sb = tb + ((size_t)S4 << ush);
       if (!C::DENSE) {
-        const uint4 v = *(const uint4*)(rb + (size_t)ch * ustride);
+        const uint4 v = *(const uint4*)(sb + (lane_off + (chl << ush)));
         L.mk[0] = v.x; L.mk[1] = v.y; L.mk[2] = v.z; L.mk[3] = v.w;
       }
       // code bits of the chunk: bit ch*CHB of the code plane, fetched as whole 16-byte units
-      const uint32_t u0 = code_u0 + (C::VEC16 ? (uint32_t)ch * (C::CHB / 128) : (((uint32_t)ch * C::CHB) >> 7));
+      if (C::VEC16) {
+        const uint8_t* const cb = tb + ((size_t)(code_u0 + (uint32_t)S4 * (C::CHB / 128)) << ush);
+        const uint32_t voff = lane_off + ((chl * (C::CHB / 128)) << ush);
 #pragma unroll
-      for (int i = 0; i < C::NL / 4; ++i) {
-        const uint4 v = *(const uint4*)(rb + (size_t)(u0 + i) * ustride);
-        L.raw[4 * i] = v.x; L.raw[4 * i + 1] = v.y; L.raw[4 * i + 2] = v.z; L.raw[4 * i + 3] = v.w;
-      }
-      const size_t mi0 = ((size_t)(row >> rsh) * m_G + (size_t)ch * C::NGC) * mmul + (row & rmask);
-      if (C::NGC == 1) {
-        L.zraw = m_zero[mi0];
-        L.sc[0] = m_scale[mi0];
+        for (int i = 0; i < C::NL / 4; ++i) {
+          const uint4 v = *(const uint4*)(cb + ((size_t)i << ush) + voff);
+          L.raw[4 * i] = v.x; L.raw[4 * i + 1] = v.y; L.raw[4 * i + 2] = v.z; L.raw[4 * i + 3] = v.w;
+        }
       } else {
-        L.zraw = (uint32_t)m_zero[mi0] | ((uint32_t)m_zero[mi0 + mmul] << 8);
-        L.sc[0] = m_scale[mi0];
-        L.sc[C::NGC - 1] = m_scale[mi0 + mmul];
+        const uint32_t u = (((uint32_t)S4 + chl) * (uint32_t)C::CHB) >> 7;
+        const uint32_t voff = lane_off + (u << ush);
+#pragma unroll
+        for (int i = 0; i < C::NL / 4; ++i) {
+          const uint4 v = *(const uint4*)(tb + ((size_t)(code_u0 + i) << ush) + voff);
+          L.raw[4 * i] = v.x; L.raw[4 * i + 1] = v.y; L.raw[4 * i + 2] = v.z; L.raw[4 * i + 3] = v.w;
+        }
+      }
+      const size_t gs = sz_t + ((size_t)(S4 * C::NGC) << csh);
+      const uint32_t gv = __umul24(wrc, sz_mul) + ((chl * C::NGC) << csh);
+      const uint8_t* const zp = m_zero + gs;
+      const uint16_t* const sp = m_scale + gs;
+      if (C::NGC == 1) {
+        L.zraw = zp[gv];
+        L.sc[0] = sp[gv];
+      } else {
+        const uint8_t* const zp1 = zp + ((size_t)1 << csh);
+        const uint16_t* const sp1 = sp + ((size_t)1 << csh);
+        L.zraw = (uint32_t)zp[gv] | ((uint32_t)zp1[gv] << 8);
+        L.sc[0] = sp[gv];
+        L.sc[C::NGC - 1] = sp1[gv];
       }
     };
 
-    // this wave's sequence of (tile, part, macro-step) positions: items wave, wave+16, ...
-    struct Pos { int tl, part, S; };
-    const int ntl = t_hi - t_lo;
-    const int dq_t = GV_WAVES / SK, dq_p = GV_WAVES % SK;
+    // This wave's sequence of (tile, part, macro-step) positions.  Its first three items are
+    // wave, wave + 16, wave + 32 (known without asking anybody, so that the first loads can go
+    // out before the workgroup has met at a barrier); every later item is the next one not yet
+    // taken, from a counter in LDS.  The wavefronts of a SIMD do not advance at the same pace
+    // (the oldest wins the issue arbitration), and with a fixed deal the slowest one would work
+    // through its last items alone, with nobody to hide its latencies.  Which wavefront sums
+    // which item does not enter the result.
+    struct Pos { int tl, part, S, k; };                            // k: items taken by this wavefront so far
+    constexpr int STATIC_ROUNDS = 3;
+    int* const next_item = cnt + h.nslot;
+    const uint32_t inv_sk = 65536u / (uint32_t)SK + 1u;           // it / SK == (it * inv_sk) >> 16 for it < 4096, SK <= 16
     auto advance = [&](Pos& p) -> bool {                           // false past the last position
       const int s_end = (p.part * spi + spi < nS) ? p.part * spi + spi : nS;
       if (p.S + 1 < s_end) { ++p.S; return true; }
-      p.tl += dq_t; p.part += dq_p;
-      if (p.part >= SK) { p.part -= SK; ++p.tl; }
+      ++p.k;
+      int it = wave + GV_WAVES * p.k;
+      if (p.k >= STATIC_ROUNDS) {
+        int v = 0;
+        if (lane == 0) v = atomicAdd(next_item, 1);
+        it = __builtin_amdgcn_readfirstlane(v);
+      }
+      p.tl = it < 4096 ? (int)(((uint32_t)it * inv_sk) >> 16) : it / SK;
+      p.part = it - p.tl * SK;
       p.S = p.part * spi;
-      return p.tl < ntl;
+      return it < nitems;
     };
-    Pos p0{wave / SK, wave % SK, (wave % SK) * spi};
-    bool v0 = p0.tl < ntl;
+    Pos p0{wave / SK, wave % SK, (wave % SK) * spi, 0};
+    bool v0 = wave < nitems;
     Pos p1 = p0; bool v1 = v0 && advance(p1);
     Pos p2 = p1; bool v2 = v1 && advance(p2);
     // The activation loads go out before the first weight loads: the weight prefetch of a whole
@@ -294,12 +440,13 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     // copying a buffer would wait for the loads that are still filling it.
     // Configurations with long code streams or four activation rows keep one step in flight
     // instead of two: three buffers would not fit the 128 registers of a 16-wavefront workgroup.
-    constexpr bool DEEP = C::NL <= 8 && MP < 4;
+    constexpr bool DEEP = C::NL <= 8 && (MP < 4 || QB);
     Loads<C> LA, LB, LC;
     issue(t_lo + p0.tl, p0.S, LA);
 
     // ---- stage: selector table and counters (once), activation digits and deltas of this matrix
     if (!first) __syncthreads();                                  // previous matrix fully consumed
+    if (tid == 0) *next_item = STATIC_ROUNDS * GV_WAVES;
     if (first) {
       if (tid < 256) {
         const uint2 e = make_selectors((uint32_t)tid, C::SEL_KIND);
@@ -335,6 +482,43 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
         for (int p = 0; p < MP; ++p) ysum[p] = 0.f;
       }
       if (DEEP) issue(t_lo + p2.tl, p2.S, tgt); else issue(t_lo + p1.tl, p1.S, tgt);
+      if constexpr (QB) {
+        const int a_m = wr >> 2;                                    // activation row of this lane's A row
+        uint32_t zs[4];                                             // zero | scale << 8 of the groups 4S .. 4S+3
+#pragma unroll
+        for (int c = 0; c < 4; ++c) zs[c] = (uint32_t)__shfl((int)cur.zraw, wr + 16 * c, 64);
+        const bool a_on = a_dig < NDIG && a_m < h.M;
+        const uint32_t a_base = xq_off + (uint32_t)((a_m * NDIG + a_dig) * N + kq * 32);
+        const int dm = kq < h.M ? kq : 0;                           // the activation row this quarter sums
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const int chunk = 4 * S + c;
+          const uint32_t aaddr = (a_on && chunk < NCH) ? a_base + (uint32_t)chunk * 128u : z_off;
+          uint32_t rkc[4];
+          uint2 selc[4];
+          fetch_selectors<C>(cur.mk[c], lut, l16, rkc, selc);
+          uint32_t st[C::NW];
+#pragma unroll
+          for (int k = 0; k < C::NW; ++k) st[k] = cur.raw[c * C::NW + k];
+          const uint32_t z = zs[c] & 0xFFu;
+          const uint32_t nz = 0x80808080u - z * 0x01010101u;
+          v4i acc = (v4i){0, 0, 0, 0};
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            const v4i av = *(const v4i*)(smem + aaddr + 16 * half);
+            uint32_t bfrag[4];
+            decode_half<C, BITS>(st, rkc, selc, nz, half, bfrag);
+            const v4i bv = (v4i){(int)bfrag[0], (int)bfrag[1], (int)bfrag[2], (int)bfrag[3]};
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bv, acc, 0, 0, 0);
+            asm("s_nop 1" : "+v"(acc));                             // see the other decode path
+          }
+          // the 128 columns of group `chunk` are complete: rows 4 kq .. 4 kq + 2 of the result
+          // are the three digit sums of activation row kq
+          const float dl = delta[dm * (NCH + 4) + chunk];           // 0 past the last chunk
+          const float f = fmaf((float)(acc[0] * 256 + acc[1]), 256.f, (float)acc[2]);
+          ysum[c] = fmaf(f, h2f((uint16_t)(zs[c] >> 8)) * dl, ysum[c]);
+        }
+      } else
       {
         const int chunk = 4 * S + kq;
         const bool valid = chunk < NCH;
@@ -352,60 +536,32 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 #pragma unroll
         for (int p = 0; p < MP; ++p) acc[p] = (v4i){0, 0, 0, 0};
 
+        // selector reads run one block ahead of the permutes; with one activation row the A
+        // fragment is read one MFMA ahead as well
+        constexpr bool APF = MP == 1;
+        uint32_t rkb[2][4];
+        uint2 selb[2][4];
+        fetch_selectors<C>(cur.mk[0], lut, l16, rkb[0], selb[0]);
+        v4i avn = (v4i){0, 0, 0, 0};
+        if (APF) avn = *(const v4i*)(smem + aaddr[0]);
 #pragma unroll
         for (int jb = 0; jb < 4; ++jb) {
+          if (jb < 3) fetch_selectors<C>(cur.mk[jb + 1], lut, l16, rkb[(jb + 1) & 1], selb[(jb + 1) & 1]);
           uint32_t st[C::NW];                                     // code stream of block jb
           block_stream<C, BITS>(cw, jb, st);
           const uint32_t z = (C::NGC == 1) ? cur.zraw : ((cur.zraw >> (8 * (jb >> 1))) & 0xFFu);
           const uint32_t nz = 0x80808080u - z * 0x01010101u;
-          const uint32_t mw = cur.mk[jb];
-          uint32_t mb[4], rk[4];
-          if (!C::DENSE) {
-            mb[0] = mw & 0xFFu; mb[1] = __builtin_amdgcn_ubfe(mw, 8, 8); mb[2] = __builtin_amdgcn_ubfe(mw, 16, 8); mb[3] = mw >> 24;
-            rk[0] = 0; rk[1] = (uint32_t)__builtin_popcount(mb[0]);
-            rk[2] = rk[1] + (uint32_t)__builtin_popcount(mb[1]); rk[3] = rk[2] + (uint32_t)__builtin_popcount(mb[2]);
-          }
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
-            uint32_t bfrag[4];
-#pragma unroll
-            for (int jj2 = 0; jj2 < 2; ++jj2) {
-              const int jj = 2 * half + jj2;                       // mask byte inside the block
-              uint32_t p0, p1;
-              if (C::DENSE) {
-                if (C::SB == 4) {
-                  const uint32_t w = st[jj];
-                  p0 = bias_pool(w & 0x0F0F0F0Fu, nz);
-                  p1 = bias_pool((w >> 4) & 0x0F0F0F0Fu, nz);
-                } else {                                           // 2-bit: 16 codes per dword
-                  const uint32_t w = st[half] >> (4 * jj2);
-                  p0 = bias_pool(w & 0x03030303u, nz);
-                  p1 = bias_pool((w >> 2) & 0x03030303u, nz);
-                }
-                bfrag[2 * jj2] = p0; bfrag[2 * jj2 + 1] = p1;
-              } else {
-                uint32_t w;
-                if (jj == 0) w = st[0];
-                else w = window<C::NW>(st, rk[jj] * C::SB);
-                if (C::SB == 4) {
-                  p0 = bias_pool(w & 0x0F0F0F0Fu, nz);
-                  p1 = bias_pool((w >> 4) & 0x0F0F0F0Fu, nz);
-                } else {
-                  const uint32_t lo16 = w & 0xFFFFu;
-                  const uint32_t t2 = (lo16 << 14) | lo16;
-                  p0 = bias_pool(t2 & 0x03030303u, nz);
-                  p1 = bias_pool((t2 >> 4) & 0x03030303u, nz);
-                }
-                const uint2 sel = lut[mb[jj] * LUT_LANES + l16];
-                bfrag[2 * jj2] = perm(p1, p0, sel.x);
-                bfrag[2 * jj2 + 1] = perm(p1, p0, sel.y);
-              }
-            }
             const int t = 2 * jb + half;                            // fragment index in the chunk
+            const v4i av0 = avn;
+            if (APF && t < 7) avn = *(const v4i*)(smem + aaddr[0] + 16 * (t + 1));
+            uint32_t bfrag[4];
+            decode_half<C, BITS>(st, rkb[jb & 1], selb[jb & 1], nz, half, bfrag);
             const v4i bv = (v4i){(int)bfrag[0], (int)bfrag[1], (int)bfrag[2], (int)bfrag[3]};
 #pragma unroll
             for (int p = 0; p < MP; ++p) {
-              const v4i av = *(const v4i*)(smem + aaddr[p] + 16 * t);
+              const v4i av = APF ? av0 : *(const v4i*)(smem + aaddr[p] + 16 * t);
               acc[p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bv, acc[p], 0, 0, 0);
               // One idle issue slot after every MFMA.  Without it some instantiations of this
               // kernel (register allocations in which the accumulator chain changes registers)
@@ -431,6 +587,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       float part_sum[MP];
 #pragma unroll
       for (int p = 0; p < MP; ++p) {
+        // quarter kq holds activation row kq, one running sum per chunk position; added in the
+        // order of the other decode path, so a row's result does not depend on M
+        if (QB) { part_sum[p] = (ysum[0] + ysum[MP > 1 ? 1 : 0]) + (ysum[MP > 2 ? 2 : 0] + ysum[MP > 3 ? 3 : 0]); continue; }
         const float h = ysum[p] + __shfl_xor(ysum[p], 16, 64);
         part_sum[p] = h + __shfl_xor(h, 32, 64);
       }
@@ -445,17 +604,25 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
         else ((uint16_t*)gm.y)[o] = f2bf(v);
       };
       if (SK == 1) {
+        if (QB) {
+          if (kq < h.M) store(kq, wr, part_sum[0]);
+        } else {
 #pragma unroll
-        for (int p = 0; p < MP; ++p)
-          if (kq == 0 && p < h.M) store(p, wr, part_sum[p]);
+          for (int p = 0; p < MP; ++p)
+            if (kq == 0 && p < h.M) store(p, wr, part_sum[p]);
+        }
       } else {
         // partial sums of the SK parts of a tile meet in an LDS slot; the wave that arrives last
         // adds them in part order (not arrival order), so the result does not depend on timing
         const int slot = tl & (h.nslot - 1);
         float* rs = red + (size_t)slot * h.sk_cap * h.M * 16;
+        if (QB) {
+          if (kq < h.M) rs[(part * h.M + kq) * 16 + wr] = part_sum[0];
+        } else {
 #pragma unroll
-        for (int p = 0; p < MP; ++p)
-          if (kq == 0 && p < h.M) rs[(part * h.M + p) * 16 + wr] = part_sum[p];
+          for (int p = 0; p < MP; ++p)
+            if (kq == 0 && p < h.M) rs[(part * h.M + p) * 16 + wr] = part_sum[p];
+        }
         int old = 0;
         if (lane == 0) old = atomicAdd(&cnt[slot], 1);
         old = __shfl(old, 0, 64);
@@ -537,7 +704,9 @@ static int launch_cfg(const GvBatch& b, size_t lds, int blocks, hipStream_t st) 
 template <int BITS, int KEEP, int GRP>
 static int launch_mp(const GvBatch& b, size_t lds, int blocks, hipStream_t st) {
   if (b.h.M == 1) return launch_cfg<BITS, KEEP, GRP, 1>(b, lds, blocks, st);
-  if (b.h.M == 2) return launch_cfg<BITS, KEEP, GRP, 2>(b, lds, blocks, st);
+  if constexpr (!block_split_capable(BITS, KEEP, GRP)) {
+    if (b.h.M == 2) return launch_cfg<BITS, KEEP, GRP, 2>(b, lds, blocks, st);
+  }
   return launch_cfg<BITS, KEEP, GRP, 4>(b, lds, blocks, st);
 }
 
@@ -574,8 +743,10 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
     g.order = !dense ? 0 : (m.bits == 2 ? 2 : 1);
     g.y = calls[i].y; g.bias = calls[i].bias; g.ldy = calls[i].ldy;
     g.ntiles = (m.K + 15) / 16; g.nS = (m.N / 128 + 3) / 4; g.cost0 = cost;
-    g.rsh = m.tiled ? 4 : 0; g.rmask = m.tiled ? 15 : 0;
-    g.row_a = m.tiled ? m.stride * 16u : m.stride; g.ustride = m.tiled ? 256u : 16u;
+    g.tile_a = (uint32_t)m.stride * 16u;                          // sixteen rows in either order
+    g.lane_mul = m.tiled ? 16u : (uint32_t)m.stride;
+    g.sz_mul = m.tiled ? 1u : (uint32_t)m.G;
+    g.ush = m.tiled ? 8 : 4; g.csh = m.tiled ? 4 : 0;
     cost += g.ntiles * g.nS;
     gb.h.cost_end[i] = cost;
     tiles += g.ntiles;
@@ -586,9 +757,9 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
   for (int i = n; i < GV_MAX_BATCH; ++i) gb.h.cost_end[i] = cost;
   gb.h.xq_cap = xq_cap; gb.h.delta_cap = delta_cap;
   int blocks = tiles < 256 ? tiles : 256;                       // one persistent workgroup per CU
-  // macro-steps per work item: about two items per wavefront over the whole launch, so that
+  // macro-steps per work item: about four items per wavefront over the whole launch, so that
   // the tail is short; a tile is split into at most 16 parts
-  int spi = cost / (blocks * GV_WAVES * 2);
+  int spi = cost / (blocks * GV_WAVES * 4);
   spi = spi < 1 ? 1 : (spi > 8 ? 8 : spi);
   int sk_cap = 1;
   for (int i = 0; i < n; ++i) {
@@ -606,7 +777,7 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
   gb.h.sk_cap = sk_cap; gb.h.nslot = nslot; gb.h.red_floats = nslot * slot_floats;
   gb.h.cq = cost / blocks; gb.h.cr = cost % blocks;
   const size_t lds = (size_t)LUT_BYTES + ZERO_BYTES + xq_cap + (size_t)delta_cap * 4 +
-                     (size_t)gb.h.red_floats * 4 + (size_t)nslot * 4;
+                     (size_t)gb.h.red_floats * 4 + (size_t)nslot * 4 + 16;   // + the item counter
   const int bits = gb.mat[0].m.bits;
   return bits == 2 ? launch_keep<2>(gb, lds, blocks, st) : bits == 3 ? launch_keep<3>(gb, lds, blocks, st)
        : bits == 4 ? launch_keep<4>(gb, lds, blocks, st) : CBK_ERR_UNSUPPORTED;
