@@ -6,7 +6,7 @@ namespace cbk {
 int launch_dequant(const DMat&, int, int, int, void*, int, int64_t, hipStream_t);
 int launch_gemv_generic(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*,
                         hipStream_t);
-struct GvCall { DMat m; const void* x; int64_t ldx; void* y; int64_t ldy; const void* bias; };
+struct GvCall { DMat m; const void* x; int64_t ldx; void* y; int64_t ldy; const void* bias; int par; };
 int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, void* ws, size_t ws_bytes,
                            hipStream_t);
 bool gemv_fast_takes(const DMat&, int M);
@@ -24,6 +24,55 @@ static inline bool gemm_big_takes(const DMat& m, int M) {
 }
 
 static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// Row range [lo, hi) of a fixed-stride matrix as a matrix of its own with a single col_scale
+// vector (row `cs_row` of the fused one).  lo is a multiple of 16, so the range is a contiguous
+// byte slice of data, scale and zero in the row-major and in the tiled order alike.
+static DMat row_range(const DMat& m, int lo, int hi, int cs_row) {
+  DMat s = m;
+  s.data = m.data + (size_t)lo * m.stride;
+  s.scale = m.scale + (size_t)lo * m.G;
+  s.zero = m.zero + (size_t)lo * m.G;
+  s.K = hi - lo;
+  s.cs = m.cs ? m.cs + (size_t)cs_row * m.N : nullptr;
+  s.cs_rows = m.cs ? 1 : 0;
+  s.cs_split0 = s.cs_split1 = 0;
+  return s;
+}
+
+// The q|k|v ranges of a matrix with three col_scale vectors, if each starts on a 16-row tile.
+// Returns the number of non-empty ranges (0: not decomposable).
+static int fused_ranges(const DMat& m, int (&lo)[3], int (&hi)[3], int (&row)[3]) {
+  if (m.cs_rows != 3 || family_of(m.layout) == FAM_SPARSE) return 0;
+  const int b0 = m.cs_split0, b1 = m.cs_split0 + m.cs_split1;
+  if (b0 % 16 || b1 % 16) return 0;
+  const int l[3] = {0, b0, b1}, h[3] = {b0, b1, m.K};
+  int n = 0;
+  for (int r = 0; r < 3; ++r)
+    if (h[r] > l[r]) { lo[n] = l[r]; hi[n] = h[r]; row[n] = r; ++n; }
+  return n;
+}
+
+// One call of the decode kernel per col_scale vector: a q|k|v matrix becomes up to three row
+// ranges; a gate/up matrix (two vectors by row parity) stays whole and is marked `par`, the
+// kernel then stages both scaled activation vectors and every row keeps the sum of its own.
+static int expand_fused(const GvCall& c, size_t ysz, GvCall* out) {
+  if (c.m.cs_rows != 3) {
+    out[0] = c;
+    out[0].par = c.m.cs_rows == 2 ? 1 : 0;
+    return 1;
+  }
+  int lo[3], hi[3], row[3];
+  const int n = fused_ranges(c.m, lo, hi, row);
+  for (int i = 0; i < n; ++i) {
+    out[i] = c;
+    out[i].m = row_range(c.m, lo[i], hi[i], row[i]);
+    out[i].y = (uint8_t*)c.y + (size_t)lo[i] * ysz;
+    out[i].bias = c.bias ? (const uint8_t*)c.bias + (size_t)lo[i] * ysz : nullptr;
+    out[i].par = 0;
+  }
+  return n;
+}
 
 static int canon(const cbk_desc* in, cbk_desc* o) {
   if (!in || !o) return CBK_ERR_NULL;
@@ -146,6 +195,8 @@ size_t cbk_workspace_bytes(const cbk_desc* in, int M) {
   if (to_dmat(in, &m, false)) return 0;
   if (M >= 1 && M <= 16 && gemv_fast_takes(m, 1)) return gemv_fast_workspace(m, 1);
   if (gemm_big_takes(m, M)) return gemm_big_workspace(m, M);
+  int lo[3], hi[3], row[3];
+  if (M > 128 && fused_ranges(m, lo, hi, row)) return gemm_big_workspace(row_range(m, lo[0], hi[0], row[0]), M);
   return 0;
 }
 
@@ -172,35 +223,51 @@ int cbk_gemv_batch(int n, const cbk_desc* descs, const void* const* xs, const in
   if (n < 1 || n > kMaxBatch) return CBK_ERR_SHAPE;
   if (!descs || !xs || !ldxs || !ys || !ldys) return CBK_ERR_NULL;
   if (M > 16) return CBK_ERR_SHAPE;
+  const size_t ysz = y_dtype == CBK_F32 ? 4 : 2;
   GvCall calls[kMaxBatch];
-  // activation rows per pass: as many (4, 2 or 1) as the digits of every matrix fit in LDS with
-  int mc = M >= 4 ? 4 : (M >= 2 ? 2 : 1);
+  int nc = 0;
   bool fast = true;
   for (int i = 0; i < n; ++i) {
-    int rc = to_dmat(descs + i, &calls[i].m, true);
+    GvCall c;
+    int rc = to_dmat(descs + i, &c.m, true);
     if (rc) return rc;
-    rc = check_io(xs[i], x_dtype, M, ldxs[i], ys[i], y_dtype, ldys[i], calls[i].m.N, calls[i].m.K);
+    rc = check_io(xs[i], x_dtype, M, ldxs[i], ys[i], y_dtype, ldys[i], c.m.N, c.m.K);
     if (rc) return rc;
-    calls[i].x = xs[i]; calls[i].ldx = ldxs[i]; calls[i].y = ys[i]; calls[i].ldy = ldys[i];
-    calls[i].bias = biases ? biases[i] : nullptr;
-    while (mc > 1 && !gemv_fast_takes(calls[i].m, mc) && gemv_fast_takes(calls[i].m, 1)) mc >>= 1;
-    fast = fast && gemv_fast_takes(calls[i].m, 1) && gemv_same_config(calls[0].m, calls[i].m);
+    c.x = xs[i]; c.ldx = ldxs[i]; c.y = ys[i]; c.ldy = ldys[i];
+    c.bias = biases ? biases[i] : nullptr;
+    c.par = 0;
+    GvCall sub[3];
+    const int k = fast ? expand_fused(c, ysz, sub) : 0;
+    if (k == 0 || nc + k > kMaxBatch) { fast = false; continue; }
+    for (int j = 0; j < k; ++j) calls[nc++] = sub[j];
+  }
+  // activation rows per pass: as many (4, 2 or 1) as the digits of every matrix fit in LDS with;
+  // a gate/up matrix stages two scaled copies of every activation row
+  const int vm = fast && calls[0].par ? 2 : 1;
+  int mc = M * vm >= 4 ? 4 / vm : (M * vm >= 2 ? 2 / vm : 1);
+  for (int i = 0; fast && i < nc; ++i) {
+    while (mc > 1 && !gemv_fast_takes(calls[i].m, mc * vm) && gemv_fast_takes(calls[i].m, vm)) mc >>= 1;
+    fast = gemv_fast_takes(calls[i].m, vm) && gemv_same_config(calls[0].m, calls[i].m) && calls[i].par == calls[0].par;
   }
   hipStream_t st = (hipStream_t)stream;
   if (fast) {
-    const size_t ysz = y_dtype == CBK_F32 ? 4 : 2;
     for (int m0 = 0, mp; m0 < M; m0 += mp) {            // the weights are streamed once per pass
       mp = M - m0 < mc ? M - m0 : mc;
       GvCall part[kMaxBatch];
-      for (int i = 0; i < n; ++i) {
+      for (int i = 0; i < nc; ++i) {
         part[i] = calls[i];
         part[i].x = (const uint8_t*)calls[i].x + (size_t)m0 * calls[i].ldx * 2;
         part[i].y = (uint8_t*)calls[i].y + (size_t)m0 * calls[i].ldy * ysz;
       }
-      int rc = launch_gemv_fast_batch(n, part, x_dtype, mp, y_dtype, workspace, workspace_bytes, st);
+      int rc = launch_gemv_fast_batch(nc, part, x_dtype, mp, y_dtype, workspace, workspace_bytes, st);
       if (rc) return rc;
     }
     return CBK_OK;
+  }
+  if (n == 1) {
+    DMat m;
+    to_dmat(descs, &m, true);
+    return launch_gemv_generic(m, xs[0], x_dtype, M, ldxs[0], ys[0], y_dtype, ldys[0], biases ? biases[0] : nullptr, st);
   }
   // mixed or unsupported configurations: one matrix at a time
   size_t off = 0;
@@ -223,9 +290,7 @@ int cbk_gemv(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ldx,
   rc = check_io(x, x_dtype, M, ldx, y, y_dtype, ldy, m.N, m.K);
   if (rc) return rc;
   if (M > 16) return CBK_ERR_SHAPE;
-  if (gemv_fast_takes(m, 1))
-    return cbk_gemv_batch(1, in, &x, &ldx, x_dtype, M, &y, &ldy, y_dtype, &bias, workspace, workspace_bytes, stream);
-  return launch_gemv_generic(m, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, (hipStream_t)stream);
+  return cbk_gemv_batch(1, in, &x, &ldx, x_dtype, M, &y, &ldy, y_dtype, &bias, workspace, workspace_bytes, stream);
 }
 
 int cbk_gemm(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ldx, void* y, int y_dtype,
@@ -238,6 +303,21 @@ int cbk_gemm(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ldx,
   if (gemm_big_takes(m, M))
     return launch_gemm_big(m, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, workspace, workspace_bytes,
                            (hipStream_t)stream);
+  int lo[3], hi[3], row[3];
+  const int nr = M > 128 ? fused_ranges(m, lo, hi, row) : 0;
+  if (nr) {
+    // q|k|v: each range is a matrix with one col_scale vector; the launches share the
+    // workspace (pre-scaled activations), which the stream order keeps apart
+    const size_t ysz = y_dtype == CBK_F32 ? 4 : 2;
+    for (int i = 0; i < nr; ++i) {
+      const DMat s = row_range(m, lo[i], hi[i], row[i]);
+      rc = launch_gemm_big(s, x, x_dtype, M, ldx, (uint8_t*)y + (size_t)lo[i] * ysz, y_dtype, ldy,
+                           bias ? (const uint8_t*)bias + (size_t)lo[i] * ysz : nullptr, workspace, workspace_bytes,
+                           (hipStream_t)stream);
+      if (rc) return rc;
+    }
+    return CBK_OK;
+  }
   return launch_gemm(m, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, (hipStream_t)stream);
 }
 

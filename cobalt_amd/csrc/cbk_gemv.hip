@@ -66,6 +66,8 @@ struct GvMat {
   const uint16_t* x;       // activations [M][ldx], fp16 or bf16 bits
   int64_t ldx;
   int order;               // digit order inside a 16-column fragment: 0 column order, 1 / 2 dense
+  int par;                 // 1: two col_scale vectors by row parity; activation row v of the kernel is
+                           // row v / 2 of x scaled by vector v % 2, and weight row k keeps the rows v = k (mod 2)
   void* y;
   const void* bias;
   int64_t ldy;
@@ -127,12 +129,16 @@ struct XLoad { uint4 x[2], c[2]; };
 
 // global loads of staging item `it` (activation row it / (N/16), columns 16 * (it % (N/16)) ...)
 __device__ inline void stage_load(const uint16_t* x, int64_t ldx, const uint16_t* cs, int n16, int it, bool one_row,
-                                  XLoad& r) {
+                                  int par, XLoad& r) {
   const int row = one_row ? 0 : it / n16, c16 = it - row * n16;
-  const uint16_t* xp = x + (size_t)row * ldx + c16 * 16;
+  const int xrow = par ? row >> 1 : row;
+  const uint16_t* xp = x + (size_t)xrow * ldx + c16 * 16;
   r.x[0] = ((const uint4*)xp)[0]; r.x[1] = ((const uint4*)xp)[1];
   r.c[0] = make_uint4(0, 0, 0, 0); r.c[1] = make_uint4(0, 0, 0, 0);
-  if (cs) { r.c[0] = ((const uint4*)(cs + c16 * 16))[0]; r.c[1] = ((const uint4*)(cs + c16 * 16))[1]; }
+  if (cs) {
+    const uint16_t* cp = cs + (par ? (size_t)(row & 1) * n16 * 16 : (size_t)0) + c16 * 16;
+    r.c[0] = ((const uint4*)cp)[0]; r.c[1] = ((const uint4*)cp)[1];
+  }
 }
 
 // conversion of one loaded item into digits and delta in LDS; the eight consecutive lanes of a
@@ -435,7 +441,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     const int n16 = N >> 4, xitems = h.M * n16;                   // a multiple of 8
     int xit = tid;
     XLoad xl;
-    if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, MP == 1, xl);
+    if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, MP == 1, gm.par, xl);
     // Three load buffers rotate through the roles (being decoded, next, being loaded) by name:
     // copying a buffer would wait for the loads that are still filling it.
     // Configurations with long code streams or four activation rows keep one step in flight
@@ -462,7 +468,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     while (xit < xitems) {
       stage_convert<(!C::DENSE ? 0 : (BITS == 2 ? 2 : 1))>(xl, m.cs != nullptr, h.xdt, N, n16, xit, MP == 1, xq, delta);
       xit += GV_THREADS;
-      if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, MP == 1, xl);
+      if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, MP == 1, gm.par, xl);
     }
     // the second step of loads goes out only now: issued together with the first, the two
     // bursts of all wavefronts interleave in the memory system and every first step lands late
@@ -596,6 +602,10 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       auto store = [&](int om, int r, float v) {
         const int k = tile * 16 + r;
         if (k >= m.K) return;
+        if (gm.par) {                                             // the sum scaled for the other parity is dropped
+          if ((om ^ k) & 1) return;
+          om >>= 1;
+        }
         if (gm.bias) v += (h.ydt == CBK_F32) ? ((const float*)gm.bias)[k]
                         : (h.ydt == CBK_F16) ? h2f(((const uint16_t*)gm.bias)[k]) : bf2f(((const uint16_t*)gm.bias)[k]);
         const size_t o = (size_t)om * gm.ldy + k;
@@ -662,7 +672,7 @@ static bool keep_supported(int keep) { return keep == 10 || keep == 16 || keep =
 
 bool gemv_fast_takes(const DMat& m, int M) {
   if (M < 1 || M > GV_MAX_M) return false;
-  if (m.cs_rows > 1) return false;
+  if (m.cs_rows == 3) return false;                              // the caller splits q|k|v into its ranges
   if (!(m.flags & CBK_FLAG_ZERO_LE_128)) return false;
   const int fam = family_of(m.layout);
   if (fam == FAM_BLK) { if (!keep_supported(m.keep)) return false; }
@@ -686,6 +696,7 @@ struct GvCall {           // one matrix of a batched call, host side
   void* y;
   int64_t ldy;
   const void* bias;
+  int par;                  // gate/up matrix: M counts real activation rows, the kernel sees 2 M
 };
 
 template <int BITS, int KEEP, int GRP, int MP>
@@ -733,6 +744,11 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
                            hipStream_t st) {
   if (n < 1 || n > GV_MAX_BATCH) return CBK_ERR_SHAPE;
   GvBatch gb;
+  const int par = calls[0].par ? 1 : 0;
+  for (int i = 0; i < n; ++i)
+    if ((calls[i].par ? 1 : 0) != par || (calls[i].m.cs_rows == 2) != (par == 1)) return CBK_ERR_UNSUPPORTED;
+  M *= par + 1;                                                   // activation rows as the kernel counts them
+  if (M > GV_MAX_M) return CBK_ERR_SHAPE;
   gb.h.n = n; gb.h.M = M; gb.h.xdt = xdt; gb.h.ydt = ydt;
   int cost = 0, xq_cap = 0, delta_cap = 0, tiles = 0;
   for (int i = 0; i < n; ++i) {
@@ -741,6 +757,7 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
     GvMat& g = gb.mat[i];
     g.m = m; g.x = (const uint16_t*)calls[i].x; g.ldx = calls[i].ldx;
     g.order = !dense ? 0 : (m.bits == 2 ? 2 : 1);
+    g.par = par;
     g.y = calls[i].y; g.bias = calls[i].bias; g.ldy = calls[i].ldy;
     g.ntiles = (m.K + 15) / 16; g.nS = (m.N / 128 + 3) / 4; g.cost0 = cost;
     g.tile_a = (uint32_t)m.stride * 16u;                          // sixteen rows in either order
@@ -781,12 +798,6 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
   const int bits = gb.mat[0].m.bits;
   return bits == 2 ? launch_keep<2>(gb, lds, blocks, st) : bits == 3 ? launch_keep<3>(gb, lds, blocks, st)
        : bits == 4 ? launch_keep<4>(gb, lds, blocks, st) : CBK_ERR_UNSUPPORTED;
-}
-
-int launch_gemv_fast(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
-                     const void* bias, void* ws, size_t ws_bytes, hipStream_t st) {
-  GvCall c{m, x, ldx, y, ldy, bias};
-  return launch_gemv_fast_batch(1, &c, xdt, M, ydt, ws, ws_bytes, st);
 }
 
 }  // namespace cbk

@@ -222,6 +222,82 @@ def test_gemv_rows_are_independent_of_batch_and_run_to_run_identical():
     assert torch.equal(ops.gemv(pm, x, out_dtype=torch.float32), y4)
 
 
+# ------------------------------------------------------------------ row-fused matrices
+FUSED_CASES = [(F.BLK1632_4, 4, 128, 16), (F.BLKC, 3, 128, 10), (F.BLKC, 2, 64, 23), (F.DENSE4, 4, 128, 0)]
+
+
+def _fused(case, K, N, cs_rows, splits, seed, tiled):
+    raw = make_raw(case, K, N, seed=seed)
+    pk = oracle_pack(case, raw)
+    rng = np.random.default_rng(seed)
+    cs = (rng.random((cs_rows, N)) * 1.5 + 0.5).astype(np.float16)
+    pm = packed_from_oracle(case, pk, cs, K, N, DEV, cs_splits=splits, tiled=tiled)
+    W = R.dequant(pk, K, N, case[0], col_scale=cs, cs_splits=splits, **kw_of(case))
+    return pm, W
+
+
+@pytest.mark.parametrize("tiled", [False, True], ids=["rowmajor", "tiled"])
+@pytest.mark.parametrize("case", FUSED_CASES, ids=case_id)
+def test_gemv_fused_col_scale_rows(case, tiled):
+    """Fused q|k|v (three col_scale vectors by row range) and gate/up (two by row parity):
+    docs/FORMAT.md:126-151, cobalt_format.h:77-99.  Ranges on 16-row tiles go through the MFMA
+    kernel range by range; the (40, 8) split does not and takes the row kernel."""
+    K, N = 208, 1024
+    for cs_rows, splits in ((2, (0, 0)), (3, (96, 48)), (3, (208, 0)), (3, (40, 8))):
+        pm, W = _fused(case, K, N, cs_rows, splits, seed=K + cs_rows + splits[0], tiled=tiled)
+        for M in (1, 2, 3, 4, 5, 8):
+            for dtype in (torch.float16, torch.bfloat16):
+                x = acts(M, N, dtype, seed=M)
+                bias = acts(1, K, torch.float32, seed=9)[0]
+                ref = R.forward_ref(W, _np(x)) + _np(bias)[None, :]
+                y = ops.gemv(pm, x.to(DEV), bias=bias.to(DEV), out_dtype=torch.float32)
+                err = rel_fro(_np(y), ref)
+                assert err < TOL, f"{case_id(case)} cs_rows={cs_rows} splits={splits} M={M} {dtype}: {err}"
+
+
+def test_gemv_fused_rows_equal_their_unfused_parts_bit_for_bit():
+    """A q|k|v matrix gives, row for row, the bits of its three parts run on their own, and a
+    gate/up matrix the bits of the even-row and odd-row matrices (same sums, same order; at a
+    size where the fused and the separate launches cut the columns into the same parts)."""
+    case = (F.BLK1632_4, 4, 128, 16)
+    K, N = 256, 4096
+    raw = make_raw(case, K, N, seed=77)
+    pk = oracle_pack(case, raw)
+    rng = np.random.default_rng(5)
+    x = acts(2, N, torch.float16, seed=4).to(DEV)
+    cs3 = (rng.random((3, N)) * 1.5 + 0.5).astype(np.float16)
+    fused = packed_from_oracle(case, pk, cs3, K, N, DEV, cs_splits=(128, 64), tiled=True)
+    y = ops.gemv(fused, x, out_dtype=torch.float32)
+    for r, (lo, hi) in enumerate(((0, 128), (128, 192), (192, 256))):
+        sub = {k: (v[lo:hi] if k != "row_off" else v) for k, v in pk.items() if k in ("scale", "zero")}
+        stride = R.row_stride(case[0], N)
+        sub["data"] = np.concatenate([pk["data"][lo * stride: hi * stride], np.zeros(64, np.uint8)])
+        part = packed_from_oracle(case, sub, cs3[r], hi - lo, N, DEV, tiled=True)
+        assert torch.equal(ops.gemv(part, x, out_dtype=torch.float32), y[:, lo:hi])
+    cs2 = cs3[:2]
+    gu = packed_from_oracle(case, pk, cs2, K, N, DEV, tiled=True)
+    y2 = ops.gemv(gu, x, out_dtype=torch.float32)
+    whole = [ops.gemv(packed_from_oracle(case, pk, cs2[c], K, N, DEV, tiled=True), x, out_dtype=torch.float32)
+             for c in range(2)]
+    assert torch.equal(y2[:, 0::2], whole[0][:, 0::2]) and torch.equal(y2[:, 1::2], whole[1][:, 1::2])
+
+
+@pytest.mark.parametrize("case", FUSED_CASES[:2], ids=case_id)
+def test_gemm_fused_col_scale_rows(case):
+    """Prefill on fused matrices: q|k|v ranges run the 256 x 256 kernel range by range, gate/up
+    (row parity) the 128 x 128 kernel."""
+    K, N = 640, 1024
+    for cs_rows, splits in ((3, (256, 128)), (3, (48, 16)), (2, (0, 0))):
+        pm, W = _fused(case, K, N, cs_rows, splits, seed=K + cs_rows + splits[0], tiled=True)
+        for M, dtype in ((300, torch.bfloat16), (129, torch.float16), (64, torch.float16)):
+            x = acts(M, N, dtype, seed=M)
+            bias = acts(1, K, torch.float32, seed=9)[0]
+            ref = R.forward_ref(W, _np(x)) + _np(bias)[None, :]
+            y = ops.gemm(pm, x.to(DEV), bias=bias.to(DEV), out_dtype=torch.float32)
+            err = rel_fro(_np(y), ref)
+            assert err < TOL, f"{case_id(case)} cs_rows={cs_rows} splits={splits} M={M}: {err}"
+
+
 # ------------------------------------------------------------------ prefill GEMM
 @pytest.mark.parametrize("tiled", [False, True], ids=["rowmajor", "tiled"])
 @pytest.mark.parametrize("case", FIXED_CASES, ids=case_id)
