@@ -20,7 +20,8 @@ int launch_gemm_big(const DMat&, const void*, int, int, int64_t, void*, int, int
 size_t gemm_big_workspace(const DMat&, int M);
 // the 256 x 256 tile kernel pays off once a call fills at least one token tile halfway
 static inline bool gemm_big_takes(const DMat& m, int M) {
-  return M > 128 && family_of(m.layout) != FAM_SPARSE && m.cs_rows <= 1;
+  if (M <= 128 || family_of(m.layout) == FAM_SPARSE) return false;
+  return m.cs_rows <= 2 || (m.cs_split0 % 256 == 0 && (m.cs_split0 + m.cs_split1) % 256 == 0);
 }
 
 static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }

@@ -52,6 +52,14 @@ struct GbArgs {
   int64_t ldy;
   const void* bias;
   int tiles_t, tiles_r;
+  // par = 1: gate/up matrix, two col_scale vectors by row parity.  A workgroup then takes 256
+  // rows of one parity out of 512 (rows r0 + 2 i + p), and X' of that parity's vector, which
+  // starts xps elements after the other one.
+  int par;
+  size_t xps;
+  // q|k|v matrix whose ranges start on row tiles: rows from vs0 on use the second X', rows from
+  // vs1 on the third (both INT_MAX for any other matrix)
+  int vs0, vs1;
 };
 
 // One wavefront-wide copy of 64 x 16 bytes from global memory straight into LDS (no VGPRs, no
@@ -89,7 +97,7 @@ __device__ inline uint4 bytes_to_halfs(uint32_t b0, uint32_t b1, h2_t s2) {
 // turning the tile around in LDS makes the global stores whole 16-byte pieces of consecutive
 // output columns: 256 B (f16) or 512 B (f32) per token.  Compile-time indexed and branch-free
 // per element: the 256 accumulators make this straight-line code, and it has to stay small.
-template <int YDT>
+template <int YDT, int kstep>                                    // local row i is output column row0 + kstep * i
 __device__ inline void gb_epilogue(const GbArgs& a, v16f (&acc)[4][4], uint8_t* smem, int lane, int wave, int tok0,
                                    int row0) {
   constexpr int ESZ = YDT == CBK_F32 ? 4 : 2;
@@ -101,7 +109,7 @@ __device__ inline void gb_epilogue(const GbArgs& a, v16f (&acc)[4][4], uint8_t* 
   float bv[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int k = row0 + 32 * j + (lane & 31);
+    const int k = row0 + kstep * (32 * j + (lane & 31));
     bv[j] = 0.f;
     if (a.bias && k < K) bv[j] = load_act<YDT>(a.bias, k);
   }
@@ -126,15 +134,15 @@ __device__ inline void gb_epilogue(const GbArgs& a, v16f (&acc)[4][4], uint8_t* 
     for (int t = 0; t < 32 * PPR / 64; ++t) {
       const int pc = t * 64 + lane;
       const int row = pc / PPR, c = pc % PPR;
-      const int tok = tok0 + 32 * i + row, k = row0 + c * EPP;
+      const int tok = tok0 + 32 * i + row, k = row0 + kstep * (c * EPP);
       if (tok >= a.M || k >= K) continue;
       const uint8_t* src = ep + row * PITCH + c * 16;
       uint8_t* dst = (uint8_t*)a.y + ((size_t)tok * a.ldy + k) * ESZ;
-      if (vec_ok && k + EPP <= K) *(uint4*)dst = *(const uint4*)src;
+      if (vec_ok && kstep == 1 && k + EPP <= K) *(uint4*)dst = *(const uint4*)src;
       else
-        for (int e = 0; e < EPP && k + e < K; ++e) {
-          if (ESZ == 4) ((float*)dst)[e] = ((const float*)src)[e];
-          else ((uint16_t*)dst)[e] = ((const uint16_t*)src)[e];
+        for (int e = 0; e < EPP && k + kstep * e < K; ++e) {
+          if (ESZ == 4) ((float*)dst)[kstep * e] = ((const float*)src)[e];
+          else ((uint16_t*)dst)[kstep * e] = ((const uint16_t*)src)[e];
         }
     }
   }
@@ -142,7 +150,10 @@ __device__ inline void gb_epilogue(const GbArgs& a, v16f (&acc)[4][4], uint8_t* 
 
 // BITS 2 / 3 / 4: byte-permute decoder for (BITS, KEEP, GRP), KEEP = 0 for the dense layouts.
 // BITS 0: generic 32-column reader, any fixed-stride layout.
-template <int BITS, int KEEP, int GRP>
+// PAR 0: one col_scale vector.  1: gate/up matrix (GbArgs::par).  2: q|k|v matrix (GbArgs::vs0, vs1).
+// Three instantiations rather than run-time switches: the schedule of the main loop is tuned
+// to the instruction and measurably shifts with every value that is added to it.
+template <int BITS, int KEEP, int GRP, int PAR>
 __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   constexpr bool FASTD = BITS != 0;
   using C = CodeCfg<FASTD ? BITS : 4, KEEP, FASTD ? GRP : 128>;
@@ -163,7 +174,9 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   const int lin = xcd * per + idx;                                 // token-tile-major linear id
   if (lin >= nb) return;
   const int tt = lin / a.tiles_r, tr = lin % a.tiles_r;
-  const int t0 = tt * GB_T, r0 = tr * GB_R;
+  constexpr int kstep = PAR == 1 ? 2 : 1;                         // row stride of this workgroup's rows
+  const int pp = PAR == 1 ? (tr & 1) : 0;                         // and their parity
+  const int t0 = tt * GB_T, r0 = PAR == 1 ? (tr >> 1) * (2 * GB_R) + pp : tr * GB_R;
   const int N = m.N, Npad = a.Npad;
   const int nst = Npad / GB_K;                                    // a multiple of 4; stages past N see X' = 0
   const int nch = N >> 7;                                         // 128-column chunks of the weight rows
@@ -184,7 +197,7 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
   // this thread's weight row
-  const int wrow = r0 + tid;
+  const int wrow = r0 + kstep * tid;
   const bool wok = wrow < m.K;
   const int wrc = wok ? wrow : m.K - 1;
   const RowView rv = row_view(m, wrc);
@@ -196,7 +209,8 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   const int wv = __builtin_amdgcn_readfirstlane(wave);
   const uint32_t xvo_e = (uint32_t)((lane >> 3) * Npad * 2 + (((lane & 7) ^ (lane >> 4)) * 16));
   const uint32_t xvo_o = (uint32_t)((lane >> 3) * Npad * 2 + (((lane & 7) ^ (4 + (lane >> 4))) * 16));
-  const uint8_t* xsb = (const uint8_t*)(a.xp + (size_t)(t0 + 64 * wv) * Npad);
+  const int xv = PAR == 1 ? pp : PAR == 2 ? (r0 >= a.vs0 ? 1 : 0) + (r0 >= a.vs1 ? 1 : 0) : 0;   // which col_scale vector
+  const uint8_t* xsb = (const uint8_t*)(a.xp + (size_t)xv * a.xps + (size_t)(t0 + 64 * wv) * Npad);
   const uint32_t xlds0 = (uint32_t)(uintptr_t)Xs + (uint32_t)wv * 8192u;
   auto dma_x = [&](int s, int buf) {                              // stage s -> Xs[buf]
     const uint8_t* sb = xsb + (size_t)s * (GB_K * 2);
@@ -431,15 +445,15 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
-  const int tok0 = t0 + 128 * wt, row0 = r0 + 128 * wr;
-  if (a.ydt == CBK_F32) gb_epilogue<CBK_F32>(a, acc, smem, lane, wave, tok0, row0);
-  else if (a.ydt == CBK_F16) gb_epilogue<CBK_F16>(a, acc, smem, lane, wave, tok0, row0);
-  else gb_epilogue<CBK_BF16T>(a, acc, smem, lane, wave, tok0, row0);
+  const int tok0 = t0 + 128 * wt, row0 = r0 + kstep * 128 * wr;
+  if (a.ydt == CBK_F32) gb_epilogue<CBK_F32, kstep>(a, acc, smem, lane, wave, tok0, row0);
+  else if (a.ydt == CBK_F16) gb_epilogue<CBK_F16, kstep>(a, acc, smem, lane, wave, tok0, row0);
+  else gb_epilogue<CBK_BF16T, kstep>(a, acc, smem, lane, wave, tok0, row0);
 }
 
-template <int BITS, int KEEP, int GRP>
-static int launch_big_cfg(const GbArgs& a, int blocks, hipStream_t st) {
-  auto kern = gemm_big_kernel<BITS, KEEP, GRP>;
+template <int BITS, int KEEP, int GRP, int PAR>
+static int launch_big_par(const GbArgs& a, int blocks, hipStream_t st) {
+  auto kern = gemm_big_kernel<BITS, KEEP, GRP, PAR>;
   static std::atomic<int> configured{0};
   if (!configured.load(std::memory_order_acquire)) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
@@ -448,6 +462,13 @@ static int launch_big_cfg(const GbArgs& a, int blocks, hipStream_t st) {
   }
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), GB_LDS, st, a);
   return hipGetLastError() == hipSuccess ? CBK_OK : CBK_ERR_HIP;
+}
+
+template <int BITS, int KEEP, int GRP>
+static int launch_big_cfg(const GbArgs& a, int blocks, hipStream_t st) {
+  if (a.par) return launch_big_par<BITS, KEEP, GRP, 1>(a, blocks, st);
+  if (a.vs0 != 0x7fffffff) return launch_big_par<BITS, KEEP, GRP, 2>(a, blocks, st);
+  return launch_big_par<BITS, KEEP, GRP, 0>(a, blocks, st);
 }
 
 // the (keep, group) instantiations of one code width

@@ -38,24 +38,32 @@ static inline int gb_npad(int N) { return (N + 255) / 256 * 256; }
 
 size_t gemm_big_workspace(const DMat& m, int M) {
   const size_t mpad = (size_t)(M + GB_T - 1) / GB_T * GB_T;
-  return (mpad * gb_npad(m.N) * 2 + 255) & ~(size_t)255;
+  return ((m.cs_rows > 1 ? m.cs_rows : 1) * mpad * gb_npad(m.N) * 2 + 255) & ~(size_t)255;
 }
 
 int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
                     const void* bias, void* ws, size_t ws_bytes, hipStream_t st) {
   if (family_of(m.layout) == FAM_SPARSE) return CBK_ERR_UNSUPPORTED;
-  if (m.cs_rows > 1) return CBK_ERR_UNSUPPORTED;
+  // q|k|v ranges off the row-tile grid: the caller passes them one by one
+  if (m.cs_rows == 3 && (m.cs_split0 % GB_R || (m.cs_split0 + m.cs_split1) % GB_R)) return CBK_ERR_UNSUPPORTED;
   if (ydt != CBK_F32 && ydt != CBK_F16 && ydt != CBK_BF16T) return CBK_ERR_DTYPE;
   if (!ws || ws_bytes < gemm_big_workspace(m, M)) return CBK_ERR_WORKSPACE;
   if ((uintptr_t)ws & 255) return CBK_ERR_ALIGN;
   const int Mpad = (M + GB_T - 1) / GB_T * GB_T;
   const int Npad = gb_npad(m.N);
   const int64_t items = (int64_t)Mpad * (Npad / 8);
-  hipLaunchKernelGGL(gemm_prep_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st,
-                     (const uint16_t*)x, ldx, m.cs, xdt, M, Mpad, m.N, Npad, (uint16_t*)ws);
+  const int par = m.cs_rows == 2 ? 1 : 0;
+  for (int v = 0; v < (m.cs_rows > 1 ? m.cs_rows : 1); ++v)       // one X' per col_scale vector
+    hipLaunchKernelGGL(gemm_prep_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st,
+                       (const uint16_t*)x, ldx, m.cs ? m.cs + (size_t)v * m.N : nullptr, xdt, M, Mpad, m.N, Npad,
+                       (uint16_t*)ws + (size_t)v * Mpad * Npad);
   GbArgs a;
   a.m = m; a.xp = (const uint16_t*)ws; a.M = M; a.Npad = Npad; a.y = y; a.ydt = ydt; a.ldy = ldy; a.bias = bias;
-  a.tiles_t = (M + GB_T - 1) / GB_T; a.tiles_r = (m.K + GB_R - 1) / GB_R;
+  a.par = par; a.xps = (size_t)Mpad * Npad;
+  a.vs0 = m.cs_rows == 3 ? m.cs_split0 : 0x7fffffff;
+  a.vs1 = m.cs_rows == 3 ? m.cs_split0 + m.cs_split1 : 0x7fffffff;
+  a.tiles_t = (M + GB_T - 1) / GB_T;
+  a.tiles_r = par ? 2 * ((m.K + 2 * GB_R - 1) / (2 * GB_R)) : (m.K + GB_R - 1) / GB_R;
   const int nb = a.tiles_t * a.tiles_r;
   const int blocks = ((nb + 7) / 8) * 8;
   const bool le128 = (m.flags & CBK_FLAG_ZERO_LE_128) != 0;
