@@ -70,7 +70,10 @@ enum cbk_status {
  *   col_scale fp16  [cs_rows, N] or NULL (then the factor is 1), 16-byte aligned
  *   cs_rows   1: one vector.  2: fused gate/up, row k uses vector k&1.  3: fused q|k|v, rows
  *             [0,cs_split0) use vector 0, [cs_split0, cs_split0+cs_split1) vector 1, the rest 2
- *             (cobalt_format.h:77-99, docs/FORMAT.md:134-151).
+ *             (cobalt_format.h:77-99, docs/FORMAT.md:134-151).  Both kinds run the matrix-core
+ *             kernels (q|k|v: decode needs the two boundaries on multiples of 16 rows, prefill
+ *             runs range by range unless they are multiples of 256); other splits take the
+ *             float row kernel for decode.
  *   bits/group/keep  must be given for layouts 8/9; for 0-7 they may be 0 (implied).
  *   flags     CBK_FLAG_ZERO_LE_128: the caller guarantees that every stored zero point is
  *             <= 128 (always true for an on-grid zero point of a 2/3/4-bit code, and for the
@@ -117,7 +120,8 @@ size_t cbk_stream_bytes(const cbk_desc* d, size_t sparse_data_bytes);
 
 /* Device scratch needed by cbk_gemv / cbk_gemm / cbk_linear for M activation rows (0 for the
  * decode kernels; the prefill kernel for M > 128 keeps its pre-scaled fp16 activations there:
- * ceil(M/256)*256*N*2 bytes).  The workspace must be 256-byte aligned. */
+ * ceil(M/256)*256 * ceil(N/256)*256 * 2 bytes per col_scale vector, i.e. times cs_rows for a
+ * fused matrix).  The workspace must be 256-byte aligned. */
 size_t cbk_workspace_bytes(const cbk_desc* d, int M);
 
 /* Rows [row0, row0+nrows) of W_hat -> out[nrows, ld_out] in out_dtype, bit-exact float32
