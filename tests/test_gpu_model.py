@@ -1,0 +1,59 @@
+"""Whole-model installation on a Hugging Face decoder (random-initialised tiny Mistral; there are
+no checkpoints here): the packed model's logits against the same model with every packed layer
+turned back into a dense layer of its dequantised weight."""
+import copy
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _tiny_mistral():
+    tr = pytest.importorskip("transformers")
+    cfg = tr.MistralConfig(vocab_size=512, hidden_size=256, intermediate_size=512, num_hidden_layers=2,
+                           num_attention_heads=4, num_key_value_heads=2, max_position_embeddings=512,
+                           sliding_window=None, attn_implementation="eager")
+    torch.manual_seed(0)
+    return tr.MistralForCausalLM(cfg).to(DEV, torch.float16).eval()
+
+
+def test_hf_decoder_is_compressed_in_place_and_matches_its_dense_twin():
+    from cobalt_amd import model as Mo
+    from cobalt_amd.linear import CobaltLinear
+    m = _tiny_mistral()
+    g = torch.Generator().manual_seed(1)
+    calib = torch.randint(0, 512, (8, 64), generator=g).to(DEV)
+    rep = Mo.compress_model(m, calib, sparsity=0.5, bits=4, group=128, layers_per_pass=1)
+    assert len(rep) == 14 and all(abs(r["bpw"] - 3.1875) < 1e-9 for r in rep.values())
+    assert sum(isinstance(x, CobaltLinear) for x in m.modules()) == 14
+    assert all(x._pm().tiled for x in m.modules() if isinstance(x, CobaltLinear))
+    twin = Mo.dense_twin(copy.deepcopy(m), torch.float16)
+    assert not any(isinstance(x, CobaltLinear) for x in twin.modules())
+    # prefill (M = 300 rows: the 256 x 256 kernel), a short prompt (M = 24: the 128 x 128 kernel)
+    # and single-token steps (the decode kernel)
+    for shape in ((1, 300), (2, 12), (1, 1), (3, 1)):
+        ids = torch.randint(0, 512, shape, generator=g).to(DEV)
+        with torch.no_grad():
+            a = m(ids).logits.float()
+            b = twin(ids).logits.float()
+        err = float((a - b).norm() / b.norm())
+        assert err < 5e-3, (shape, err)                             # fp16 activations through two blocks
+
+
+def test_compressed_model_state_dict_round_trip():
+    from cobalt_amd import model as Mo
+    m = _tiny_mistral()
+    Mo.compress_model(m, None)
+    sd = {k: v.clone() for k, v in m.state_dict().items()}
+    m2 = _tiny_mistral()
+    Mo.compress_model(m2, None, sparsity=0.5)                       # same module structure, other bytes
+    for k in sd:
+        if k.endswith("blob"):
+            sd[k] = sd[k].clone()
+    m2.load_state_dict(sd)
+    ids = torch.randint(0, 512, (1, 5), generator=torch.Generator().manual_seed(2)).to(DEV)
+    with torch.no_grad():
+        assert torch.equal(m(ids).logits, m2(ids).logits)

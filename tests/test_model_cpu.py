@@ -1,0 +1,102 @@
+"""Whole-model installer on the CPU: block discovery, Hessian collection and module replacement
+(the packed modules themselves only run on the GPU)."""
+import types
+
+import pytest
+import torch
+import torch.nn as nn
+
+from cobalt_amd import format as F
+from cobalt_amd import model as Mo
+from cobalt_amd.linear import CobaltLinear
+
+
+class _Attn(nn.Module):
+    def __init__(s, h, kv):
+        super().__init__()
+        s.q_proj, s.k_proj, s.v_proj, s.o_proj = nn.Linear(h, h, bias=False), nn.Linear(h, kv, bias=False), \
+            nn.Linear(h, kv, bias=True), nn.Linear(h, h, bias=False)
+
+    def forward(s, x):
+        return s.o_proj(torch.tanh(s.q_proj(x)) * s.k_proj(x).mean(-1, keepdim=True) + s.v_proj(x).mean(-1, keepdim=True))
+
+
+class _Mlp(nn.Module):
+    def __init__(s, h, i):
+        super().__init__()
+        s.gate_proj, s.up_proj, s.down_proj = nn.Linear(h, i, bias=False), nn.Linear(h, i, bias=False), nn.Linear(i, h, bias=False)
+
+    def forward(s, x):
+        return s.down_proj(torch.nn.functional.silu(s.gate_proj(x)) * s.up_proj(x))
+
+
+class _Block(nn.Module):
+    def __init__(s, h, kv, i):
+        super().__init__()
+        s.self_attn, s.mlp = _Attn(h, kv), _Mlp(h, i)
+
+    def forward(s, x):
+        x = x + s.self_attn(x)
+        return x + s.mlp(x)
+
+
+class _Toy(nn.Module):
+    def __init__(s, h=256, kv=128, i=384, layers=3, vocab=64):
+        super().__init__()
+        s.embed = nn.Embedding(vocab, h)
+        s.layers = nn.ModuleList([_Block(h, kv, i) for _ in range(layers)])
+        s.lm_head = nn.Linear(h, vocab, bias=False)
+
+    def forward(s, ids):
+        x = s.embed(ids)
+        for l in s.layers:
+            x = l(x)
+        return s.lm_head(x)
+
+
+def test_blocks_are_found_and_hessians_are_sums_of_outer_products():
+    torch.manual_seed(0)
+    m = _Toy()
+    blocks = Mo.decoder_blocks(m)
+    assert [n for n, _ in blocks] == ["layers.0", "layers.1", "layers.2"]
+    ids = torch.randint(0, 64, (5, 7))
+    Hs = Mo.collect_hessians(m, blocks[:2], [ids[:3], ids[3:]])
+    assert set(Hs) == {(b, g) for b in ("layers.0", "layers.1") for g in Mo.HGROUPS}
+    X0 = m.embed(ids).reshape(-1, 256).float()                    # what layers.0's q/k/v read
+    assert torch.allclose(Hs[("layers.0", "attn_in")], X0.T @ X0, rtol=1e-5, atol=1e-4)
+    # the down projection reads the gated activation: its Hessian is [inter, inter]
+    assert Hs[("layers.1", "mlp_out")].shape == (384, 384)
+    assert not m.layers[0].self_attn.q_proj._forward_pre_hooks      # hooks are gone
+
+
+def test_compress_model_replaces_every_linear_and_honours_overrides():
+    torch.manual_seed(1)
+    m = _Toy(layers=2)
+    ids = torch.randint(0, 64, (4, 16))
+    rep = Mo.compress_model(m, ids, sparsity=0.5, bits=4, group=128, layers_per_pass=1,
+                            bits_override={"mlp.down_proj": 3}, sparsity_override={"self_attn.o_proj": 0.0})
+    assert len(rep) == 14
+    for li in range(2):
+        blk = m.layers[li]
+        for name in Mo.LINEARS:
+            mod = Mo._sub(blk, name)
+            assert isinstance(mod, CobaltLinear), name
+        assert rep[f"layers.{li}.mlp.gate_proj"]["layout"] == F.BLK1632_4
+        assert abs(rep[f"layers.{li}.mlp.gate_proj"]["bpw"] - 3.1875) < 1e-9
+        assert rep[f"layers.{li}.mlp.down_proj"]["layout"] == F.BLKC and rep[f"layers.{li}.mlp.down_proj"]["bits"] == 3
+        assert rep[f"layers.{li}.self_attn.o_proj"]["layout"] == F.DENSE4
+        assert blk.self_attn.v_proj.bias is not None and blk.self_attn.q_proj.bias is None
+    assert isinstance(m.lm_head, nn.Linear)                        # only decoder blocks are touched
+    assert Mo.compress_model(m, ids) == {}                         # nothing left to do
+    with pytest.raises(ValueError):
+        Mo.compress_model(_Toy(layers=1), ids, bits_override={"lm_head": 4})
+    with pytest.raises(ValueError):
+        Mo.compress_model(nn.Linear(8, 8), ids)
+
+
+def test_packed_forward_fails_loudly_without_a_gpu():
+    m = _Toy(layers=1)
+    Mo.compress_model(m, None)
+    if not torch.cuda.is_available():
+        with pytest.raises(Exception):
+            m(torch.randint(0, 64, (1, 4)))
