@@ -94,8 +94,10 @@ def main(argv=None):
     base = dict(layers=a.layers, hidden=a.hidden, inter=a.inter, sparsity=a.sparsity, bits=a.bits, group=a.group,
                 bpw=next(iter(rep.values()))["bpw"], data="random weights, random calibration ids",
                 compress_s=round(time.time() - t0, 1))
-    for name in ("packed", "dense fp16 twin"):
-        if name != "packed":
+    for name in ("packed", "packed, q|k|v and gate/up fused", "dense fp16 twin"):
+        if name.startswith("packed,"):
+            Mo.fuse_model(model)
+        elif name != "packed":
             model = Mo.dense_twin(model, torch.float16)
         tps = _decode_tokens_per_s(tr, model, cfg, dev, a.steps, 16, 512)
         pms = _prefill_ms(model, cfg, dev, a.prefill)

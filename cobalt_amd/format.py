@@ -421,6 +421,50 @@ def from_arrays(data, scale, zero, col_scale, K, N, layout, bits=None, group=Non
                         data.numel() - BLOB_TAIL, flags=flags)
 
 
+def fuse_rows(parts, interleave: bool = False) -> PackedMatrix:
+    """Row-fused matrix of several packed matrices that multiply the same activation
+    (docs/FORMAT.md:126-151): `interleave=False` concatenates two or three of them (q | k | v;
+    col_scale [3, N], cs_splits = the first two row counts; two parts get an empty third range),
+    `interleave=True` alternates the rows of two equally sized ones (gate, up: row 2i = gate i,
+    row 2i+1 = up i; col_scale [2, N] by row parity).  The parts are row-major, fixed-stride and
+    share layout, code width, group and survivors per block."""
+    parts = list(parts)
+    p0 = parts[0]
+    if interleave and len(parts) != 2:
+        raise ValueError("interleaving takes exactly two matrices")
+    if not interleave and not 2 <= len(parts) <= 3:
+        raise ValueError("concatenation takes two or three matrices")
+    for p in parts:
+        if p.tiled or "row_off" in p.offs:
+            raise ValueError("fuse the row-major, fixed-stride form")
+        if (p.N, p.layout, p.bits, p.group, p.keep) != (p0.N, p0.layout, p0.bits, p0.group, p0.keep):
+            raise ValueError("the parts must share N, layout, bits, group and keep")
+        if p.cs_rows != 1:
+            raise ValueError("every part carries one col_scale vector")
+    stride = row_stride(p0.layout, p0.N, p0.bits, p0.group, p0.keep or None)
+    rows = [p.array("data")[: p.K * stride].view(p.K, stride) for p in parts]
+    sc = [p.array("scale").view(p.K, p.G) for p in parts]
+    zp = [p.array("zero").view(p.K, p.G) for p in parts]
+    cs = torch.stack([p.array("col_scale").view(p.N) for p in parts])
+    if interleave:
+        if parts[0].K != parts[1].K:
+            raise ValueError("interleaving needs equally many rows")
+        il = lambda a, b: torch.stack([a, b], 1).reshape(2 * a.shape[0], a.shape[1])
+        data, scale, zero = il(*rows), il(*sc), il(*zp)
+        splits = (0, 0)
+    else:
+        data, scale, zero = torch.cat(rows), torch.cat(sc), torch.cat(zp)
+        if len(parts) == 2:
+            cs = torch.cat([cs, cs[1:]])
+        splits = (parts[0].K, parts[1].K)
+    K = data.shape[0]
+    tail = torch.zeros(BLOB_TAIL, dtype=torch.uint8, device=data.device)
+    out = from_arrays(torch.cat([data.reshape(-1), tail]), scale.contiguous(), zero.contiguous(), cs, K, p0.N,
+                      p0.layout, p0.bits, p0.group, p0.keep or None, cs_splits=splits, device=data.device)
+    out.n_survivors = sum(p.n_survivors for p in parts)
+    return out
+
+
 def synth_packed(K: int, N: int, layout: int, bits=None, group=None, keep=None, seed: int = 0,
                  device="cpu", cs_rows: int = 1) -> PackedMatrix:
     """A VALID packed matrix with random content, made directly in packed form (the idea of

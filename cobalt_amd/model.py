@@ -17,6 +17,7 @@ from typing import Callable, Dict, Iterable, List, Optional, Sequence, Tuple
 import torch
 import torch.nn as nn
 
+from . import format as F
 from .linear import CobaltLinear
 
 # names inside a decoder block (src/cobaltkernel/quantize_cobalt.py:30-38)
@@ -41,7 +42,7 @@ def decoder_blocks(model: nn.Module) -> List[Tuple[str, nn.Module]]:
     """(qualified name, module) of every block that has all seven linears, in model order."""
     out = []
     for name, mod in model.named_modules():
-        if all(isinstance(_sub(mod, l), (nn.Linear, CobaltLinear)) for l in LINEARS):
+        if all(isinstance(_sub(mod, l), (nn.Linear, CobaltLinear, FusedPart)) for l in LINEARS):
             out.append((name, mod))
     return out
 
@@ -88,6 +89,7 @@ def compress_model(model: nn.Module, calib_ids: Optional[torch.Tensor] = None, s
                    batch_size: int = 4, device_order: bool = True,
                    bits_override: Optional[Dict[str, int]] = None,
                    sparsity_override: Optional[Dict[str, float]] = None, seq_inputs: bool = False,
+                   fuse: bool = False,
                    forward: Optional[Callable[[nn.Module, torch.Tensor], object]] = None) -> Dict[str, dict]:
     """Replace the linears of every decoder block by `CobaltLinear` modules compressed against
     the calibration tokens `calib_ids` [n, seq] (None: no calibration, H = I).  Per-matrix
@@ -95,7 +97,8 @@ def compress_model(model: nn.Module, calib_ids: Optional[torch.Tensor] = None, s
     (quantize_cobalt.py:330-352).  The Hessians come from the dense model's activations: the new
     modules are installed when all blocks are done; with `seq_inputs` every pass of
     `layers_per_pass` blocks is installed at once and later passes calibrate on the compressed
-    prefix (quantize_cobalt.py:444-452).  Returns {qualified linear name: {shape, layout, bpw,
+    prefix (quantize_cobalt.py:444-452).  `fuse` row-fuses q|k|v and gate/up afterwards (fuse_model).
+    Returns {qualified linear name: {shape, layout, bpw,
     bits, sparsity}}."""
     blocks = decoder_blocks(model)
     if not blocks:
@@ -146,9 +149,101 @@ def compress_model(model: nn.Module, calib_ids: Optional[torch.Tensor] = None, s
         if seq_inputs:
             install()
     install()
+    if fuse:
+        fuse_model(model, device_order)
     if was_training:
         model.train()
     return report
+
+
+class FusedRows(nn.Module):
+    """One packed matrix for several linears that read the same activation (q|k|v concatenated,
+    gate/up interleaved): one kernel launch instead of two or three, and a prefill GEMM that
+    fills the chip where k and v alone are too small to.  The decoder block keeps calling its
+    `q_proj`, `k_proj`, ... ; they are `FusedPart` views that run the fused matrix on the first
+    call with a new activation tensor and hand out column slices of that result."""
+
+    def __init__(self, fused: CobaltLinear, slices: Sequence[Tuple[int, int, int]]):
+        super().__init__()
+        self.fused = fused
+        self.slices = [tuple(s) for s in slices]                     # (start, stop, step) along the output
+        self._x = None
+        self._xv = -1
+        self._y = None
+        self._served = 0
+
+    def part(self, x: torch.Tensor, idx: int) -> torch.Tensor:
+        if self._x is not x or self._xv != x._version:
+            self._x, self._xv, self._served = x, x._version, 0
+            self._y = self.fused(x)
+        lo, hi, st = self.slices[idx]
+        y = self._y[..., lo:hi:st]
+        self._served += 1
+        if self._served >= len(self.slices):                          # every part has been asked for: let go
+            self._x = self._y = None
+            self._xv = -1
+        return y
+
+
+class FusedPart(nn.Module):
+    def __init__(self, owner: FusedRows, idx: int, in_features: int, out_features: int):
+        super().__init__()
+        self.__dict__["_owner"] = owner                               # not a submodule: the first part registers it
+        self.idx, self.in_features, self.out_features = idx, in_features, out_features
+        if idx == 0:
+            self.rows = owner
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self._owner.part(x, self.idx)
+
+
+def _fuse_group(blk: nn.Module, names: Sequence[str], interleave: bool, device_order: bool) -> bool:
+    mods = [_sub(blk, n) for n in names]
+    if not all(isinstance(m, CobaltLinear) for m in mods):
+        return False
+    pms = [m.packed() for m in mods]
+    try:
+        fused_pm = F.fuse_rows(pms, interleave=interleave)
+    except ValueError:
+        return False                                                  # e.g. per-matrix overrides: leave them apart
+    bias = None
+    if any(m.bias is not None for m in mods):
+        bs = [m.bias.data if m.bias is not None else torch.zeros(m.out_features, device=m.blob.device, dtype=torch.float16)
+              for m in mods]
+        bias = torch.stack(bs, 1).reshape(-1) if interleave else torch.cat(bs)
+    fused = CobaltLinear(fused_pm, bias)
+    if device_order and fused.blob.is_cuda:
+        fused.to_device_order()
+    if interleave:
+        slices = [(0, fused_pm.K, 2), (1, fused_pm.K, 2)]
+    else:
+        edges = [0]
+        for p in pms:
+            edges.append(edges[-1] + p.K)
+        slices = [(edges[i], edges[i + 1], 1) for i in range(len(pms))]
+    owner = FusedRows(fused, slices)
+    for i, n in enumerate(names):
+        setattr(_sub(blk, n.rsplit(".", 1)[0]), n.rsplit(".", 1)[1], FusedPart(owner, i, pms[i].N, pms[i].K))
+    return True
+
+
+def fuse_model(model: nn.Module, device_order: bool = True) -> int:
+    """Fuse q|k|v and gate/up of every decoder block whose linears are row-major or device-order
+    `CobaltLinear` modules with matching configurations.  Returns the number of fused groups."""
+    n = 0
+    for _bname, blk in decoder_blocks(model):
+        for names, il in ((HGROUPS["attn_in"], False), (HGROUPS["mlp_in"], True)):
+            mods = [_sub(blk, x) for x in names]
+            if all(isinstance(m, CobaltLinear) for m in mods):
+                for m in mods:                                       # fusing works on the row-major bytes
+                    pm = m._pm()
+                    if pm.tiled:
+                        t = pm.to_rowmajor()
+                        m._buffers["blob"] = t.blob
+                        m._buffers["cbk_meta"] = m._meta_of(t)
+                        m._pm_cache = None
+                n += 1 if _fuse_group(blk, names, il, device_order) else 0
+    return n
 
 
 def dense_twin(model: nn.Module, dtype: Optional[torch.dtype] = None) -> nn.Module:

@@ -57,3 +57,33 @@ def test_compressed_model_state_dict_round_trip():
     ids = torch.randint(0, 512, (1, 5), generator=torch.Generator().manual_seed(2)).to(DEV)
     with torch.no_grad():
         assert torch.equal(m(ids).logits, m2(ids).logits)
+
+
+def test_fused_qkv_and_gate_up_match_the_separate_modules():
+    """`fuse=True`: q|k|v become one matrix with three col_scale vectors, gate/up one with two by
+    row parity; the block still calls its seven projections, three launches fewer per block."""
+    from cobalt_amd import model as Mo
+    from cobalt_amd.linear import CobaltLinear
+    m = _tiny_mistral()
+    g = torch.Generator().manual_seed(1)
+    calib = torch.randint(0, 512, (8, 64), generator=g).to(DEV)
+    Mo.compress_model(m, calib)
+    f = copy.deepcopy(m)
+    assert Mo.fuse_model(f) == 4
+    packed = [x for x in f.modules() if isinstance(x, CobaltLinear)]
+    assert len(packed) == 2 * 4                                       # per block: qkv, o, gate/up, down
+    assert sorted(x._pm().cs_rows for x in packed) == [1, 1, 1, 1, 2, 2, 3, 3]
+    twin = Mo.dense_twin(copy.deepcopy(f), torch.float16)
+    for shape in ((1, 300), (2, 12), (1, 1), (2, 1)):
+        ids = torch.randint(0, 512, shape, generator=g).to(DEV)
+        with torch.no_grad():
+            a, b, c = f(ids).logits.float(), m(ids).logits.float(), twin(ids).logits.float()
+        assert float((a - c).norm() / c.norm()) < 5e-3, shape
+        assert float((a - b).norm() / b.norm()) < 5e-3, shape
+    # a second call with new contents in the same tensor object must not see the cached result
+    ids = torch.randint(0, 512, (1, 4), generator=g).to(DEV)
+    with torch.no_grad():
+        y1 = f(ids).logits.clone()
+        ids.copy_(torch.randint(0, 512, (1, 4), generator=g).to(DEV))
+        y2 = f(ids).logits
+        assert not torch.equal(y1, y2) and float((y2.float() - m(ids).logits.float()).norm()) < 5e-3 * float(y2.float().norm())

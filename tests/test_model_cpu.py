@@ -100,3 +100,41 @@ def test_packed_forward_fails_loudly_without_a_gpu():
     if not torch.cuda.is_available():
         with pytest.raises(Exception):
             m(torch.randint(0, 64, (1, 4)))
+
+
+def test_fuse_rows_layouts():
+    """q|k|v concatenation and gate/up interleaving of packed matrices, checked on the bytes."""
+    a, b, c = (F.synth_packed(K, 256, F.BLK1632_4, seed=i) for i, K in enumerate((32, 16, 16)))
+    f = F.fuse_rows([a, b, c])
+    st = F.row_stride(F.BLK1632_4, 256)
+    assert (f.K, f.cs_rows, f.cs_splits) == (64, 3, (32, 16))
+    assert torch.equal(f.array("data")[32 * st: 48 * st], b.array("data")[: 16 * st])
+    assert torch.equal(f.array("scale").view(64, 2)[48:], c.array("scale").view(16, 2))
+    assert torch.equal(f.array("col_scale").view(3, 256)[1], b.array("col_scale").view(256))
+    g = F.fuse_rows([b, c], interleave=True)
+    assert (g.K, g.cs_rows) == (32, 2)
+    rows = g.array("data")[: 32 * st].view(32, st)
+    assert torch.equal(rows[0::2], b.array("data")[: 16 * st].view(16, st))
+    assert torch.equal(rows[1::2], c.array("data")[: 16 * st].view(16, st))
+    assert torch.equal(g.array("zero").view(32, 2)[1::2], c.array("zero").view(16, 2))
+    with pytest.raises(ValueError):
+        F.fuse_rows([a, b], interleave=True)                       # unequal row counts
+    with pytest.raises(ValueError):
+        F.fuse_rows([a, F.synth_packed(16, 256, F.DENSE4, seed=3)])
+
+
+def test_fuse_model_structure():
+    m = _Toy(layers=2)
+    Mo.compress_model(m, None, fuse=True)
+    blk = m.layers[0]
+    assert isinstance(blk.self_attn.q_proj, Mo.FusedPart) and isinstance(blk.mlp.up_proj, Mo.FusedPart)
+    assert isinstance(blk.self_attn.o_proj, CobaltLinear)
+    qkv = blk.self_attn.q_proj.rows.fused
+    assert (qkv.out_features, qkv.packed().cs_rows, qkv.packed().cs_splits) == (512, 3, (256, 128))
+    assert qkv.bias is not None and qkv.bias.shape == (512,)       # v_proj had a bias
+    assert float(qkv.bias[:384].abs().max()) == 0.0
+    gu = blk.mlp.gate_proj.rows.fused
+    assert (gu.out_features, gu.packed().cs_rows) == (768, 2)
+    keys = [k for k in m.state_dict() if k.startswith("layers.0.")]
+    assert sum(k.endswith("blob") for k in keys) == 4              # one packed image per fused group
+    assert len(Mo.decoder_blocks(m)) == 2
