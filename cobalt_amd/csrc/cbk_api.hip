@@ -197,8 +197,13 @@ size_t cbk_workspace_bytes(const cbk_desc* in, int M) {
   if (M >= 1 && M <= 16 && gemv_fast_takes(m, 1)) return gemv_fast_workspace(m, 1);
   if (gemm_big_takes(m, M)) return gemm_big_workspace(m, M);
   int lo[3], hi[3], row[3];
-  if (M > 128 && fused_ranges(m, lo, hi, row)) return gemm_big_workspace(row_range(m, lo[0], hi[0], row[0]), M);
-  return 0;
+  const int nr = M > 128 ? fused_ranges(m, lo, hi, row) : 0;
+  size_t need = 0;
+  for (int i = 0; i < nr; ++i) {                                    // run one after the other on the same bytes
+    const size_t b = gemm_big_workspace(row_range(m, lo[i], hi[i], row[i]), M);
+    need = need > b ? need : b;
+  }
+  return need;
 }
 
 size_t cbk_gemv_batch_workspace_bytes(int n, const cbk_desc* descs, int M) {

@@ -60,6 +60,12 @@ struct GbArgs {
   // q|k|v matrix whose ranges start on row tiles: rows from vs0 on use the second X', rows from
   // vs1 on the third (both INT_MAX for any other matrix)
   int vs0, vs1;
+  // split of the column range (PAR 3): nsplit workgroups per output tile take nst_part stages
+  // each and leave float32 partial tiles [nsplit][.][part_ld] at part; a second kernel adds them
+  int nsplit, nst_part;
+  float* part;
+  size_t part_stride;      // elements between the partial matrices
+  int64_t part_ld;
 };
 
 // One wavefront-wide copy of 64 x 16 bytes from global memory straight into LDS (no VGPRs, no
@@ -151,6 +157,7 @@ __device__ inline void gb_epilogue(const GbArgs& a, v16f (&acc)[4][4], uint8_t* 
 // BITS 2 / 3 / 4: byte-permute decoder for (BITS, KEEP, GRP), KEEP = 0 for the dense layouts.
 // BITS 0: generic 32-column reader, any fixed-stride layout.
 // PAR 0: one col_scale vector.  1: gate/up matrix (GbArgs::par).  2: q|k|v matrix (GbArgs::vs0, vs1).
+// 3: one col_scale vector, column range split over several workgroups (GbArgs::nsplit).
 // Three instantiations rather than run-time switches: the schedule of the main loop is tuned
 // to the instruction and measurably shifts with every value that is added to it.
 template <int BITS, int KEEP, int GRP, int PAR>
@@ -168,17 +175,23 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wt = wave >> 1, wr = wave & 1;
   // XCD-aware order: blockIdx % 8 picks the XCD; give each XCD whole token tiles
-  const int nb = a.tiles_t * a.tiles_r;
+  constexpr bool SPLIT = PAR == 3;
+  const int nb = a.tiles_t * a.tiles_r * (SPLIT ? a.nsplit : 1);
   const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
   const int per = (nb + 7) >> 3;
   const int lin = xcd * per + idx;                                 // token-tile-major linear id
   if (lin >= nb) return;
-  const int tt = lin / a.tiles_r, tr = lin % a.tiles_r;
+  const int part = SPLIT ? lin % a.nsplit : 0, tile = SPLIT ? lin / a.nsplit : lin;
+  const int tt = tile / a.tiles_r, tr = tile % a.tiles_r;
   constexpr int kstep = PAR == 1 ? 2 : 1;                         // row stride of this workgroup's rows
   const int pp = PAR == 1 ? (tr & 1) : 0;                         // and their parity
   const int t0 = tt * GB_T, r0 = PAR == 1 ? (tr >> 1) * (2 * GB_R) + pp : tr * GB_R;
   const int N = m.N, Npad = a.Npad;
-  const int nst = Npad / GB_K;                                    // a multiple of 4; stages past N see X' = 0
+  // stages of this workgroup: all of them, or its part of them; a multiple of 4 either way;
+  // stages past N see X' = 0
+  const int s_begin = SPLIT ? part * a.nst_part : 0;
+  const int nst = SPLIT ? (Npad / GB_K - s_begin < a.nst_part ? Npad / GB_K - s_begin : a.nst_part) : Npad / GB_K;
+  const int c_begin = s_begin >> 1;                               // first 128-column chunk
   const int nch = N >> 7;                                         // 128-column chunks of the weight rows
 
   if (BITMAP) {
@@ -210,7 +223,7 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   const uint32_t xvo_e = (uint32_t)((lane >> 3) * Npad * 2 + (((lane & 7) ^ (lane >> 4)) * 16));
   const uint32_t xvo_o = (uint32_t)((lane >> 3) * Npad * 2 + (((lane & 7) ^ (4 + (lane >> 4))) * 16));
   const int xv = PAR == 1 ? pp : PAR == 2 ? (r0 >= a.vs0 ? 1 : 0) + (r0 >= a.vs1 ? 1 : 0) : 0;   // which col_scale vector
-  const uint8_t* xsb = (const uint8_t*)(a.xp + (size_t)xv * a.xps + (size_t)(t0 + 64 * wv) * Npad);
+  const uint8_t* xsb = (const uint8_t*)(a.xp + (size_t)xv * a.xps + (size_t)(t0 + 64 * wv) * Npad + (size_t)s_begin * GB_K);
   const uint32_t xlds0 = (uint32_t)(uintptr_t)Xs + (uint32_t)wv * 8192u;
   auto dma_x = [&](int s, int buf) {                              // stage s -> Xs[buf]
     const uint8_t* sb = xsb + (size_t)s * (GB_K * 2);
@@ -239,6 +252,7 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
 
   auto load_chunk = [&](int c, WChunk& w) {
     if (!FASTD) return;
+    c += c_begin;
     c = c < nch ? c : nch - 1;
     w.ci = (uint32_t)c;
     if (BITMAP) {
@@ -275,7 +289,7 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
       uint32_t packed[16];
       if (wok) {
         int q[32];
-        int t = (s * GB_K >> 5) + (b8 >> 2);
+        int t = ((s + s_begin) * GB_K >> 5) + (b8 >> 2);
         t = t < (N >> 5) ? t : (N >> 5) - 1;
         const uint32_t keep = decode_block32(m, rv, t, q);
         const int g = (t * BLOCK) / m.group;
@@ -446,6 +460,14 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   __syncthreads();
 
   const int tok0 = t0 + 128 * wt, row0 = r0 + kstep * 128 * wr;
+  if (SPLIT) {                                                    // float32 partial tile, no bias
+    GbArgs b = a;
+    b.y = a.part + (size_t)part * a.part_stride;
+    b.ldy = a.part_ld;
+    b.bias = nullptr;
+    gb_epilogue<CBK_F32, 1>(b, acc, smem, lane, wave, tok0, row0);
+    return;
+  }
   if (a.ydt == CBK_F32) gb_epilogue<CBK_F32, kstep>(a, acc, smem, lane, wave, tok0, row0);
   else if (a.ydt == CBK_F16) gb_epilogue<CBK_F16, kstep>(a, acc, smem, lane, wave, tok0, row0);
   else gb_epilogue<CBK_BF16T, kstep>(a, acc, smem, lane, wave, tok0, row0);
@@ -468,6 +490,7 @@ template <int BITS, int KEEP, int GRP>
 static int launch_big_cfg(const GbArgs& a, int blocks, hipStream_t st) {
   if (a.par) return launch_big_par<BITS, KEEP, GRP, 1>(a, blocks, st);
   if (a.vs0 != 0x7fffffff) return launch_big_par<BITS, KEEP, GRP, 2>(a, blocks, st);
+  if (a.nsplit > 1) return launch_big_par<BITS, KEEP, GRP, 3>(a, blocks, st);
   return launch_big_par<BITS, KEEP, GRP, 0>(a, blocks, st);
 }
 

@@ -36,9 +36,68 @@ __global__ __launch_bounds__(256) void gemm_prep_kernel(const uint16_t* x, int64
 
 static inline int gb_npad(int N) { return (N + 255) / 256 * 256; }
 
+// ---- y = sum of the float32 partial tiles (+ bias), eight outputs per thread
+__global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float* part, size_t part_stride, int64_t part_ld,
+                                                               int nsplit, int M, int K, const void* bias, void* y,
+                                                               int ydt, int64_t ldy) {
+  const int k8 = (K + 7) >> 3;
+  const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (id >= (int64_t)M * k8) return;
+  const int tok = (int)(id / k8), k0 = (int)(id % k8) * 8;
+  float v[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = 0.f;
+  for (int p = 0; p < nsplit; ++p) {                                // fixed order: run-to-run identical
+    const float* src = part + (size_t)p * part_stride + (size_t)tok * part_ld + k0;
+    const float4 a = ((const float4*)src)[0], b = ((const float4*)src)[1];
+    v[0] += a.x; v[1] += a.y; v[2] += a.z; v[3] += a.w; v[4] += b.x; v[5] += b.y; v[6] += b.z; v[7] += b.w;
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int k = k0 + e;
+    if (k >= K) break;
+    float o = v[e];
+    if (bias) o += ydt == CBK_F32 ? ((const float*)bias)[k] : ydt == CBK_F16 ? h2f(((const uint16_t*)bias)[k]) : bf2f(((const uint16_t*)bias)[k]);
+    const size_t at = (size_t)tok * ldy + k;
+    if (ydt == CBK_F32) ((float*)y)[at] = o;
+    else if (ydt == CBK_F16) ((uint16_t*)y)[at] = f2h(o);
+    else ((uint16_t*)y)[at] = f2bf(o);
+  }
+}
+
+// How many workgroups share one output tile.  A launch of fewer tiles than a multiple of the
+// 256 CUs leaves CUs idle for a whole tile time; cutting the column range gives them work at
+// the price of the float32 partial tiles (written and read once).  Times in microseconds from
+// measurements of this kernel: 1.7 per stage and 10 per workgroup, 4 TB/s for the partials.
+static int gb_nsplit(const DMat& m, int M) {
+  const bool le128 = (m.flags & CBK_FLAG_ZERO_LE_128) != 0;
+  const int fam = family_of(m.layout);
+  if (m.cs_rows > 1 || !le128 || !(fam == FAM_BLK || fam == FAM_DENSE) || m.bits < 2 || m.bits > 4) return 1;
+  const int tiles = ((M + GB_T - 1) / GB_T) * ((m.K + GB_R - 1) / GB_R);
+  const int nst = gb_npad(m.N) / GB_K;
+  int best = 1;
+  double t1 = 0, best_t = 0;
+  for (int s = 1; s <= 8; ++s) {
+    const int per = ((nst + s - 1) / s + 3) / 4 * 4;                // stages per part, a multiple of 4
+    if (s > 1 && (s - 1) * per >= nst) continue;                    // a part would be empty
+    const double rounds = (double)((tiles * s + 255) / 256);
+    double t = rounds * (per * 1.7 + 10.0);
+    if (s > 1) t += 2.0 * s * (double)M * m.K * 4 / 4.0e6 + 5.0;
+    if (s == 1) t1 = best_t = t;
+    else if (t < best_t) { best = s; best_t = t; }
+  }
+  if (best_t > 0.93 * t1) best = 1;                                 // not worth a second kernel
+  return best;
+}
+
+static inline size_t gb_kpad(int K) { return (size_t)(K + 7) / 8 * 8; }
+
 size_t gemm_big_workspace(const DMat& m, int M) {
   const size_t mpad = (size_t)(M + GB_T - 1) / GB_T * GB_T;
-  return ((m.cs_rows > 1 ? m.cs_rows : 1) * mpad * gb_npad(m.N) * 2 + 255) & ~(size_t)255;
+  size_t b = ((m.cs_rows > 1 ? m.cs_rows : 1) * mpad * gb_npad(m.N) * 2 + 255) & ~(size_t)255;
+  const int ns = gb_nsplit(m, M);
+  if (ns > 1) b += ((size_t)ns * M * gb_kpad(m.K) * 4 + 255) & ~(size_t)255;
+  return b;
 }
 
 int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
@@ -62,9 +121,15 @@ int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, v
   a.par = par; a.xps = (size_t)Mpad * Npad;
   a.vs0 = m.cs_rows == 3 ? m.cs_split0 : 0x7fffffff;
   a.vs1 = m.cs_rows == 3 ? m.cs_split0 + m.cs_split1 : 0x7fffffff;
+  const int nst_all = Npad / GB_K;
+  a.nsplit = gb_nsplit(m, M);
+  a.nst_part = ((nst_all + a.nsplit - 1) / a.nsplit + 3) / 4 * 4;
+  a.part_ld = (int64_t)gb_kpad(m.K);
+  a.part_stride = (size_t)M * gb_kpad(m.K);
+  a.part = (float*)((uint8_t*)ws + (((size_t)(m.cs_rows > 1 ? m.cs_rows : 1) * Mpad * Npad * 2 + 255) & ~(size_t)255));
   a.tiles_t = (M + GB_T - 1) / GB_T;
   a.tiles_r = par ? 2 * ((m.K + 2 * GB_R - 1) / (2 * GB_R)) : (m.K + GB_R - 1) / GB_R;
-  const int nb = a.tiles_t * a.tiles_r;
+  const int nb = a.tiles_t * a.tiles_r * a.nsplit;
   const int blocks = ((nb + 7) / 8) * 8;
   const bool le128 = (m.flags & CBK_FLAG_ZERO_LE_128) != 0;
   const int fam = family_of(m.layout);
@@ -75,7 +140,16 @@ int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, v
     else if (m.bits == 3) rc = launch_gemm_big_b3(a, keep, m.group, blocks, st);
     else if (m.bits == 4) rc = launch_gemm_big_b4(a, keep, m.group, blocks, st);
   }
-  if (rc == CBK_ERR_UNSUPPORTED) rc = launch_big_cfg<0, 0, 128>(a, blocks, st);   // generic reader
+  if (rc == CBK_ERR_UNSUPPORTED) {
+    if (a.nsplit > 1) return CBK_ERR_UNSUPPORTED;                   // (gb_nsplit only splits what the cases above take)
+    rc = launch_big_cfg<0, 0, 128>(a, blocks, st);                  // generic reader
+  }
+  if (rc == CBK_OK && a.nsplit > 1) {
+    const int64_t items = (int64_t)M * ((m.K + 7) / 8);
+    hipLaunchKernelGGL(gemm_split_reduce_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st,
+                       (const float*)a.part, a.part_stride, a.part_ld, a.nsplit, M, m.K, bias, y, ydt, ldy);
+    if (hipGetLastError() != hipSuccess) rc = CBK_ERR_HIP;
+  }
   return rc;
 }
 

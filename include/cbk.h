@@ -121,7 +121,8 @@ size_t cbk_stream_bytes(const cbk_desc* d, size_t sparse_data_bytes);
 /* Device scratch needed by cbk_gemv / cbk_gemm / cbk_linear for M activation rows (0 for the
  * decode kernels; the prefill kernel for M > 128 keeps its pre-scaled fp16 activations there:
  * ceil(M/256)*256 * ceil(N/256)*256 * 2 bytes per col_scale vector, i.e. times cs_rows for a
- * fused matrix).  The workspace must be 256-byte aligned. */
+ * fused matrix, plus float32 partial outputs when the library splits the column range of a
+ * launch that would not fill the chip).  Ask, do not compute.  256-byte aligned. */
 size_t cbk_workspace_bytes(const cbk_desc* d, int M);
 
 /* Rows [row0, row0+nrows) of W_hat -> out[nrows, ld_out] in out_dtype, bit-exact float32
