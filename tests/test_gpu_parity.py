@@ -222,6 +222,24 @@ def test_gemv_rows_are_independent_of_batch_and_run_to_run_identical():
     assert torch.equal(ops.gemv(pm, x, out_dtype=torch.float32), y4)
 
 
+@pytest.mark.parametrize("case", [(F.BLK1632_4, 4, 128, 16), (F.BLKC, 3, 64, 10), (F.DENSE4, 4, 128, 0)], ids=case_id)
+def test_linear_ragged_and_extreme_shapes(case):
+    """One row, one chunk, row counts off the 16-row and 256-row tiles, column counts off the
+    512-column step, and a row too long for the decode kernel's activation staging: every
+    activation count from the decode kernel to the split prefill kernel."""
+    for (K, N) in ((1, 128), (17, 384), (33, 640), (257, 128), (300, 1152), (4, 28672)):
+        raw = make_raw(case, K, N, seed=K + N)
+        pk = oracle_pack(case, raw)
+        W = R.dequant(pk, K, N, case[0], col_scale=raw["col_scale"], **kw_of(case))
+        for tiled in (False, True):
+            pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV, tiled=tiled)
+            for M in (1, 4, 7, 17, 129, 300):
+                x = acts(M, N, torch.float16, seed=M)
+                ref = R.forward_ref(W, _np(x))
+                err = rel_fro(_np(ops.linear(pm, x.to(DEV), out_dtype=torch.float32)), ref)
+                assert err < TOL, f"{case_id(case)} {K}x{N} tiled={tiled} M={M}: {err}"
+
+
 # ------------------------------------------------------------------ row-fused matrices
 FUSED_CASES = [(F.BLK1632_4, 4, 128, 16), (F.BLKC, 3, 128, 10), (F.BLKC, 2, 64, 23), (F.DENSE4, 4, 128, 0)]
 
