@@ -50,6 +50,9 @@ constexpr int GV_THREADS = GV_WAVES * 64;
 constexpr int LUT_LANES = CBK_LUT_LANES;      // lane-private copies of the selector table
 constexpr int LUT_BYTES = 256 * LUT_LANES * 8;
 constexpr int ZERO_BYTES = 256;
+constexpr int CNT_SLOTS = 64;                 // most reduction slots (arrival counters)
+constexpr int GV_STATIC_ROUNDS = 3;           // items per wavefront that are dealt, not taken from the counter
+constexpr int CNT_BYTES = (CNT_SLOTS + 4) * 4; // counters and the item counter, at a fixed place
 constexpr int X_LDS_BUDGET = 112 * 1024;      // activation digits: M * 3 * N bytes (of 160 KB LDS)
 constexpr int NDIG = 3;                       // int8 digits per activation
 constexpr int GV_MAX_M = 4;
@@ -279,11 +282,27 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // in a scalar register: positions are scalar work
   uint2* lut = (uint2*)smem;
   uint8_t* zreg = smem + LUT_BYTES;
-  int8_t* xq = (int8_t*)(zreg + ZERO_BYTES);
+  int* cnt = (int*)(zreg + ZERO_BYTES);                // [CNT_SLOTS] arrival counters, then the item counter
+  int8_t* xq = (int8_t*)cnt + CNT_BYTES;
+  // Selector table, zero row and counters do not depend on the arguments: they are written
+  // while the argument block is on its way, and published by a barrier nobody waits long at.
+  {
+    using C0 = Cfg<BITS, KEEP, GRP, MP>;
+    if (tid < 256) {
+      const uint2 e = make_selectors((uint32_t)tid, C0::SEL_KIND);
+#pragma unroll
+      for (int j = 0; j < LUT_LANES; ++j) lut[tid * LUT_LANES + j] = e;
+    } else if (tid < 256 + ZERO_BYTES / 4) {
+      ((uint32_t*)zreg)[tid - 256] = 0u;
+    } else if (tid < 256 + ZERO_BYTES / 4 + CNT_SLOTS + 4) {
+      const int ci = tid - 256 - ZERO_BYTES / 4;                     // the two item counters start past the dealt items
+      cnt[ci] = ci >= CNT_SLOTS ? GV_STATIC_ROUNDS * GV_WAVES : 0;
+    }
+    __syncthreads();
+  }
   const GvHead h = b.h;
   float* delta = (float*)(xq + h.xq_cap);
   float* red = delta + h.delta_cap;                    // [nslot][sk_cap][M][16] partial sums
-  int* cnt = (int*)(red + h.red_floats);               // [nslot] arrival counters
 
   const int wr = lane & 15, kq = lane >> 4;            // weight row in tile / lane quarter
   const uint32_t l16 = lane & (LUT_LANES - 1);
@@ -298,6 +317,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
   const int c0 = bx * h.cq + (bx < h.cr ? bx : h.cr);
   const int c1 = c0 + h.cq + (bx < h.cr ? 1 : 0);
   bool first = true;
+  int mat_iter = 0;                                    // matrices this workgroup has started
   // first matrix with cost units at or after c0
   int mi0 = 0;
 #pragma unroll
@@ -413,8 +433,10 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     // through its last items alone, with nobody to hide its latencies.  Which wavefront sums
     // which item does not enter the result.
     struct Pos { int tl, part, S, k; };                            // k: items taken by this wavefront so far
-    constexpr int STATIC_ROUNDS = 3;
-    int* const next_item = cnt + h.nslot;
+    constexpr int STATIC_ROUNDS = GV_STATIC_ROUNDS;
+    // two item counters take turns: the one of the next matrix is reset while this one is in use,
+    // a barrier before anybody reads it and a barrier after everybody has stopped reading it
+    int* const next_item = cnt + CNT_SLOTS + (mat_iter & 1);
     const uint32_t inv_sk = 65536u / (uint32_t)SK + 1u;           // it / SK == (it * inv_sk) >> 16 for it < 4096, SK <= 16
     auto advance = [&](Pos& p) -> bool {                           // false past the last position
       const int s_end = (p.part * spi + spi < nS) ? p.part * spi + spi : nS;
@@ -452,19 +474,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 
     // ---- stage: selector table and counters (once), activation digits and deltas of this matrix
     if (!first) __syncthreads();                                  // previous matrix fully consumed
-    if (tid == 0) *next_item = STATIC_ROUNDS * GV_WAVES;
-    if (first) {
-      if (tid < 256) {
-        const uint2 e = make_selectors((uint32_t)tid, C::SEL_KIND);
-#pragma unroll
-        for (int j = 0; j < LUT_LANES; ++j) lut[tid * LUT_LANES + j] = e;
-      } else if (tid < 256 + ZERO_BYTES / 4) {
-        ((uint32_t*)zreg)[tid - 256] = 0u;
-      } else if (tid < 256 + ZERO_BYTES / 4 + h.nslot) {
-        cnt[tid - 256 - ZERO_BYTES / 4] = 0;
-      }
-      first = false;
-    }
+    if (tid == 0) cnt[CNT_SLOTS + ((mat_iter + 1) & 1)] = STATIC_ROUNDS * GV_WAVES;
+    ++mat_iter;
+    first = false;
     while (xit < xitems) {
       stage_convert<(!C::DENSE ? 0 : (BITS == 2 ? 2 : 1))>(xl, m.cs != nullptr, h.xdt, N, n16, xit, MP == 1, xq, delta);
       xit += GV_THREADS;
@@ -793,8 +805,8 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
   while (nslot > 2 && (size_t)nslot * slot_floats * 4 > 24 * 1024) nslot >>= 1;
   gb.h.sk_cap = sk_cap; gb.h.nslot = nslot; gb.h.red_floats = nslot * slot_floats;
   gb.h.cq = cost / blocks; gb.h.cr = cost % blocks;
-  const size_t lds = (size_t)LUT_BYTES + ZERO_BYTES + xq_cap + (size_t)delta_cap * 4 +
-                     (size_t)gb.h.red_floats * 4 + (size_t)nslot * 4 + 16;   // + the item counter
+  const size_t lds = (size_t)LUT_BYTES + ZERO_BYTES + CNT_BYTES + xq_cap + (size_t)delta_cap * 4 +
+                     (size_t)gb.h.red_floats * 4;
   const int bits = gb.mat[0].m.bits;
   return bits == 2 ? launch_keep<2>(gb, lds, blocks, st) : bits == 3 ? launch_keep<3>(gb, lds, blocks, st)
        : bits == 4 ? launch_keep<4>(gb, lds, blocks, st) : CBK_ERR_UNSUPPORTED;
