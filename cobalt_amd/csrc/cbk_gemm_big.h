@@ -130,11 +130,7 @@ __device__ inline void gb_epilogue(const GbArgs& a, v16f (&acc)[4][4], uint8_t* 
         uint8_t* d = epl + (8 * (r >> 2) + (r & 3)) * PITCH + 32 * j * ESZ;
         if (YDT == CBK_F32) *(float*)d = v;
         else if (YDT == CBK_F16) *(uint16_t*)d = f2h(v);
-        else {
-          const uint32_t u = __float_as_uint(v);
-          const uint32_t rn = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-          *(uint16_t*)d = (uint16_t)(((u & 0x7fffffffu) > 0x7f800000u) ? ((u >> 16) | 0x40u) : rn);
-        }
+        else *(__bf16*)d = (__bf16)v;                              // v_cvt_pk_bf16_f32: round to nearest even
       }
 #pragma unroll
     for (int t = 0; t < 32 * PPR / 64; ++t) {
