@@ -4,9 +4,12 @@ Decode (the `value` of the JSON line).  One "step" is one pass of the hot path o
 decoder-layer set: the seven M-row GEMVs of a layer (q, k, v, o, gate, up, down) at sparsity
 0.5, 4-bit codes, group 128 (layout BLK1632_4, 3.1875 bits per weight), launched as the four
 dependency phases of a decoder layer (q,k,v | o | gate,up | down), one batched kernel launch
-per phase, replayed from HIP graphs.  The packed weights of several distinct layer sets are
-resident in HBM before the timed region; successive steps rotate through them so that the
-streamed set exceeds twice the 256 MB Infinity Cache.  `value` is algorithmic bytes (packed
+per phase, replayed from HIP graphs: one graph holds about 32 steps in a row, as a decoder
+replays all its layers for a token in one graph (a replay boundary costs several microseconds
+on the GPU; single-step graphs serve the remainder, so that exactly K steps are timed).  The
+packed weights of several distinct layer sets are resident in HBM before the timed region;
+successive steps rotate through them so that the streamed set exceeds twice the 256 MB
+Infinity Cache.  `value` is algorithmic bytes (packed
 rows + scales + zeros + col_scale + activations in + outputs out) streamed per second.
 
 `roofline` describes the decode kernel: algorithmic bytes per launch over the average launch
@@ -137,8 +140,8 @@ def prefill_gemm(torch, F, ops, dev, workload, layout, bits, group, keep, M, dt,
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--workload", default="mistral7b", choices=list(SHAPES))
     ap.add_argument("--m", type=int, default=1)
     ap.add_argument("--dtype", default="f16", choices=["f16", "bf16"])
@@ -231,6 +234,7 @@ def main():
             step(i)
         stream.synchronize()
         graphs = None
+        per_graph = 0
         if not a.no_graph:                                      # one HIP graph per distinct layer set
             graphs = []
             for i in range(n_copies):
@@ -238,14 +242,33 @@ def main():
                 with torch.cuda.graph(g, stream=stream):
                     step(i)
                 graphs.append(g)
+            # and one graph of about 32 layer sets in a row (whole rotations of the distinct sets),
+            # as a decoder replays all its layers per token
+            per_graph = -(-32 // n_copies) * n_copies
+            g_all = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g_all, stream=stream):
+                for i in range(per_graph):
+                    step(i)
         run = (lambda i: graphs[i % n_copies].replay()) if graphs else step
-        for i in range(a.warmup):
-            run(i)
+
+        def run_steps(first, count):                             # exactly `count` steps, layer sets in rotation
+            i = first
+            while count > 0:
+                if graphs and i % n_copies == 0 and count >= per_graph:
+                    g_all.replay()
+                    i += per_graph
+                    count -= per_graph
+                else:
+                    run(i)
+                    i += 1
+                    count -= 1
+            return i
+
+        nxt = run_steps(0, a.warmup)
         stream.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(stream)
-        for i in range(a.steps):
-            run(a.warmup + i)
+        run_steps(nxt, a.steps)
         e1.record(stream)
         stream.synchronize()
         ms_per_step = e0.elapsed_time(e1) / a.steps
@@ -276,13 +299,15 @@ def main():
                                f"{bpw:.4f} bpw",
                    "layer_set_bytes": step_bytes, "distinct_layer_sets": n_copies,
                    "launches_per_step": launches, "launch_grouping": a.launch,
-                   "hip_graph": not a.no_graph, "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
+                   "hip_graph": not a.no_graph,
+                   "steps_per_graph_replay": (per_graph if not a.no_graph else 0), "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC.get((a.workload, a.launch, M)),
                      "kernel": "cbk::gemv_mfma_kernel", "avg_launch_us": round(us_per_launch, 3),
                      "launches_timed": a.steps * launches, "bytes_per_launch": int(bytes_per_launch)},
     }
+    g_all = None
     del graphs, sets, calls, keep_alive
     torch.cuda.empty_cache()
     if not a.no_prefill:
