@@ -224,8 +224,7 @@ __device__ inline void fetch_selectors(uint32_t mw, const uint2* lut, uint32_t l
 
 // Sixteen columns (half `half` of the block whose code stream is st) as signed bytes q - zero,
 // pruned columns 0: the B operand of one MFMA.
-// The selectors of the block's four mask bytes (sel) were read from the table earlier, so that
-// the LDS latency is not waited for here.
+// sel4: the selectors of the block's four mask bytes, read from the table by fetch_selectors.
 template <class C, int BITS>
 __device__ inline void decode_half(const uint32_t (&st)[C::NW], const uint32_t (&rk)[4], const uint2 (&sel4)[4],
                                    uint32_t nz, int half, uint32_t (&bfrag)[4]) {
@@ -323,8 +322,11 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 #pragma unroll
   for (int i = 0; i < GV_MAX_BATCH; ++i) mi0 += (i < h.n && h.cost_end[i] <= c0) ? 1 : 0;
 
+  // The first record is requested together with the header: most workgroups start with it, and
+  // for them the second round trip through the argument block before any load goes out is gone.
+  GvMat gm = b.mat[0];
   for (int mi = mi0; mi < h.n; ++mi) {
-    const GvMat gm = b.mat[mi];                                   // one read of the whole record
+    if (mi != 0) gm = b.mat[mi];                                  // one read of the whole record
     if (gm.cost0 >= c1) break;                                    // uniform over the workgroup
     const DMat& m = gm.m;
     const int nS = gm.nS;
@@ -554,17 +556,11 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 #pragma unroll
         for (int p = 0; p < MP; ++p) acc[p] = (v4i){0, 0, 0, 0};
 
-        // selector reads run one block ahead of the permutes; with one activation row the A
-        // fragment is read one MFMA ahead as well
-        constexpr bool APF = MP == 1;
-        uint32_t rkb[2][4];
-        uint2 selb[2][4];
-        fetch_selectors<C>(cur.mk[0], lut, l16, rkb[0], selb[0]);
-        v4i avn = (v4i){0, 0, 0, 0};
-        if (APF) avn = *(const v4i*)(smem + aaddr[0]);
 #pragma unroll
         for (int jb = 0; jb < 4; ++jb) {
-          if (jb < 3) fetch_selectors<C>(cur.mk[jb + 1], lut, l16, rkb[(jb + 1) & 1], selb[(jb + 1) & 1]);
+          uint32_t rkc[4];
+          uint2 selc[4];
+          fetch_selectors<C>(cur.mk[jb], lut, l16, rkc, selc);
           uint32_t st[C::NW];                                     // code stream of block jb
           block_stream<C, BITS>(cw, jb, st);
           const uint32_t z = (C::NGC == 1) ? cur.zraw : ((cur.zraw >> (8 * (jb >> 1))) & 0xFFu);
@@ -572,14 +568,12 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
             const int t = 2 * jb + half;                            // fragment index in the chunk
-            const v4i av0 = avn;
-            if (APF && t < 7) avn = *(const v4i*)(smem + aaddr[0] + 16 * (t + 1));
             uint32_t bfrag[4];
-            decode_half<C, BITS>(st, rkb[jb & 1], selb[jb & 1], nz, half, bfrag);
+            decode_half<C, BITS>(st, rkc, selc, nz, half, bfrag);
             const v4i bv = (v4i){(int)bfrag[0], (int)bfrag[1], (int)bfrag[2], (int)bfrag[3]};
 #pragma unroll
             for (int p = 0; p < MP; ++p) {
-              const v4i av = APF ? av0 : *(const v4i*)(smem + aaddr[p] + 16 * t);
+              const v4i av = *(const v4i*)(smem + aaddr[p] + 16 * t);
               acc[p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bv, acc[p], 0, 0, 0);
               // One idle issue slot after every MFMA.  Without it some instantiations of this
               // kernel (register allocations in which the accumulator chain changes registers)
@@ -786,9 +780,9 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
   for (int i = n; i < GV_MAX_BATCH; ++i) gb.h.cost_end[i] = cost;
   gb.h.xq_cap = xq_cap; gb.h.delta_cap = delta_cap;
   int blocks = tiles < 256 ? tiles : 256;                       // one persistent workgroup per CU
-  // macro-steps per work item: about four items per wavefront over the whole launch, so that
+  // macro-steps per work item: about two items per wavefront over the whole launch, so that
   // the tail is short; a tile is split into at most 16 parts
-  int spi = cost / (blocks * GV_WAVES * 4);
+  int spi = cost / (blocks * GV_WAVES * 2);
   spi = spi < 1 ? 1 : (spi > 8 ? 8 : spi);
   int sk_cap = 1;
   for (int i = 0; i < n; ++i) {
