@@ -458,7 +458,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     Pos p0{wave / SK, wave % SK, (wave % SK) * spi, 0};
     bool v0 = wave < nitems;
     Pos p1 = p0; bool v1 = v0 && advance(p1);
-    Pos p2 = p1; bool v2 = v1 && advance(p2);
+    Pos p2 = p1; bool v2 = v1 && advance(p2);                     // known a step early: taking an item is an LDS round trip
     // The activation loads go out before the first weight loads: the weight prefetch of a whole
     // launch is tens of megabytes, and a request queued behind it would keep every wavefront
     // from decoding until that burst has drained.
@@ -466,12 +466,11 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     int xit = tid;
     XLoad xl;
     if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, MP == 1, gm.par, xl);
-    // Three load buffers rotate through the roles (being decoded, next, being loaded) by name:
-    // copying a buffer would wait for the loads that are still filling it.
-    // Configurations with long code streams or four activation rows keep one step in flight
-    // instead of two: three buffers would not fit the 128 registers of a 16-wavefront workgroup.
-    constexpr bool DEEP = C::NL <= 8 && (MP < 4 || QB);
-    Loads<C> LA, LB, LC;
+    // Two load buffers swap roles (being decoded, being loaded) by name: copying a buffer would
+    // wait for the loads that are still filling it.  One step of loads in flight per wavefront
+    // is the measured optimum (sixteen wavefronts per CU already cover the latency; a second
+    // step in flight made the Mistral layer set 8 % slower).
+    Loads<C> LA, LB;
     issue(t_lo + p0.tl, p0.S, LA);
 
     // ---- stage: selector table and counters (once), activation digits and deltas of this matrix
@@ -484,9 +483,6 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       xit += GV_THREADS;
       if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, MP == 1, gm.par, xl);
     }
-    // the second step of loads goes out only now: issued together with the first, the two
-    // bursts of all wavefronts interleave in the memory system and every first step lands late
-    if (DEEP) issue(t_lo + p1.tl, p1.S, LB);
     __syncthreads();
 
     int bars = 0;                                                 // group barriers passed so far
@@ -501,7 +497,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 #pragma unroll
         for (int p = 0; p < MP; ++p) ysum[p] = 0.f;
       }
-      if (DEEP) issue(t_lo + p2.tl, p2.S, tgt); else issue(t_lo + p1.tl, p1.S, tgt);
+      issue(t_lo + p1.tl, p1.S, tgt);
       if constexpr (QB) {
         const int a_m = wr >> 2;                                    // activation row of this lane's A row
         uint32_t zs[4];                                             // zero | scale << 8 of the groups 4S .. 4S+3
@@ -657,13 +653,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     };
     while (true) {
       if (!v0) break;
-      do_step(LA, DEEP ? LC : LB);
+      do_step(LA, LB);
       if (!v0) break;
       do_step(LB, LA);
-      if (DEEP) {
-        if (!v0) break;
-        do_step(LC, LB);
-      }
     }
     // every wave passes the same number of group barriers
     const int ngroups = ((t_hi - t_lo) + gt - 1) / gt;
@@ -780,9 +772,11 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
   for (int i = n; i < GV_MAX_BATCH; ++i) gb.h.cost_end[i] = cost;
   gb.h.xq_cap = xq_cap; gb.h.delta_cap = delta_cap;
   int blocks = tiles < 256 ? tiles : 256;                       // one persistent workgroup per CU
-  // macro-steps per work item: about two items per wavefront over the whole launch, so that
-  // the tail is short; a tile is split into at most 16 parts
-  int spi = cost / (blocks * GV_WAVES * 2);
+  // macro-steps per work item: about one and a half items per wavefront over the whole launch
+  // (the end of an item costs about as many instructions as a step; measured best between one
+  // and two); a tile is split into at most 16 parts, and into a power of two of them where the
+  // row is long enough: the items then spread evenly over the four SIMDs
+  int spi = (int)((long long)cost * 2 / ((long long)blocks * GV_WAVES * 3));
   spi = spi < 1 ? 1 : (spi > 8 ? 8 : spi);
   int sk_cap = 1;
   for (int i = 0; i < n; ++i) {
@@ -790,7 +784,11 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
     int s = spi;
     while ((g.nS + s - 1) / s > 16) ++s;
     g.sk = (g.nS + s - 1) / s;
+    int p2 = 1;
+    while (p2 < g.sk) p2 <<= 1;
+    if (p2 <= 16 && p2 <= g.nS) g.sk = p2;
     g.spi = (g.nS + g.sk - 1) / g.sk;                  // equal parts
+    g.sk = (g.nS + g.spi - 1) / g.spi;
     sk_cap = sk_cap > g.sk ? sk_cap : g.sk;
   }
   // reduction slots: as many as fit 24 KB, a power of two between 2 and 64
