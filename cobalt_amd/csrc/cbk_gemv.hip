@@ -19,10 +19,9 @@
 // the A operand therefore carry (activation row, quarter, digit) variants that are non-zero
 // in one quarter only, and the 16x16 result keeps the groups apart.  One persistent workgroup
 // of sixteen wavefronts per CU owns a contiguous range of row tiles; a tile is cut into up
-// to 16 column parts; a wavefront's first three (tile, part) items are fixed, the later ones it
-// takes from a counter in LDS.  There is no barrier per tile: the partial sums of a tile meet
-// in an LDS slot and the wavefront that arrives last adds them in part order, so results are
-// run-to-run identical and do not depend on which wavefront summed which item.
+// to 16 column parts and the (tile, part) items are dealt round-robin to the wavefronts.  There
+// is no barrier per tile: the partial sums of a tile meet in an LDS slot and the wavefront that
+// arrives last adds them in part order, so results are run-to-run identical.
 // For 2 <= M <= 4 the headline configurations put the lane quarters on the four 32-column
 // blocks of one chunk instead of on four chunks (see block_split_capable below), so that
 // every MFMA serves all activation rows; sums are formed in the same order as for M = 1, so
@@ -51,8 +50,7 @@ constexpr int LUT_LANES = CBK_LUT_LANES;      // lane-private copies of the sele
 constexpr int LUT_BYTES = 256 * LUT_LANES * 8;
 constexpr int ZERO_BYTES = 256;
 constexpr int CNT_SLOTS = 64;                 // most reduction slots (arrival counters)
-constexpr int GV_STATIC_ROUNDS = 3;           // items per wavefront that are dealt, not taken from the counter
-constexpr int CNT_BYTES = (CNT_SLOTS + 4) * 4; // counters and the item counter, at a fixed place
+constexpr int CNT_BYTES = CNT_SLOTS * 4;       // at a fixed place: zeroed before the arguments are read
 constexpr int X_LDS_BUDGET = 112 * 1024;      // activation digits: M * 3 * N bytes (of 160 KB LDS)
 constexpr int NDIG = 3;                       // int8 digits per activation
 constexpr int GV_MAX_M = 4;
@@ -281,7 +279,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // in a scalar register: positions are scalar work
   uint2* lut = (uint2*)smem;
   uint8_t* zreg = smem + LUT_BYTES;
-  int* cnt = (int*)(zreg + ZERO_BYTES);                // [CNT_SLOTS] arrival counters, then the item counter
+  int* cnt = (int*)(zreg + ZERO_BYTES);                // [CNT_SLOTS] arrival counters
   int8_t* xq = (int8_t*)cnt + CNT_BYTES;
   // Selector table, zero row and counters do not depend on the arguments: they are written
   // while the argument block is on its way, and published by a barrier nobody waits long at.
@@ -293,9 +291,8 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       for (int j = 0; j < LUT_LANES; ++j) lut[tid * LUT_LANES + j] = e;
     } else if (tid < 256 + ZERO_BYTES / 4) {
       ((uint32_t*)zreg)[tid - 256] = 0u;
-    } else if (tid < 256 + ZERO_BYTES / 4 + CNT_SLOTS + 4) {
-      const int ci = tid - 256 - ZERO_BYTES / 4;                     // the two item counters start past the dealt items
-      cnt[ci] = ci >= CNT_SLOTS ? GV_STATIC_ROUNDS * GV_WAVES : 0;
+    } else if (tid < 256 + ZERO_BYTES / 4 + CNT_SLOTS) {
+      cnt[tid - 256 - ZERO_BYTES / 4] = 0;
     }
     __syncthreads();
   }
@@ -316,7 +313,6 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
   const int c0 = bx * h.cq + (bx < h.cr ? bx : h.cr);
   const int c1 = c0 + h.cq + (bx < h.cr ? 1 : 0);
   bool first = true;
-  int mat_iter = 0;                                    // matrices this workgroup has started
   // first matrix with cost units at or after c0
   int mi0 = 0;
 #pragma unroll
@@ -337,7 +333,6 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     const int N = m.N, NCH = N >> 7;
     // items: tile tl (local), part j of SK; part j covers macro-steps [j*spi, min(nS,(j+1)*spi))
     const int SK = gm.sk, spi = gm.spi;
-    const int nitems = (t_hi - t_lo) * SK;
     const int gt = h.nslot >> 1;                                  // tiles per barrier group
 
     // matrix constants, read from the kernel arguments once
@@ -427,38 +422,23 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       }
     };
 
-    // This wave's sequence of (tile, part, macro-step) positions.  Its first three items are
-    // wave, wave + 16, wave + 32 (known without asking anybody, so that the first loads can go
-    // out before the workgroup has met at a barrier); every later item is the next one not yet
-    // taken, from a counter in LDS.  The wavefronts of a SIMD do not advance at the same pace
-    // (the oldest wins the issue arbitration), and with a fixed deal the slowest one would work
-    // through its last items alone, with nobody to hide its latencies.  Which wavefront sums
-    // which item does not enter the result.
-    struct Pos { int tl, part, S, k; };                            // k: items taken by this wavefront so far
-    constexpr int STATIC_ROUNDS = GV_STATIC_ROUNDS;
-    // two item counters take turns: the one of the next matrix is reset while this one is in use,
-    // a barrier before anybody reads it and a barrier after everybody has stopped reading it
-    int* const next_item = cnt + CNT_SLOTS + (mat_iter & 1);
-    const uint32_t inv_sk = 65536u / (uint32_t)SK + 1u;           // it / SK == (it * inv_sk) >> 16 for it < 4096, SK <= 16
+    // this wave's sequence of (tile, part, macro-step) positions: items wave, wave + 16, ...
+    // (taking the later items from a shared counter instead was measured: no faster at one step
+    // of loads in flight, slower on large launches)
+    struct Pos { int tl, part, S; };
+    const int ntl = t_hi - t_lo;
+    const int dq_t = GV_WAVES / SK, dq_p = GV_WAVES % SK;
     auto advance = [&](Pos& p) -> bool {                           // false past the last position
       const int s_end = (p.part * spi + spi < nS) ? p.part * spi + spi : nS;
       if (p.S + 1 < s_end) { ++p.S; return true; }
-      ++p.k;
-      int it = wave + GV_WAVES * p.k;
-      if (p.k >= STATIC_ROUNDS) {
-        int v = 0;
-        if (lane == 0) v = atomicAdd(next_item, 1);
-        it = __builtin_amdgcn_readfirstlane(v);
-      }
-      p.tl = it < 4096 ? (int)(((uint32_t)it * inv_sk) >> 16) : it / SK;
-      p.part = it - p.tl * SK;
+      p.tl += dq_t; p.part += dq_p;
+      if (p.part >= SK) { p.part -= SK; ++p.tl; }
       p.S = p.part * spi;
-      return it < nitems;
+      return p.tl < ntl;
     };
-    Pos p0{wave / SK, wave % SK, (wave % SK) * spi, 0};
-    bool v0 = wave < nitems;
+    Pos p0{wave / SK, wave % SK, (wave % SK) * spi};
+    bool v0 = p0.tl < ntl;
     Pos p1 = p0; bool v1 = v0 && advance(p1);
-    Pos p2 = p1; bool v2 = v1 && advance(p2);                     // known a step early: taking an item is an LDS round trip
     // The activation loads go out before the first weight loads: the weight prefetch of a whole
     // launch is tens of megabytes, and a request queued behind it would keep every wavefront
     // from decoding until that burst has drained.
@@ -475,8 +455,6 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 
     // ---- stage: selector table and counters (once), activation digits and deltas of this matrix
     if (!first) __syncthreads();                                  // previous matrix fully consumed
-    if (tid == 0) cnt[CNT_SLOTS + ((mat_iter + 1) & 1)] = STATIC_ROUNDS * GV_WAVES;
-    ++mat_iter;
     first = false;
     while (xit < xitems) {
       stage_convert<(!C::DENSE ? 0 : (BITS == 2 ? 2 : 1))>(xl, m.cs != nullptr, h.xdt, N, n16, xit, MP == 1, xq, delta);
@@ -648,8 +626,8 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
         }
       }
       }
-      p0 = p1; v0 = v1; p1 = p2; v1 = v2;
-      if (v2) v2 = advance(p2);
+      p0 = p1; v0 = v1;
+      if (v1) v1 = advance(p1);
     };
     while (true) {
       if (!v0) break;
