@@ -198,6 +198,19 @@ __device__ inline void stage_convert(const XLoad& r, bool has_cs, int xdt, int N
   if (c16 < 4) delta[row * (NCH + 4) + NCH + c16] = 0.f;          // chunks past N
 }
 
+// y(l) + y(l ^ 16), then that + the same of lane l ^ 32: the sum over the four lane quarters, in
+// every lane, with the two row-swap instructions of gfx950 instead of two trips through the LDS
+// crossbar.  (Through inline assembly: the compiler's builtin for the swaps returned the same
+// register for both results.)  The s_nop covers the wait states between a VALU write and the swap.
+__device__ inline float quarter_sum(float y) {
+  float a = y, b = y;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  const float t = a + b;
+  float c = t, d = t;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(c), "+v"(d));
+  return c + d;
+}
+
 // ------------------------------------------------------------------ one 32-column block
 // mask bytes of a block and the number of survivors before each of them
 template <class C>
@@ -576,8 +589,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
         // quarter kq holds activation row kq, one running sum per chunk position; added in the
         // order of the other decode path, so a row's result does not depend on M
         if (QB) { part_sum[p] = (ysum[0] + ysum[MP > 1 ? 1 : 0]) + (ysum[MP > 2 ? 2 : 0] + ysum[MP > 3 ? 3 : 0]); continue; }
-        const float h = ysum[p] + __shfl_xor(ysum[p], 16, 64);
-        part_sum[p] = h + __shfl_xor(h, 32, 64);
+        part_sum[p] = quarter_sum(ysum[p]);
       }
       auto store = [&](int om, int r, float v) {
         const int k = tile * 16 + r;
@@ -615,7 +627,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
         }
         int old = 0;
         if (lane == 0) old = atomicAdd(&cnt[slot], 1);
-        old = __shfl(old, 0, 64);
+        old = __builtin_amdgcn_readfirstlane(old);                 // lane 0 holds it, and every lane is active here
         if (old == SK - 1) {                                      // uniform over the wave
           for (int om = kq; om < h.M; om += 4) {
             float v = 0.f;
