@@ -346,7 +346,8 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     const int N = m.N, NCH = N >> 7;
     // items: tile tl (local), part j of SK; part j covers macro-steps [j*spi, min(nS,(j+1)*spi))
     const int SK = gm.sk, spi = gm.spi;
-    const int gt = h.nslot >> 1;                                  // tiles per barrier group
+    const int gt = h.nslot >> 1;                                  // tiles per barrier group, a power of two
+    const int gsh = 31 - __builtin_clz((unsigned)gt);               // its logarithm: no division per item
 
     // matrix constants, read from the kernel arguments once
     const uint8_t* const m_data = m.data;
@@ -484,7 +485,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       const int s_end = (part * spi + spi < nS) ? part * spi + spi : nS;
       if (S == part * spi) {                                      // first step of an item
         // slots of tile group g are reused by group g + 2: wait until group g - 1 is complete
-        for (const int g = tl / gt; bars < g; ++bars) __syncthreads();
+        for (const int g = tl >> gsh; bars < g; ++bars) __syncthreads();
 #pragma unroll
         for (int p = 0; p < MP; ++p) ysum[p] = 0.f;
       }
@@ -648,7 +649,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       do_step(LB, LA);
     }
     // every wave passes the same number of group barriers
-    const int ngroups = ((t_hi - t_lo) + gt - 1) / gt;
+    const int ngroups = ((t_hi - t_lo) + gt - 1) >> gsh;
     for (; bars < ngroups - 1; ++bars) __syncthreads();
   }
 }
