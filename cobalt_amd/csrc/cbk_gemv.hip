@@ -366,10 +366,13 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       const int rlim = m_K - 1 - tile * 16;                         // rows past K repeat row K - 1
       const uint32_t wrc = (uint32_t)(wr < rlim ? wr : rlim);
       const uint32_t lane_off = __umul24(wrc, lane_mul);
-      const uint8_t* const tb = m_data + (size_t)tile * tile_a;
-      const size_t sz_t = (size_t)tile * (size_t)(16 * m_G);
       const int klim = NCH - 1 - S4;                                // chunks past N repeat chunk NCH - 1
       const uint32_t chl = (uint32_t)(kq < klim ? kq : klim);
+      // Every address is one of the matrix's three base pointers plus a 32-bit offset (the host
+      // admits only matrices whose arrays are smaller than 4 GB): a scalar part that depends on
+      // (tile, S) and a lane part; one add per load, no 64-bit arithmetic per step.
+      const uint32_t so_t = (uint32_t)tile * tile_a;                 // scalar: start of the tile's rows
+      const uint32_t so_g = (uint32_t)tile * (uint32_t)(16 * m_G);   // scalar: first scale / zero of the tile
       if constexpr (QB) {
         // block kq of the chunks 4S .. 4S+3: one mask dword and CB / 8 code bytes each
         constexpr uint32_t BB = C::CB / 8;
@@ -379,8 +382,8 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
         for (int c = 0; c < 4; ++c) {
           int chc = S4 + c;
           chc = chc < NCH ? chc : NCH - 1;
-          if (!C::DENSE) L.mk[c] = *(const uint32_t*)(tb + ((size_t)chc << ush) + voff_m);
-          const uint8_t* cp = tb + ((size_t)(code_u0 + (uint32_t)chc * (C::CHB / 128)) << ush) + voff_c;
+          if (!C::DENSE) L.mk[c] = *(const uint32_t*)(m_data + (so_t + ((uint32_t)chc << ush) + voff_m));
+          const uint8_t* cp = m_data + (so_t + ((code_u0 + (uint32_t)chc * (C::CHB / 128)) << ush) + voff_c);
           if (C::CB == 32) {
             L.raw[c] = *(const uint32_t*)cp;
           } else if (C::CB == 64) {
@@ -392,23 +395,22 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
           }
         }
         // zero point and scale of group 4S + kq; the other quarters fetch them from this lane
-        const size_t gs = sz_t + ((size_t)S4 << csh);
-        const uint32_t gv = __umul24(wrc, sz_mul) + (chl << csh);
-        L.zraw = (uint32_t)(m_zero + gs)[gv] | ((uint32_t)(m_scale + gs)[gv] << 8);
+        const uint32_t gv = so_g + ((uint32_t)S4 << csh) + __umul24(wrc, sz_mul) + (chl << csh);
+        L.zraw = (uint32_t)m_zero[gv] | ((uint32_t)m_scale[gv] << 8);
         return;
       }
-      const uint8_t* const sb = tb + ((size_t)S4 << ush);
+      const uint32_t so_s = so_t + ((uint32_t)S4 << ush);            // scalar: unit 4S of the rows
       if (!C::DENSE) {
-        const uint4 v = *(const uint4*)(sb + (lane_off + (chl << ush)));
+        const uint4 v = *(const uint4*)(m_data + (so_s + lane_off + (chl << ush)));
         L.mk[0] = v.x; L.mk[1] = v.y; L.mk[2] = v.z; L.mk[3] = v.w;
       }
       // code bits of the chunk: bit ch*CHB of the code plane, fetched as whole 16-byte units
       if (C::VEC16) {
-        const uint8_t* const cb = tb + ((size_t)(code_u0 + (uint32_t)S4 * (C::CHB / 128)) << ush);
+        const uint32_t so_c = so_t + ((code_u0 + (uint32_t)S4 * (C::CHB / 128)) << ush);
         const uint32_t voff = lane_off + ((chl * (C::CHB / 128)) << ush);
 #pragma unroll
         for (int i = 0; i < C::NL / 4; ++i) {
-          const uint4 v = *(const uint4*)(cb + ((size_t)i << ush) + voff);
+          const uint4 v = *(const uint4*)(m_data + (so_c + ((uint32_t)i << ush) + voff));
           L.raw[4 * i] = v.x; L.raw[4 * i + 1] = v.y; L.raw[4 * i + 2] = v.z; L.raw[4 * i + 3] = v.w;
         }
       } else {
@@ -416,23 +418,19 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
         const uint32_t voff = lane_off + (u << ush);
 #pragma unroll
         for (int i = 0; i < C::NL / 4; ++i) {
-          const uint4 v = *(const uint4*)(tb + ((size_t)(code_u0 + i) << ush) + voff);
+          const uint4 v = *(const uint4*)(m_data + (so_t + ((code_u0 + (uint32_t)i) << ush) + voff));
           L.raw[4 * i] = v.x; L.raw[4 * i + 1] = v.y; L.raw[4 * i + 2] = v.z; L.raw[4 * i + 3] = v.w;
         }
       }
-      const size_t gs = sz_t + ((size_t)(S4 * C::NGC) << csh);
-      const uint32_t gv = __umul24(wrc, sz_mul) + ((chl * C::NGC) << csh);
-      const uint8_t* const zp = m_zero + gs;
-      const uint16_t* const sp = m_scale + gs;
+      const uint32_t gv = so_g + ((uint32_t)(S4 * C::NGC) << csh) + __umul24(wrc, sz_mul) + ((chl * C::NGC) << csh);
       if (C::NGC == 1) {
-        L.zraw = zp[gv];
-        L.sc[0] = sp[gv];
+        L.zraw = m_zero[gv];
+        L.sc[0] = m_scale[gv];
       } else {
-        const uint8_t* const zp1 = zp + ((size_t)1 << csh);
-        const uint16_t* const sp1 = sp + ((size_t)1 << csh);
-        L.zraw = (uint32_t)zp[gv] | ((uint32_t)zp1[gv] << 8);
-        L.sc[0] = sp[gv];
-        L.sc[C::NGC - 1] = sp1[gv];
+        const uint32_t gv1 = gv + (1u << csh);
+        L.zraw = (uint32_t)m_zero[gv] | ((uint32_t)m_zero[gv1] << 8);
+        L.sc[0] = m_scale[gv];
+        L.sc[C::NGC - 1] = m_scale[gv1];
       }
     };
 
@@ -668,6 +666,9 @@ bool gemv_fast_takes(const DMat& m, int M) {
   else if (fam == FAM_DENSE) { if (m.bits == 8) return false; }
   else return false;
   if (m.bits != 2 && m.bits != 3 && m.bits != 4) return false;
+  // 32-bit offsets inside the kernel: every array of the matrix below 4 GB
+  if ((uint64_t)((m.K + 15) / 16 * 16) * m.stride + 1024 >= (1ull << 32)) return false;
+  if ((uint64_t)((m.K + 15) / 16 * 16) * m.G * 2 >= (1ull << 32)) return false;
   return (size_t)M * NDIG * m.N <= (size_t)X_LDS_BUDGET;
 }
 
