@@ -628,10 +628,18 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
         if (lane == 0) old = atomicAdd(&cnt[slot], 1);
         old = __builtin_amdgcn_readfirstlane(old);                 // lane 0 holds it, and every lane is active here
         if (old == SK - 1) {                                      // uniform over the wave
-          for (int om = kq; om < h.M; om += 4) {
+          // quarter kq finishes activation row kq (M <= 4); the partial sums are read four at a
+          // time (parts past SK re-read the last one and do not count) and added in part order
+          if (kq < h.M) {
             float v = 0.f;
-            for (int j = 0; j < SK; ++j) v += rs[(j * h.M + om) * 16 + wr];
-            store(om, wr, v);
+            for (int j0 = 0; j0 < SK; j0 += 4) {
+              float pv[4];
+#pragma unroll
+              for (int j = 0; j < 4; ++j) pv[j] = rs[((j0 + j < SK ? j0 + j : SK - 1) * h.M + kq) * 16 + wr];
+#pragma unroll
+              for (int j = 0; j < 4; ++j) v += j0 + j < SK ? pv[j] : 0.f;
+            }
+            store(kq, wr, v);
           }
           if (lane == 0) cnt[slot] = 0;
         }
