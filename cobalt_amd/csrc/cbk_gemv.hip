@@ -477,7 +477,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 
     int bars = 0;                                                 // group barriers passed so far
     float ysum[MP];
-    auto do_step = [&](Loads<C>& cur, Loads<C>& tgt) {             // decode `cur`, load two steps ahead into `tgt`
+    auto do_step = [&](Loads<C>& cur, Loads<C>& tgt) {             // decode `cur`, load the next step into `tgt`
       const int tl = p0.tl, part = p0.part, S = p0.S;
       const int tile = t_lo + tl;
       const int s_end = (part * spi + spi < nS) ? part * spi + spi : nS;
