@@ -33,7 +33,10 @@ SIGNATURES = {
                                       ctypes.c_int, ctypes.c_int, ctypes.POINTER(_P), ctypes.POINTER(ctypes.c_int64),
                                       ctypes.c_int, ctypes.POINTER(_P), _P, ctypes.c_size_t, _P]),
     "cbk_linear": (ctypes.c_int, _MM),
+    "cbk_linear_act_workspace_bytes": (ctypes.c_size_t, [_DP, ctypes.c_int, ctypes.c_int]),
+    "cbk_linear_act": (ctypes.c_int, _MM[:9] + [ctypes.c_int] + _MM[9:]),
 }
+ACT_CODE = {"gelu_tanh": 0, "silu": 1}
 
 
 class CbkError(RuntimeError):

@@ -13,6 +13,8 @@ bool gemv_fast_takes(const DMat&, int M);
 bool gemv_same_config(const DMat&, const DMat&);
 size_t gemv_fast_workspace(const DMat&, int M);
 constexpr int kMaxBatch = 8;
+int launch_act_mul(const void* t, int tdt, int64_t ldt, void* y, int ydt, int64_t ldy, int M, int K2, int act,
+                   const void* bias, hipStream_t st);
 int launch_gemm(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*,
                 hipStream_t);
 int launch_gemm_big(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*, void*, size_t,
@@ -343,6 +345,40 @@ int cbk_linear(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ld
     return CBK_OK;
   }
   return cbk_gemm(in, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, workspace, workspace_bytes, stream);
+}
+
+// Where cbk_linear_act keeps t = x . W_hat^T: float32 up to 128 activation rows, else the output type.
+static int act_mid_dtype(int M, int y_dtype) { return M <= 128 ? CBK_F32 : y_dtype; }
+static size_t act_mid_bytes(int K, int M, int y_dtype) {
+  const size_t b = (size_t)M * K * (act_mid_dtype(M, y_dtype) == CBK_F32 ? 4 : 2);
+  return (b + 255) & ~(size_t)255;
+}
+
+size_t cbk_linear_act_workspace_bytes(const cbk_desc* in, int M, int y_dtype) {
+  cbk_desc d;
+  if (M < 1 || canon(in, &d)) return 0;
+  return act_mid_bytes(d.K, M, y_dtype) + cbk_workspace_bytes(in, M);
+}
+
+int cbk_linear_act(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ldx, void* y, int y_dtype,
+                   int64_t ldy, const void* bias, int act, void* workspace, size_t workspace_bytes, void* stream) {
+  DMat m;
+  int rc = to_dmat(in, &m, true);
+  if (rc) return rc;
+  if (m.K & 1) return CBK_ERR_SHAPE;
+  if (act != CBK_ACT_GELU_TANH && act != CBK_ACT_SILU) return CBK_ERR_UNSUPPORTED;
+  if (y_dtype != CBK_F32 && y_dtype != CBK_F16 && y_dtype != CBK_BF16T) return CBK_ERR_DTYPE;
+  if (!y) return CBK_ERR_NULL;
+  if (M < 1 || ldy < m.K / 2) return CBK_ERR_SHAPE;
+  if ((uintptr_t)y & (y_dtype == CBK_F32 ? 3 : 1)) return CBK_ERR_ALIGN;
+  const size_t mid = act_mid_bytes(m.K, M, y_dtype);
+  if (!workspace || ((uintptr_t)workspace & 255) || workspace_bytes < mid + cbk_workspace_bytes(in, M))
+    return CBK_ERR_WORKSPACE;
+  const int tdt = act_mid_dtype(M, y_dtype);
+  rc = cbk_linear(in, x, x_dtype, M, ldx, workspace, tdt, m.K, nullptr, (uint8_t*)workspace + mid,
+                  workspace_bytes - mid, stream);                  // the activation kernel adds the bias
+  if (rc) return rc;
+  return launch_act_mul(workspace, tdt, m.K, y, y_dtype, ldy, M, m.K / 2, act, bias, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -143,6 +143,10 @@ class CobaltLinear(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return ops.linear(self._pm(), x, self.bias)
 
+    def forward_act(self, x: torch.Tensor, act: str) -> torch.Tensor:
+        """For a gate/up matrix (rows 2i gate, 2i+1 up): act(gate(x)) * up(x), [.., out_features / 2]."""
+        return ops.linear_act(self._pm(), x, act, self.bias)
+
     def dequantize(self, dtype=torch.float32) -> torch.Tensor:
         return ops.dequant(self._pm(), dtype)
 

@@ -227,9 +227,70 @@ def _fuse_group(blk: nn.Module, names: Sequence[str], interleave: bool, device_o
     return True
 
 
-def fuse_model(model: nn.Module, device_order: bool = True) -> int:
+def _gate_act_of(mlp: nn.Module) -> Optional[str]:
+    """'gelu_tanh' or 'silu' if `mlp.act_fn` is that function (checked on values), else None."""
+    fn = getattr(mlp, "act_fn", None)
+    if not callable(fn):
+        return None
+    t = torch.linspace(-6.0, 6.0, 49)
+    try:
+        with torch.no_grad():
+            v = fn(t)
+    except Exception:
+        return None
+    if not isinstance(v, torch.Tensor) or v.shape != t.shape:
+        return None
+    if torch.allclose(v, torch.nn.functional.gelu(t, approximate="tanh"), atol=1e-6):
+        return "gelu_tanh"
+    if torch.allclose(v, torch.nn.functional.silu(t), atol=1e-6):
+        return "silu"
+    return None
+
+
+def _gated_forward(self, x):
+    """down(act(gate(x)) * up(x)) with the first half in one call on the fused gate/up matrix
+    (EPI_GEGLU_BF16 / EPI_SWIGLU_BF16, src/cobaltkernel/csrc/cobalt_gemm.cuh:30-33)."""
+    fused = self.gate_proj._owner.fused
+    if isinstance(fused, CobaltLinear):
+        h = fused.forward_act(x, self._cbk_act)
+    else:                                                             # a dense twin of the fused matrix
+        t = fused(x)
+        g = t[..., 0::2]
+        g = torch.nn.functional.gelu(g, approximate="tanh") if self._cbk_act == "gelu_tanh" else torch.nn.functional.silu(g)
+        h = g * t[..., 1::2]
+    return self.down_proj(h)
+
+
+def _install_gated_forward(mlp: nn.Module) -> bool:
+    """Give a gated MLP whose gate/up are fused (and whose forward is
+    down_proj(act_fn(gate_proj(x)) * up_proj(x)), as the Hugging Face decoders' is) the one-call
+    forward.  The module's own forward is run beside it once; it stays if the two disagree."""
+    act = _gate_act_of(mlp)
+    gp = getattr(mlp, "gate_proj", None)
+    if act is None or not isinstance(gp, FusedPart) or not isinstance(gp._owner.fused, CobaltLinear):
+        return False
+    fused = gp._owner.fused
+    if not fused.blob.is_cuda:
+        return False
+    import types
+    x = torch.randn(3, fused.in_features, device=fused.blob.device, dtype=torch.float16, generator=None) * 0.5
+    with torch.no_grad():
+        a = mlp(x).float()
+        mlp._cbk_act = act
+        mlp.forward = types.MethodType(_gated_forward, mlp)
+        b = mlp(x).float()
+    if not bool(torch.isfinite(b).all()) or float((a - b).norm()) > 2e-2 * float(a.norm()) + 1e-6:
+        del mlp.forward
+        del mlp._cbk_act
+        return False
+    return True
+
+
+def fuse_model(model: nn.Module, device_order: bool = True, gated_mlp: bool = True) -> int:
     """Fuse q|k|v and gate/up of every decoder block whose linears are row-major or device-order
-    `CobaltLinear` modules with matching configurations.  Returns the number of fused groups."""
+    `CobaltLinear` modules with matching configurations.  With `gated_mlp`, an MLP of the form
+    down(act(gate(x)) * up(x)) with a tanh-GELU or SiLU gate then computes act(gate) * up in the
+    same call as the fused matrix.  Returns the number of fused groups."""
     n = 0
     for _bname, blk in decoder_blocks(model):
         for names, il in ((HGROUPS["attn_in"], False), (HGROUPS["mlp_in"], True)):
@@ -242,7 +303,10 @@ def fuse_model(model: nn.Module, device_order: bool = True) -> int:
                         m._buffers["blob"] = t.blob
                         m._buffers["cbk_meta"] = m._meta_of(t)
                         m._pm_cache = None
-                n += 1 if _fuse_group(blk, names, il, device_order) else 0
+                ok = _fuse_group(blk, names, il, device_order)
+                n += 1 if ok else 0
+                if ok and il and gated_mlp:
+                    _install_gated_forward(_sub(blk, names[0].rsplit(".", 1)[0]))
     return n
 
 

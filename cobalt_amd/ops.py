@@ -94,6 +94,44 @@ def linear(pm, x, bias=None, out_dtype=None, workspace=None):
     return _matmul("cbk_linear", pm, x, bias, out_dtype, workspace)
 
 
+def linear_act(pm, x, act: str, bias=None, out_dtype=None):
+    """First half of a gated MLP on a gate/up matrix (rows 2i gate, 2i+1 up):
+    y[..., i] = act(t[..., 2i]) * t[..., 2i+1] with t = x @ W_hat.T (+ bias), act 'gelu_tanh' or
+    'silu' (EPI_GEGLU_BF16 / EPI_SWIGLU_BF16, src/cobaltkernel/csrc/cobalt_gemm.cuh:30-33)."""
+    if act not in _lib.ACT_CODE:
+        raise ValueError(f"act must be one of {sorted(_lib.ACT_CODE)}, got {act!r}")
+    _require_gpu(pm, x, bias)
+    if x.shape[-1] != pm.N:
+        raise ValueError(f"x has {x.shape[-1]} input features, the matrix has N={pm.N}")
+    if pm.K % 2:
+        raise ValueError("a gate/up matrix has an even number of rows")
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, pm.N)
+    if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) % 8) or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    M = x2.shape[0]
+    out_dtype = out_dtype or x.dtype
+    y = torch.empty(M, pm.K // 2, dtype=out_dtype, device=x.device)
+    if M == 0:
+        return y.reshape(*lead, pm.K // 2)
+    if bias is not None and bias.dtype != out_dtype:
+        bias = bias.to(out_dtype)
+    L = _lib.lib()
+    d = pm.desc()
+    need = L.cbk_linear_act_workspace_bytes(ctypes.byref(d), M, dtype_code(out_dtype))
+    key = (pm.blob.device, torch.cuda.current_stream(pm.blob.device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.empty(max(need, 1 << 20), dtype=torch.uint8, device=pm.blob.device)
+        _workspaces[key] = ws
+    ldx = x2.stride(0) if M > 1 else pm.N
+    rc = L.cbk_linear_act(ctypes.byref(d), x2.data_ptr(), dtype_code(x2.dtype), M, ldx, y.data_ptr(),
+                          dtype_code(out_dtype), pm.K // 2, bias.data_ptr() if bias is not None else None,
+                          _lib.ACT_CODE[act], ws.data_ptr(), ws.numel(), _stream_ptr(x.device))
+    _lib.check(rc, "cbk_linear_act")
+    return y.reshape(*lead, pm.K // 2)
+
+
 def gemv_batch(pms, xs, biases=None, out_dtype=None):
     """Independent decode GEMVs in one launch pair: ys[i] = xs[i] @ W_hat_i.T (+ biases[i]).
     All xs share the number of rows (<= 16) and the dtype; at most 8 matrices."""

@@ -48,6 +48,9 @@ enum cbk_layout {
 
 enum cbk_dtype { CBK_F32 = 0, CBK_F16 = 1, CBK_BF16T = 2 };
 
+/* gate activations of cbk_linear_act (cobalt_gemm.cuh:216-220: tanh-GELU, x / (1 + exp(-x))) */
+enum cbk_act { CBK_ACT_GELU_TANH = 0, CBK_ACT_SILU = 1 };
+
 enum cbk_status {
   CBK_OK = 0,
   CBK_ERR_NULL = -1,        /* a required pointer is NULL                                 */
@@ -165,6 +168,19 @@ int cbk_gemm(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
 int cbk_linear(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
                void* y, int y_dtype, int64_t ldy, const void* bias,
                void* workspace, size_t workspace_bytes, void* stream);
+
+/* The first half of a gated MLP in one call, for a matrix whose rows 2i / 2i+1 are the gate and
+ * up rows of output i (K even; normally cs_rows == 2):
+ *   y[m, i] = act(t[m, 2i]) * t[m, 2i+1],   t = x . W_hat^T (+ bias, K entries of type y_dtype),
+ * y [M, K/2] with ldy >= K/2.  Up to 128 activation rows t is kept in float32 and the result is
+ * rounded once, as EPI_GEGLU_BF16 / EPI_SWIGLU_BF16 of cbk::gemm_tile do
+ * (cobalt_gemm.cuh:30-33, :586-592; checked by test_gemm.py:196-210); above that t is stored in
+ * y_dtype between the matrix kernel and the activation kernel (one more rounding of gate and
+ * up).  The workspace holds t and the scratch of cbk_linear: cbk_linear_act_workspace_bytes(). */
+size_t cbk_linear_act_workspace_bytes(const cbk_desc* d, int M, int y_dtype);
+int cbk_linear_act(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
+                   void* y, int y_dtype, int64_t ldy, const void* bias, int act,
+                   void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -73,6 +73,16 @@ def test_fused_qkv_and_gate_up_match_the_separate_modules():
     packed = [x for x in f.modules() if isinstance(x, CobaltLinear)]
     assert len(packed) == 2 * 4                                       # per block: qkv, o, gate/up, down
     assert sorted(x._pm().cs_rows for x in packed) == [1, 1, 1, 1, 2, 2, 3, 3]
+    # the MLPs compute silu(gate) * up in the call of the fused matrix; without that they slice
+    mlps = [blk.mlp for _n, blk in Mo.decoder_blocks(f)]
+    assert all(getattr(x, "_cbk_act", None) == "silu" for x in mlps)
+    f2 = copy.deepcopy(m)
+    Mo.fuse_model(f2, gated_mlp=False)
+    assert not any(hasattr(blk.mlp, "_cbk_act") for _n, blk in Mo.decoder_blocks(f2))
+    h = torch.randn(2, 7, 256, generator=g).to(DEV, torch.float16)
+    with torch.no_grad():
+        ya, yb = mlps[0](h).float(), f2.model.layers[0].mlp(h).float()
+    assert float((ya - yb).norm() / yb.norm()) < 2e-3
     twin = Mo.dense_twin(copy.deepcopy(f), torch.float16)
     for shape in ((1, 300), (2, 12), (1, 1), (2, 1)):
         ids = torch.randint(0, 512, shape, generator=g).to(DEV)

@@ -2,13 +2,15 @@
 seeded inputs.  Bars: dequantised weights bit-exact (value equality; -0.0 == 0.0, as the
 reference's own check does, src/prod/verify.py:139); layer outputs within relative Frobenius
 error 1e-3 of x @ W_hat.T with W_hat in float32 and a float64 accumulator."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
 
 from oracle import cbk_ref as R
 from cobalt_amd import format as F
-from cobalt_amd import ops
+from cobalt_amd import _lib, ops
 from cobalt_amd.linear import CobaltLinear
 from helpers import (FIXED_CASES, SPARSE_CASES, acts, case_id, kw_of, make_raw, oracle_pack, packed_from_oracle,
                      product_pack, rel_fro)
@@ -314,6 +316,68 @@ def test_gemm_fused_col_scale_rows(case):
             y = ops.gemm(pm, x.to(DEV), bias=bias.to(DEV), out_dtype=torch.float32)
             err = rel_fro(_np(y), ref)
             assert err < TOL, f"{case_id(case)} cs_rows={cs_rows} splits={splits} M={M}: {err}"
+
+
+def _gated_ref(t, act):
+    """act(gate) * up in float64 from t[.., 2i] / t[.., 2i+1]: the tanh-GELU and SiLU formulas of
+    cobalt_gemm.cuh:216-220; the reference checks its epilogue against
+    torch.nn.functional.gelu(gate, approximate="tanh") * up (test_gemm.py:204-209)."""
+    g, u = t[:, 0::2].astype(np.float64), t[:, 1::2].astype(np.float64)
+    if act == "gelu_tanh":
+        a = 0.5 * g * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (g + 0.044715 * g ** 3)))
+    else:
+        a = g / (1.0 + np.exp(-g))
+    return a * u
+
+
+@pytest.mark.parametrize("act", ["gelu_tanh", "silu"])
+@pytest.mark.parametrize("case", FUSED_CASES[:2], ids=case_id)
+def test_linear_act_gated_epilogue(case, act):
+    """Gate/up matrix through cbk_linear_act at decode, mid and prefill row counts.  float32 and
+    f16 outputs meet the layer tolerance; a bf16 output carries its own 2^-9 rounding (and, above
+    128 rows, that of the stored gate and up values), so it is held to 4e-3."""
+    K, N = 640, 1024
+    pm, W = _fused(case, K, N, 2, (0, 0), seed=K + 5, tiled=True)
+    bias = acts(1, K, torch.float16, seed=11)[0]
+    for M, dtype, odt, with_bias in ((1, torch.float16, torch.float32, False), (4, torch.bfloat16, torch.bfloat16, False),
+                                     (64, torch.float16, torch.float16, True), (129, torch.float16, torch.float32, True),
+                                     (300, torch.bfloat16, torch.bfloat16, False), (300, torch.float16, torch.float16, False)):
+        x = acts(M, N, dtype, seed=M + 1)
+        b = bias.to(odt) if with_bias else None
+        t = R.forward_ref(W, _np(x))
+        if with_bias:
+            t = t + _np(b)[None, :]
+        ref = _gated_ref(t, act)
+        y = ops.linear_act(pm, x.to(DEV), act, bias=None if b is None else b.to(DEV), out_dtype=odt)
+        assert y.shape == (M, K // 2) and y.dtype == odt
+        err = rel_fro(_np(y), ref)
+        tol = 4e-3 if odt == torch.bfloat16 else TOL
+        assert err < tol, f"{case_id(case)} {act} M={M} {dtype}->{odt}: {err}"
+    # the first half of an MLP equals the two-step form on the same kernels
+    x = acts(8, N, torch.float16, seed=3).to(DEV)
+    t = ops.linear(pm, x, out_dtype=torch.float32)
+    two = (torch.nn.functional.gelu(t[:, 0::2], approximate="tanh") if act == "gelu_tanh"
+           else torch.nn.functional.silu(t[:, 0::2])) * t[:, 1::2]
+    one = ops.linear_act(pm, x, act, out_dtype=torch.float32)
+    assert rel_fro(_np(one), _np(two)) < 1e-6
+
+
+def test_linear_act_rejects_bad_calls():
+    case = FUSED_CASES[0]
+    pm, _ = _fused(case, 64, 256, 2, (0, 0), seed=1, tiled=False)
+    x = acts(2, 256, torch.float16, seed=1).to(DEV)
+    with pytest.raises(ValueError):
+        ops.linear_act(pm, x, "relu")
+    L, d = _lib.lib(), pm.desc()
+    y = torch.empty(2, 32, dtype=torch.float16, device=DEV)
+    ws = torch.empty(1 << 20, dtype=torch.uint8, device=DEV)
+    args = lambda act, wsb, ldy: (ctypes.byref(d), x.data_ptr(), 1, 2, 256, y.data_ptr(), 1, ldy, None, act,
+                                  ws.data_ptr(), wsb, None)
+    assert L.cbk_linear_act(*args(7, ws.numel(), 32)) == -8           # unknown activation
+    assert L.cbk_linear_act(*args(0, 16, 32)) == -6                   # workspace too small
+    assert L.cbk_linear_act(*args(0, ws.numel(), 16)) == -3           # ldy below K / 2
+    assert L.cbk_linear_act(*args(0, ws.numel(), 32)) == 0
+    torch.cuda.synchronize()
 
 
 # ------------------------------------------------------------------ prefill GEMM
