@@ -398,6 +398,34 @@ def test_gemm_matches_oracle(case, dtype, tiled):
         assert err < TOL, f"{case_id(case)} M={M}: {err}"
 
 
+@pytest.mark.parametrize("cs_rows", [1, 2, 3])
+def test_gemm_more_tiles_than_one_round_over_the_cus(cs_rows):
+    """260 tiles of 256 x 256 (more than the 256 CUs take at once), ragged K and M, plain and
+    row-fused: checked against the bit-exact dequantised weights (float64 matmul on the device)
+    and for run-to-run identical results."""
+    K, N, M = 256 * 130 - 24, 2048, 500                             # 2 x 130 = 260 tiles
+    mk = lambda k, seed: F.synth_packed(k, N, F.BLK1632_4, 4, 128, 16, seed=seed, device=DEV)
+    if cs_rows == 1:
+        pm = mk(K, 1)
+    elif cs_rows == 2:
+        pm = F.fuse_rows([mk(K // 2, 2), mk(K // 2, 3)], interleave=True)
+    else:
+        pm = F.fuse_rows([mk(256 * 40, 4), mk(256 * 30, 5), mk(K - 256 * 70, 6)])
+    assert pm.cs_rows == cs_rows and pm.K == K
+    pm = pm.to_tiled()
+    W = ops.dequant(pm, torch.float32).double()
+    x = acts(M, N, torch.float16, seed=5).to(DEV)
+    bias = torch.randn(K, generator=torch.Generator().manual_seed(1)).to(DEV)
+    ref = x.double() @ W.T + bias.double()
+    y = ops.gemm(pm, x, bias=bias, out_dtype=torch.float32)
+    err = float((y.double() - ref).norm() / ref.norm())
+    assert err < TOL, err
+    assert torch.equal(ops.gemm(pm, x, bias=bias, out_dtype=torch.float32), y)
+    yb = ops.gemm(pm, x.to(torch.bfloat16), out_dtype=torch.bfloat16)
+    refb = x.to(torch.bfloat16).double() @ W.T
+    assert float((yb.double() - refb).norm() / refb.norm()) < 4e-3
+
+
 @pytest.mark.parametrize("case", [(F.BLK1632_4, 4, 128, 16), (F.DENSE4, 4, 128, 0), (F.BLKC, 3, 64, 23)], ids=case_id)
 def test_gemm_odd_chunk_count_and_ragged_tiles(case):
     """N = 3 chunks of 128 (the kernel works on chunk pairs and pads), K and M not multiples of
