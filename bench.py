@@ -100,6 +100,48 @@ def cpu_baseline(pms, shapes, xs, ys, M, budget_s=20.0):
                 gpu_vs_oracle_rel_fro=worst)
 
 
+def measured_ceilings(torch, dev):
+    """What this GPU reaches on back-to-back dense f16 MFMAs and on a plain streaming read of
+    1 GiB (libcbk_bench.so, built by `python -m cobalt_amd.build`): ceilings to read the kernels'
+    figures against, beside the published peaks.  None if the helper library is not built."""
+    import ctypes
+    path = os.path.join(ROOT, "cobalt_amd", "libcbk_bench.so")
+    if not os.path.exists(path):
+        return None
+    L = ctypes.CDLL(path)
+    L.cbk_bench_mfma_f16.restype = ctypes.c_int
+    L.cbk_bench_mfma_f16.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    L.cbk_bench_read.restype = ctypes.c_int
+    L.cbk_bench_read.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    st = torch.cuda.current_stream(dev)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def timed(fn, reps):
+        for _ in range(3):
+            fn()
+        e0.record(st)
+        for _ in range(reps):
+            fn()
+        e1.record(st)
+        st.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    blocks, iters = 2 * cus, 4000
+    sink = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
+    ms = timed(lambda: L.cbk_bench_mfma_f16(blocks, iters, sink.data_ptr(), st.cuda_stream), 5)
+    mfma = blocks * 4 * iters * 16 * 2.0 * 32 * 32 * 16 / ms / 1e9
+    buf = torch.empty(2**30, dtype=torch.uint8, device=dev)
+    buf.random_(0, 256)
+    sink4 = torch.zeros(1, dtype=torch.int32, device=dev)
+    ms = timed(lambda: L.cbk_bench_read(buf.data_ptr(), buf.numel(), 16 * cus, sink4.data_ptr(), st.cuda_stream), 10)
+    read = buf.numel() / ms / 1e6
+    del buf, sink, sink4
+    return {"mfma_f16_dense_tflops": round(mfma, 1), "hbm_read_gbs": round(read, 1),
+            "how": "libcbk_bench.so: 16 independent v_mfma_f32_32x32x16_f16 per wavefront, one wavefront per SIMD; "
+                   "grid-stride 16-byte reads of 1 GiB"}
+
+
 def prefill_gemm(torch, F, ops, dev, workload, layout, bits, group, keep, M, dt, reps=20, warm=10):
     """Prefill kernel on the MLP matrices (gate, up, down) of a layer set."""
     shapes = {n: (K, N) for n, K, N in SHAPES[workload]}
@@ -313,6 +355,13 @@ def main():
     if not a.no_prefill:
         out["prefill_gemm"] = prefill_gemm(torch, F, ops, dev, a.prefill_workload, layout, a.bits, a.group, a.keep,
                                            a.prefill_m, torch.float16 if a.prefill_dtype == "f16" else torch.bfloat16)
+    ceil = measured_ceilings(torch, dev)
+    if ceil:
+        out["measured_ceilings"] = ceil
+        out["roofline"]["frac_of_measured_read"] = round(achieved / ceil["hbm_read_gbs"], 4)
+        if "prefill_gemm" in out:
+            out["prefill_gemm"]["roofline"]["frac_of_measured_mfma"] = round(
+                out["prefill_gemm"]["tflops"] / ceil["mfma_f16_dense_tflops"], 4)
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline(first_rowmajor, shapes, xs, y_first, M)
         # outputs are rounded to the activation dtype (2^-11 relative) on top of the kernel's own error

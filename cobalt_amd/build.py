@@ -38,6 +38,22 @@ def build_lib(verbose=True, extra=()):
     return LIB
 
 
+BENCH_LIB = os.path.join(HERE, "libcbk_bench.so")
+
+
+def build_bench_lib(verbose=True):
+    """libcbk_bench.so: the measured-ceiling probes bench.py reports beside the published peaks."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc] + FLAGS + [os.path.join(CSRC, "cbk_bench.hip"), "-o", BENCH_LIB]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if out.returncode != 0:
+        raise RuntimeError("hipcc failed on cbk_bench.hip:\n" + out.stdout)
+    return BENCH_LIB
+
+
 if __name__ == "__main__":
     build_lib()
-    print("built", LIB)
+    build_bench_lib()
+    print("built", LIB, BENCH_LIB)

@@ -72,6 +72,16 @@ def test_library_exports_every_declared_symbol():
     assert _lib.lib().cbk_abi_version() == 1
 
 
+def test_bench_helper_library_loads():
+    """libcbk_bench.so (the measured-ceiling probes of bench.py) is built beside the C-ABI library
+    and exports its two entry points; nothing is launched here."""
+    path = os.path.join(ROOT, "cobalt_amd", "libcbk_bench.so")
+    if not os.path.exists(path):
+        pytest.skip("libcbk_bench.so is not built (python -m cobalt_amd.build)")
+    L = ctypes.CDLL(path)
+    assert hasattr(L, "cbk_bench_mfma_f16") and hasattr(L, "cbk_bench_read")
+
+
 def test_descriptor_validation_and_strides():
     L = _lib.lib()
     for case in FIXED_CASES:
