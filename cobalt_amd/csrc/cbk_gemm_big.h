@@ -1,4 +1,4 @@
-// Prefill GEMM for M > 128:  Y[M, K] = X[M, N] . W_hat[K, N]^T on the gfx950 matrix cores.
+// Prefill GEMM:  Y[M, K] = X[M, N] . W_hat[K, N]^T on the gfx950 matrix cores.
 //
 // Workgroup tile 256 tokens x 256 weight rows, 64 input columns per stage, four wavefronts
 // each owning a 128 x 128 sub-tile (4 x 4 blocks of v_mfma_f32_32x32x16_f16, 256 accumulator
@@ -33,13 +33,14 @@
 
 namespace cbk {
 
-constexpr int GB_T = 256;       // tokens per workgroup tile
+constexpr int GB_T = 256;       // tokens per workgroup tile (TI = 4); the TI = 1 kernels take 64
 constexpr int GB_R = 256;       // weight rows per workgroup tile
 constexpr int GB_K = 64;        // input columns per stage
 constexpr int GB_P = GB_K + 8;  // LDS row pitch of the weight tile in halfs (144 B): conflict-free 16-byte reads
 constexpr int GB_LUT = 256 * 8 * 8;   // selector table, 8 lane-private copies of 256 x 8 B
-constexpr int GB_XBUF = GB_T * GB_K * 2;   // one activation stage in LDS: 256 rows x 128 B, unpadded, swizzled
-constexpr size_t GB_LDS = (size_t)2 * GB_XBUF + (size_t)2 * GB_R * GB_P * 2 + GB_LUT;
+// one activation stage in LDS: 64 TI rows x 128 B, unpadded, swizzled
+constexpr int gb_xbuf(int ti) { return 64 * ti * GB_K * 2; }
+constexpr size_t gb_lds(int ti) { return (size_t)2 * gb_xbuf(ti) + (size_t)2 * GB_R * GB_P * 2 + GB_LUT; }
 
 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
 
@@ -52,6 +53,7 @@ struct GbArgs {
   int64_t ldy;
   const void* bias;
   int tiles_t, tiles_r;
+  int ti;                  // 32-token blocks per wavefront: 4 (256-token tiles) or 1 (64-token tiles)
   // par = 1: gate/up matrix, two col_scale vectors by row parity.  A workgroup then takes 256
   // rows of one parity out of 512 (rows r0 + 2 i + p), and X' of that parity's vector, which
   // starts xps elements after the other one.
@@ -103,8 +105,8 @@ __device__ inline uint4 bytes_to_halfs(uint32_t b0, uint32_t b1, h2_t s2) {
 // turning the tile around in LDS makes the global stores whole 16-byte pieces of consecutive
 // output columns: 256 B (f16) or 512 B (f32) per token.  Compile-time indexed and branch-free
 // per element: the 256 accumulators make this straight-line code, and it has to stay small.
-template <int YDT, int kstep>                                    // local row i is output column row0 + kstep * i
-__device__ inline void gb_epilogue(const GbArgs& a, v16f (&acc)[4][4], uint8_t* smem, int lane, int wave, int tok0,
+template <int YDT, int kstep, int TI>                            // local row i is output column row0 + kstep * i
+__device__ inline void gb_epilogue(const GbArgs& a, v16f (&acc)[TI][4], uint8_t* smem, int lane, int wave, int tok0,
                                    int row0) {
   constexpr int ESZ = YDT == CBK_F32 ? 4 : 2;
   constexpr int PITCH = 128 * ESZ + 16;                          // bytes per token row in LDS
@@ -121,7 +123,7 @@ __device__ inline void gb_epilogue(const GbArgs& a, v16f (&acc)[4][4], uint8_t* 
   }
   const bool vec_ok = ((a.ldy * ESZ) & 15) == 0 && (((uintptr_t)a.y) & 15) == 0;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < TI; ++i) {
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -156,8 +158,12 @@ __device__ inline void gb_epilogue(const GbArgs& a, v16f (&acc)[4][4], uint8_t* 
 // 3: one col_scale vector, column range split over several workgroups (GbArgs::nsplit).
 // Three instantiations rather than run-time switches: the schedule of the main loop is tuned
 // to the instruction and measurably shifts with every value that is added to it.
-template <int BITS, int KEEP, int GRP, int PAR>
+// TI: 32-token blocks per wavefront.  4: the 256-token tile described above.  1: a 64-token tile
+// (each wavefront 32 tokens x 128 rows) for calls of at most 64 activation rows, whose time is
+// the weight decode: a quarter of the matrix instructions per stage, the same decode.
+template <int BITS, int KEEP, int GRP, int PAR, int TI = 4>
 __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
+  constexpr int GB_XBUF = gb_xbuf(TI);
   constexpr bool FASTD = BITS != 0;
   using C = CodeCfg<FASTD ? BITS : 4, KEEP, FASTD ? GRP : 128>;
   constexpr bool BITMAP = FASTD && !C::DENSE;
@@ -181,7 +187,7 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   const int tt = tile / a.tiles_r, tr = tile % a.tiles_r;
   constexpr int kstep = PAR == 1 ? 2 : 1;                         // row stride of this workgroup's rows
   const int pp = PAR == 1 ? (tr & 1) : 0;                         // and their parity
-  const int t0 = tt * GB_T, r0 = PAR == 1 ? (tr >> 1) * (2 * GB_R) + pp : tr * GB_R;
+  const int t0 = tt * (64 * TI), r0 = PAR == 1 ? (tr >> 1) * (2 * GB_R) + pp : tr * GB_R;
   const int N = m.N, Npad = a.Npad;
   // stages of this workgroup: all of them, or its part of them; a multiple of 4 either way;
   // stages past N see X' = 0
@@ -197,9 +203,9 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   }
   const uint32_t l8 = lane & 7;
 
-  v16f acc[4][4];
+  v16f acc[TI][4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TI; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -211,21 +217,21 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   const int wrc = wok ? wrow : m.K - 1;
   const RowView rv = row_view(m, wrc);
   const size_t meta0 = meta_index(m, wrc, 0), meta_step = m.tiled ? 16 : 1;
-  // Activation tile: wavefront w copies rows 64w .. 64w+63 of every stage with eight direct
-  // copies of eight rows each; lane l of copy q takes row 64w + 8q + l/8 and fills physical
-  // piece l%8 of it, i.e. fetches logical piece (l%8) ^ ((4q + l/16) & 7).  That is one of two
-  // values per lane (q even / odd), so two lane offsets and a scalar base per copy suffice.
+  // Activation tile: wavefront w copies rows 16 TI w .. 16 TI (w+1) - 1 of every stage with 2 TI
+  // direct copies of eight rows each; lane l of copy q takes row 16 TI w + 8q + l/8 and fills
+  // physical piece l%8 of it, i.e. fetches logical piece (l%8) ^ ((4q + l/16) & 7).  That is one
+  // of two values per lane (q even / odd), so two lane offsets and a scalar base per copy suffice.
   const int wv = __builtin_amdgcn_readfirstlane(wave);
   const uint32_t xvo_e = (uint32_t)((lane >> 3) * Npad * 2 + (((lane & 7) ^ (lane >> 4)) * 16));
   const uint32_t xvo_o = (uint32_t)((lane >> 3) * Npad * 2 + (((lane & 7) ^ (4 + (lane >> 4))) * 16));
   const int xv = PAR == 1 ? pp : PAR == 2 ? (r0 >= a.vs0 ? 1 : 0) + (r0 >= a.vs1 ? 1 : 0) : 0;   // which col_scale vector
-  const uint8_t* xsb = (const uint8_t*)(a.xp + (size_t)xv * a.xps + (size_t)(t0 + 64 * wv) * Npad + (size_t)s_begin * GB_K);
-  const uint32_t xlds0 = (uint32_t)(uintptr_t)Xs + (uint32_t)wv * 8192u;
+  const uint8_t* xsb = (const uint8_t*)(a.xp + (size_t)xv * a.xps + (size_t)(t0 + 16 * TI * wv) * Npad + (size_t)s_begin * GB_K);
+  const uint32_t xlds0 = (uint32_t)(uintptr_t)Xs + (uint32_t)wv * (2048u * TI);
   auto dma_x = [&](int s, int buf) {                              // stage s -> Xs[buf]
     const uint8_t* sb = xsb + (size_t)s * (GB_K * 2);
     const uint32_t ld = xlds0 + (uint32_t)buf * GB_XBUF;
 #pragma unroll
-    for (int q = 0; q < 8; ++q)
+    for (int q = 0; q < 2 * TI; ++q)
       dma_x16(sb + (size_t)q * 8 * Npad * 2, (q & 1) ? xvo_o : xvo_e, ld + q * 1024);
   };
   // fragment reads: this lane's row inside a 32-row block and its four swizzled piece offsets
@@ -349,12 +355,12 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   };
 
   // fragment registers, two sets; set 0 of the next stage is loaded at the end of the current one
-  v8h af[2][4], bf[2][4];
+  v8h af[2][TI], bf[2][4];
   auto read_frags = [&](int buf, int kk, int set) {
-    const uint8_t* xb = (const uint8_t*)Xs + (size_t)buf * GB_XBUF + (128 * wt + (lane & 31)) * 128;
+    const uint8_t* xb = (const uint8_t*)Xs + (size_t)buf * GB_XBUF + (32 * TI * wt + (lane & 31)) * 128;
     const _Float16* wb = Ws + (size_t)buf * GB_R * GB_P + (128 * wr + (lane & 31)) * GB_P + 8 * (lane >> 5);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) af[set][i] = *(const v8h*)(xb + 4096 * i + xpc[kk]);
+    for (int i = 0; i < TI; ++i) af[set][i] = *(const v8h*)(xb + 4096 * i + xpc[kk]);
 #pragma unroll
     for (int j = 0; j < 4; ++j) bf[set][j] = *(const v8h*)(wb + 32 * j * GB_P + 16 * kk);
   };
@@ -424,16 +430,16 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
         if (LOADW) load_chunk(cl, wl);
       }
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < TI; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[c][i], bf[c][j], acc[i][j], 0, 0, 0);
       if (kk < 3) {
 #pragma unroll
-        for (int g = 0; g < 16; ++g) {                            // one MFMA, then a slice of the decode
+        for (int g = 0; g < 4 * TI; ++g) {                        // one MFMA, then a slice of the decode
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          if (kk == 2) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-          else __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+          if (kk == 2) __builtin_amdgcn_sched_group_barrier(0x002, 16 / TI, 0);
+          else __builtin_amdgcn_sched_group_barrier(0x002, 20 / TI, 0);
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -455,39 +461,44 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
-  const int tok0 = t0 + 128 * wt, row0 = r0 + kstep * 128 * wr;
+  const int tok0 = t0 + 32 * TI * wt, row0 = r0 + kstep * 128 * wr;
   if (SPLIT) {                                                    // float32 partial tile, no bias
     GbArgs b = a;
     b.y = a.part + (size_t)part * a.part_stride;
     b.ldy = a.part_ld;
     b.bias = nullptr;
-    gb_epilogue<CBK_F32, 1>(b, acc, smem, lane, wave, tok0, row0);
+    gb_epilogue<CBK_F32, 1, TI>(b, acc, smem, lane, wave, tok0, row0);
     return;
   }
-  if (a.ydt == CBK_F32) gb_epilogue<CBK_F32, kstep>(a, acc, smem, lane, wave, tok0, row0);
-  else if (a.ydt == CBK_F16) gb_epilogue<CBK_F16, kstep>(a, acc, smem, lane, wave, tok0, row0);
-  else gb_epilogue<CBK_BF16T, kstep>(a, acc, smem, lane, wave, tok0, row0);
+  if (a.ydt == CBK_F32) gb_epilogue<CBK_F32, kstep, TI>(a, acc, smem, lane, wave, tok0, row0);
+  else if (a.ydt == CBK_F16) gb_epilogue<CBK_F16, kstep, TI>(a, acc, smem, lane, wave, tok0, row0);
+  else gb_epilogue<CBK_BF16T, kstep, TI>(a, acc, smem, lane, wave, tok0, row0);
 }
 
-template <int BITS, int KEEP, int GRP, int PAR>
+template <int BITS, int KEEP, int GRP, int PAR, int TI>
 static int launch_big_par(const GbArgs& a, int blocks, hipStream_t st) {
-  auto kern = gemm_big_kernel<BITS, KEEP, GRP, PAR>;
+  auto kern = gemm_big_kernel<BITS, KEEP, GRP, PAR, TI>;
   static std::atomic<int> configured{0};
   if (!configured.load(std::memory_order_acquire)) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
       return CBK_ERR_HIP;
     configured.store(1, std::memory_order_release);
   }
-  hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), GB_LDS, st, a);
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), gb_lds(TI), st, a);
   return hipGetLastError() == hipSuccess ? CBK_OK : CBK_ERR_HIP;
+}
+
+template <int BITS, int KEEP, int GRP, int TI>
+static int launch_big_ti(const GbArgs& a, int blocks, hipStream_t st) {
+  if (a.par) return launch_big_par<BITS, KEEP, GRP, 1, TI>(a, blocks, st);
+  if (a.vs0 != 0x7fffffff) return launch_big_par<BITS, KEEP, GRP, 2, TI>(a, blocks, st);
+  if (a.nsplit > 1) return launch_big_par<BITS, KEEP, GRP, 3, TI>(a, blocks, st);
+  return launch_big_par<BITS, KEEP, GRP, 0, TI>(a, blocks, st);
 }
 
 template <int BITS, int KEEP, int GRP>
 static int launch_big_cfg(const GbArgs& a, int blocks, hipStream_t st) {
-  if (a.par) return launch_big_par<BITS, KEEP, GRP, 1>(a, blocks, st);
-  if (a.vs0 != 0x7fffffff) return launch_big_par<BITS, KEEP, GRP, 2>(a, blocks, st);
-  if (a.nsplit > 1) return launch_big_par<BITS, KEEP, GRP, 3>(a, blocks, st);
-  return launch_big_par<BITS, KEEP, GRP, 0>(a, blocks, st);
+  return a.ti == 1 ? launch_big_ti<BITS, KEEP, GRP, 1>(a, blocks, st) : launch_big_ti<BITS, KEEP, GRP, 4>(a, blocks, st);
 }
 
 // the (keep, group) instantiations of one code width

@@ -1,4 +1,4 @@
-// Prefill GEMM for M > 128: activation pre-scaling kernel, the generic-reader instantiation
+// Prefill GEMM: activation pre-scaling kernel, the generic-reader instantiation
 // and the dispatch over the per-code-width instantiations (cbk_gemm_big_b2/3/4.hip).  The
 // kernel itself is in cbk_gemm_big.h.
 #include "cbk_gemm_big.h"
@@ -69,19 +69,24 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float* par
 // 256 CUs leaves CUs idle for a whole tile time; cutting the column range gives them work at
 // the price of the float32 partial tiles (written and read once).  Times in microseconds from
 // measurements of this kernel: 1.7 per stage and 10 per workgroup, 4 TB/s for the partials.
+// 32-token blocks per wavefront: calls of at most 64 activation rows take the 64-token tile
+static inline int gb_ti(int M) { return M <= 64 ? 1 : 4; }
+
 static int gb_nsplit(const DMat& m, int M) {
   const bool le128 = (m.flags & CBK_FLAG_ZERO_LE_128) != 0;
   const int fam = family_of(m.layout);
   if (m.cs_rows > 1 || !le128 || !(fam == FAM_BLK || fam == FAM_DENSE) || m.bits < 2 || m.bits > 4) return 1;
-  const int tiles = ((M + GB_T - 1) / GB_T) * ((m.K + GB_R - 1) / GB_R);
+  const int T = 64 * gb_ti(M);
+  const int tiles = ((M + T - 1) / T) * ((m.K + GB_R - 1) / GB_R);
   const int nst = gb_npad(m.N) / GB_K;
+  const double t_stage = T == 64 ? 0.7 : 1.7, t_wg = T == 64 ? 8.0 : 10.0;
   int best = 1;
   double t1 = 0, best_t = 0;
   for (int s = 1; s <= 8; ++s) {
     const int per = ((nst + s - 1) / s + 3) / 4 * 4;                // stages per part, a multiple of 4
     if (s > 1 && (s - 1) * per >= nst) continue;                    // a part would be empty
     const double rounds = (double)((tiles * s + 255) / 256);
-    double t = rounds * (per * 1.7 + 10.0);
+    double t = rounds * (per * t_stage + t_wg);
     if (s > 1) t += 2.0 * s * (double)M * m.K * 4 / 4.0e6 + 5.0;
     if (s == 1) t1 = best_t = t;
     else if (t < best_t) { best = s; best_t = t; }
@@ -93,7 +98,7 @@ static int gb_nsplit(const DMat& m, int M) {
 static inline size_t gb_kpad(int K) { return (size_t)(K + 7) / 8 * 8; }
 
 size_t gemm_big_workspace(const DMat& m, int M) {
-  const size_t mpad = (size_t)(M + GB_T - 1) / GB_T * GB_T;
+  const size_t T = 64 * gb_ti(M), mpad = (size_t)(M + T - 1) / T * T;
   size_t b = ((m.cs_rows > 1 ? m.cs_rows : 1) * mpad * gb_npad(m.N) * 2 + 255) & ~(size_t)255;
   const int ns = gb_nsplit(m, M);
   if (ns > 1) b += ((size_t)ns * M * gb_kpad(m.K) * 4 + 255) & ~(size_t)255;
@@ -108,7 +113,8 @@ int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, v
   if (ydt != CBK_F32 && ydt != CBK_F16 && ydt != CBK_BF16T) return CBK_ERR_DTYPE;
   if (!ws || ws_bytes < gemm_big_workspace(m, M)) return CBK_ERR_WORKSPACE;
   if ((uintptr_t)ws & 255) return CBK_ERR_ALIGN;
-  const int Mpad = (M + GB_T - 1) / GB_T * GB_T;
+  const int T = 64 * gb_ti(M);
+  const int Mpad = (M + T - 1) / T * T;
   const int Npad = gb_npad(m.N);
   const int64_t items = (int64_t)Mpad * (Npad / 8);
   const int par = m.cs_rows == 2 ? 1 : 0;
@@ -127,7 +133,8 @@ int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, v
   a.part_ld = (int64_t)gb_kpad(m.K);
   a.part_stride = (size_t)M * gb_kpad(m.K);
   a.part = (float*)((uint8_t*)ws + (((size_t)(m.cs_rows > 1 ? m.cs_rows : 1) * Mpad * Npad * 2 + 255) & ~(size_t)255));
-  a.tiles_t = (M + GB_T - 1) / GB_T;
+  a.ti = gb_ti(M);
+  a.tiles_t = (M + T - 1) / T;
   a.tiles_r = par ? 2 * ((m.K + 2 * GB_R - 1) / (2 * GB_R)) : (m.K + GB_R - 1) / GB_R;
   const int nb = a.tiles_t * a.tiles_r * a.nsplit;
   const int blocks = ((nb + 7) / 8) * 8;

@@ -90,7 +90,7 @@ def gemm(pm, x, bias=None, out_dtype=None, workspace=None):
 
 
 def linear(pm, x, bias=None, out_dtype=None, workspace=None):
-    """y = x @ W_hat.T (+ bias): decode kernel up to 16 rows, prefill kernel above."""
+    """y = x @ W_hat.T (+ bias): decode kernel up to 8 rows, prefill kernel above."""
     return _matmul("cbk_linear", pm, x, bias, out_dtype, workspace)
 
 

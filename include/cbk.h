@@ -122,7 +122,7 @@ size_t cbk_row_stride(const cbk_desc* d);
 size_t cbk_stream_bytes(const cbk_desc* d, size_t sparse_data_bytes);
 
 /* Device scratch needed by cbk_gemv / cbk_gemm / cbk_linear for M activation rows (0 for the
- * decode kernels; the prefill kernel for M > 128 keeps its pre-scaled fp16 activations there:
+ * decode kernels; the prefill kernel keeps its pre-scaled fp16 activations there:
  * ceil(M/256)*256 * ceil(N/256)*256 * 2 bytes per col_scale vector, i.e. times cs_rows for a
  * fused matrix, plus float32 partial outputs when the library splits the column range of a
  * launch that would not fill the chip).  Ask, do not compute.  256-byte aligned. */
@@ -163,7 +163,7 @@ int cbk_gemm(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
              void* y, int y_dtype, int64_t ldy, const void* bias,
              void* workspace, size_t workspace_bytes, void* stream);
 
-/* The layer forward: cbk_gemv for M <= 16, cbk_gemm above (the module seam of
+/* The layer forward: cbk_gemv for M <= 8, cbk_gemm above (the module seam of
  * benchmarks/benchmark_suite.py:1200-1217). */
 int cbk_linear(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
                void* y, int y_dtype, int64_t ldy, const void* bias,

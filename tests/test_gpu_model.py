@@ -32,7 +32,7 @@ def test_hf_decoder_is_compressed_in_place_and_matches_its_dense_twin():
     assert all(x._pm().tiled for x in m.modules() if isinstance(x, CobaltLinear))
     twin = Mo.dense_twin(copy.deepcopy(m), torch.float16)
     assert not any(isinstance(x, CobaltLinear) for x in twin.modules())
-    # prefill (M = 300 rows: the 256 x 256 kernel), a short prompt (M = 24: the 128 x 128 kernel)
+    # prefill (M = 300 rows: the 256 x 256 kernel), a short prompt (M = 24: its 64-token tile)
     # and single-token steps (the decode kernel)
     for shape in ((1, 300), (2, 12), (1, 1), (3, 1)):
         ids = torch.randint(0, 512, shape, generator=g).to(DEV)

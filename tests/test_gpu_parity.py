@@ -305,7 +305,7 @@ def test_gemv_fused_rows_equal_their_unfused_parts_bit_for_bit():
 @pytest.mark.parametrize("case", FUSED_CASES[:2], ids=case_id)
 def test_gemm_fused_col_scale_rows(case):
     """Prefill on fused matrices: q|k|v ranges run the 256 x 256 kernel range by range, gate/up
-    (row parity) the 128 x 128 kernel."""
+    (row parity) as workgroups of one parity; ranges off the 16-row grid the 128 x 128 kernel."""
     K, N = 640, 1024
     for cs_rows, splits in ((3, (256, 128)), (3, (48, 16)), (2, (0, 0))):
         pm, W = _fused(case, K, N, cs_rows, splits, seed=K + cs_rows + splits[0], tiled=True)
