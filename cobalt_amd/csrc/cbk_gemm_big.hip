@@ -79,7 +79,7 @@ static int gb_nsplit(const DMat& m, int M) {
   const int T = 64 * gb_ti(M);
   const int tiles = ((M + T - 1) / T) * ((m.K + GB_R - 1) / GB_R);
   const int nst = gb_npad(m.N) / GB_K;
-  const double t_stage = T == 64 ? 0.7 : 1.7, t_wg = T == 64 ? 8.0 : 10.0;
+  const double t_stage = T == 64 ? 1.1 : 1.7, t_wg = T == 64 ? 8.0 : 10.0;   // 64-token stage: bound by the weight loads' latency
   int best = 1;
   double t1 = 0, best_t = 0;
   for (int s = 1; s <= 8; ++s) {
