@@ -14,10 +14,13 @@ numpy/float32 restatement of src/cobaltkernel/cobalt_math.py in the reference:
   cobalt_quantize     cobalt_math.py:336-371  (quant_mode='rtn', clip='none': the shipped path)
 
 Parity status.  Mask cardinalities, the RTN error bound, the OBS closed form (against a
-float64 per-row solve) and dequant are pinned by tests/test_oracle_math.py.  What stays
-"parity unpinned" at bit level: the order in which torch.topk / torch.kthvalue break exact
-ties, and the last-ulp behaviour of torch's Cholesky versus LAPACK's here.  Neither is on
-the GEMV/GEMM/dequant path; both only choose which valid RAW matrix gets produced.
+float64 per-row solve) and dequant are pinned by tests/test_oracle_math.py; the whole recipe is
+pinned against four seeded runs of the reference's own cobalt_quantize
+(tests/golden/cobalt_quantize.npz, tests/test_golden_cobalt_quantize.py): keep-masks, codes and
+zero points identical, scales and column scales equal to 2e-4 (float32 chains of LAPACK here
+and torch there; at most 3 % of them one fp16 step apart once stored).  What stays "parity
+unpinned": the order in which torch.topk / torch.kthvalue break EXACT ties, which those
+continuous inputs do not contain.  It only chooses which valid RAW matrix gets produced.
 """
 from __future__ import annotations
 
