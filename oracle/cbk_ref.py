@@ -39,7 +39,9 @@ the reference's formula, their byte layout is defined here:
 
 Parity status: every function here is pinned by tests/test_oracle_*.py through hand
 vectors, the reference documentation's known answers, an independent per-position
-decoder and round trips, except where a docstring says "parity unpinned".
+decoder and round trips, except where a docstring says "parity unpinned"; the zero-point
+repair and the variable-length layouts (SPARSE4, SPARSE4X, SPARSE4E) in addition by bytes and
+values the reference's own packer wrote (tests/golden/fix_zero_range.npz, sparse_stream.npz).
 """
 from __future__ import annotations
 
