@@ -443,6 +443,9 @@ def test_gemm_odd_chunk_count_and_ragged_tiles(case):
             assert y.dtype == odt and rel_fro(_np(y), ref) < (TOL if odt != torch.bfloat16 else 3e-3)
         xs = torch.zeros(M, N + 8, dtype=torch.float16); xs[:, :N] = x
         assert rel_fro(_np(ops.gemm(pm, xs.to(DEV)[:, :N], out_dtype=torch.float32)), ref) < TOL
+        for m in (1, 37, 64, 65):                               # the 64-token tile, ragged, and just past it
+            y = ops.gemm(pm, x[:m].to(DEV), out_dtype=torch.float32)
+            assert rel_fro(_np(y), ref[:m]) < TOL, (m, tiled)
 
 
 @pytest.mark.parametrize("case", ALL_MFMA_CASES, ids=case_id)
@@ -462,6 +465,9 @@ def test_gemm_every_kernel_configuration(case):
         err = rel_fro(_np(y), ref)
         assert err < TOL, f"{case_id(case)} tiled={tiled}: {err}"
         assert torch.equal(y, ops.gemm(pm, x.to(DEV), out_dtype=torch.float32))
+        y64 = ops.gemm(pm, x[:50].to(DEV), out_dtype=torch.float32)     # the 64-token instantiation
+        assert rel_fro(_np(y64), ref[:50]) < TOL, f"{case_id(case)} tiled={tiled} M=50"
+        assert torch.equal(y64, ops.gemm(pm, x[:50].to(DEV), out_dtype=torch.float32))
 
 
 def test_gemm_bias_dtype_and_prune_zero():
