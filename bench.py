@@ -20,6 +20,10 @@ the number of launches in it; the gaps between launches are therefore counted as
 default; --prefill-workload / --prefill-m / --prefill-dtype choose others) in TFLOP/s against
 the 2.5 PFLOP/s dense bf16/f16 MFMA peak.
 
+`gemm_m64` is the same kernel's 64-token tile at 64 activation rows (batched decoding) on the
+decode workload's MLP shapes; `measured_ceilings` are this GPU's dense f16 MFMA rate and plain
+read rate from two probe kernels.
+
 `cpu_baseline` is the C oracle (dequantise-then-matmul, OpenMP over rows) timed on the host
 cores on the SAME packed bytes as the first layer set, and doubles as a last parity check of
 the GPU outputs.
@@ -355,6 +359,10 @@ def main():
     if not a.no_prefill:
         out["prefill_gemm"] = prefill_gemm(torch, F, ops, dev, a.prefill_workload, layout, a.bits, a.group, a.keep,
                                            a.prefill_m, torch.float16 if a.prefill_dtype == "f16" else torch.bfloat16)
+        # the same kernel's 64-token tile at a batched-decoding row count, on the decode workload's shapes
+        mid = prefill_gemm(torch, F, ops, dev, a.workload, layout, a.bits, a.group, a.keep, 64,
+                           torch.float16 if a.dtype == "f16" else torch.bfloat16)
+        out["gemm_m64"] = {"workload": mid["workload"], "tflops": mid["tflops"], "per_matrix": mid["per_matrix"]}
     ceil = measured_ceilings(torch, dev)
     if ceil:
         out["measured_ceilings"] = ceil
