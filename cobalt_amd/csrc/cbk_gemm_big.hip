@@ -82,7 +82,7 @@ static int gb_nsplit(const DMat& m, int M) {
   const double t_stage = T == 64 ? 1.1 : 1.7, t_wg = T == 64 ? 8.0 : 10.0;   // 64-token stage: bound by the weight loads' latency
   int best = 1;
   double t1 = 0, best_t = 0;
-  for (int s = 1; s <= 8; ++s) {
+  for (int s = 1; s <= 16; ++s) {
     const int per = ((nst + s - 1) / s + 3) / 4 * 4;                // stages per part, a multiple of 4
     if (s > 1 && (s - 1) * per >= nst) continue;                    // a part would be empty
     const double rounds = (double)((tiles * s + 255) / 256);
