@@ -1,4 +1,6 @@
-// Prefill GEMM:  Y[M, K] = X[M, N] . W_hat[K, N]^T  with W_hat dequantised tile by tile into
+// Fallback GEMM (128 x 128 tiles, generic reader, no workspace) for what the 256 x 256 kernel
+// does not take: q|k|v matrices whose ranges start off the 16-row grid.
+//   Y[M, K] = X[M, N] . W_hat[K, N]^T  with W_hat dequantised tile by tile into
 // LDS and fed to the gfx950 matrix cores (v_mfma_f32_32x32x16_f16, fp32 accumulate).
 //
 // Numerics.  The weight tile is fp16(W_hat): the float32 value of the dequant formula,

@@ -156,7 +156,7 @@ int cbk_gemv_batch(int n, const cbk_desc* descs, const void* const* xs, const in
                    int x_dtype, int M, void* const* ys, const int64_t* ldys, int y_dtype,
                    const void* const* biases, void* workspace, size_t workspace_bytes, void* stream);
 
-/* Prefill path, any M >= 1 (built for M >= 256).  Same contract as cbk_gemv; bf16 activations
+/* Prefill path, any M >= 1 (256-token tiles; a 64-token tile up to 64 rows).  Same contract as cbk_gemv; bf16 activations
  * are carried as fp16 inside (magnitudes above 65504 saturate).  Replaces the
  * harness entry `gemm` (test_gemm.cu:151-165) and cbk::gemm_tile (cobalt_gemm.cuh:243-609). */
 int cbk_gemm(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
