@@ -307,8 +307,9 @@ def test_gemm_fused_col_scale_rows(case):
     """Prefill on fused matrices: q|k|v ranges run the 256 x 256 kernel range by range, gate/up
     (row parity) as workgroups of one parity; ranges off the 16-row grid the 128 x 128 kernel."""
     K, N = 640, 1024
-    for cs_rows, splits in ((3, (256, 128)), (3, (48, 16)), (2, (0, 0))):
-        pm, W = _fused(case, K, N, cs_rows, splits, seed=K + cs_rows + splits[0], tiled=True)
+    # (40, 24): ranges off the 16-row grid, which only the 128 x 128 fallback kernel takes
+    for cs_rows, splits in ((3, (256, 128)), (3, (48, 16)), (3, (40, 24)), (2, (0, 0))):
+        pm, W = _fused(case, K, N, cs_rows, splits, seed=K + cs_rows + splits[0], tiled=splits[0] % 16 == 0)
         for M, dtype in ((300, torch.bfloat16), (129, torch.float16), (64, torch.float16)):
             x = acts(M, N, dtype, seed=M)
             bias = acts(1, K, torch.float32, seed=9)[0]
