@@ -112,3 +112,84 @@ def total_stream_bytes(manifest: dict) -> int:
     fused matrix and are not counted twice (docs/FORMAT.md:146-151)."""
     return sum(int(e["stream_bytes"]) for entries in manifest["layers"] for e in entries.values()
                if not e.get("alias_of"))
+
+
+# ------------------------------------------------------------------ RAW artifacts
+RAW_FIELDS = ("mask", "q", "scale", "zero", "col_scale")
+
+
+def write_raw_artifact(path: str, layers: List[Dict[str, Dict[str, torch.Tensor]]], config: Optional[dict] = None,
+                       stats: Optional[List[Dict[str, dict]]] = None) -> dict:
+    """The compressor's output before packing, as the reference writes it
+    (src/cobaltkernel/quantize_cobalt.py:439-443, :467): one `layer_XX.safetensors` per decoder
+    layer holding `<name>.{mask,q,scale,zero,col_scale}` for every linear of the layer
+    (src/cobaltkernel/pack_cobalt.py:3-11), and a `manifest.json` with the run's configuration
+    and per-matrix entries (`shape`, `bits`, ...)."""
+    from safetensors.torch import save_file
+    os.makedirs(path, exist_ok=True)
+    manifest = {"config": dict(config or {}), "layers": {}}
+    for li, mats in enumerate(layers):
+        tensors, entries = {}, {}
+        for name, raw in mats.items():
+            for f in RAW_FIELDS:
+                tensors[f"{name}.{f}"] = raw[f].detach().cpu().contiguous()
+            e = {"shape": [int(raw["q"].shape[0]), int(raw["q"].shape[1])]}
+            if stats is not None:
+                e.update(stats[li].get(name, {}))
+            entries[name] = e
+        save_file(tensors, os.path.join(path, f"layer_{li:02d}.safetensors"))
+        manifest["layers"][str(li)] = entries
+    with open(os.path.join(path, "manifest.json"), "w") as f:
+        json.dump(manifest, f, indent=1)
+    return manifest
+
+
+def read_raw_artifact(path: str) -> Tuple[dict, List[Dict[str, Dict[str, torch.Tensor]]]]:
+    """(manifest, layers[i][name] = {mask, q, scale, zero, col_scale}) of a RAW artifact directory;
+    the manifest is {} if the directory has none."""
+    from safetensors.torch import load_file
+    manifest = {}
+    mp = os.path.join(path, "manifest.json")
+    if os.path.exists(mp):
+        with open(mp) as f:
+            manifest = json.load(f)
+    files = sorted(n for n in os.listdir(path) if n.startswith("layer_") and n.endswith(".safetensors"))
+    if not files:
+        raise FileNotFoundError(f"no layer_XX.safetensors in {path}")
+    layers = []
+    for n in files:
+        flat = load_file(os.path.join(path, n))
+        mats: Dict[str, Dict[str, torch.Tensor]] = {}
+        for key, t in flat.items():
+            name, field = key.rsplit(".", 1)
+            if field not in RAW_FIELDS:
+                raise ValueError(f"{n}: unexpected tensor {key}")
+            mats.setdefault(name, {})[field] = t
+        for name, raw in mats.items():
+            missing = [f for f in RAW_FIELDS if f not in raw]
+            if missing:
+                raise ValueError(f"{n}: {name} lacks {missing}")
+        layers.append(mats)
+    return manifest, layers
+
+
+def raw_layout(raw: Dict[str, torch.Tensor], bits: Optional[int] = None) -> Tuple[int, int, int, Optional[int]]:
+    """(layout, bits, group, keep) a RAW matrix packs to: dense if nothing is pruned, a blocked
+    layout if every 32-column block keeps the same number of columns.  `bits` comes from the
+    artifact's manifest when it has it, else from the largest code."""
+    K, N = raw["q"].shape
+    group = N // raw["scale"].shape[1]
+    if bits is None:
+        top = int(raw["q"].max())
+        bits = 2 if top < 4 else 3 if top < 8 else 4 if top < 16 else 8
+    keep_map = F.unpack_mask(raw["mask"], N)
+    if bool(keep_map.all()):
+        return (F.DENSE4 if (bits, group) == (4, 128) else F.DENSE8 if (bits, group) == (8, 128) else F.DENSEB), bits, group, None
+    cnt = keep_map.reshape(K, N // F.BLOCK, F.BLOCK).sum(-1)
+    k0 = int(cnt[0, 0])
+    if bool((cnt == k0).all()):
+        if (bits, group, k0) == (4, 128, 16):
+            return F.BLK1632_4, 4, 128, 16
+        return F.BLKC, bits, group, k0
+    raise ValueError("a mask without a fixed number of survivors per 32 columns packs to the variable-length "
+                     "layouts, which this package reads but does not produce")

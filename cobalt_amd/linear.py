@@ -47,16 +47,19 @@ class CobaltLinear(nn.Module):
     @classmethod
     def from_linear(cls, linear: nn.Module, X_cal: Optional[torch.Tensor] = None, H: Optional[torch.Tensor] = None,
                     sparsity: float = 0.5, bits: int = 4, group: int = 128, beta: float = 0.5, mask_block: int = 32,
-                    meta=None) -> "CobaltLinear":
+                    meta=None, raw_sink: Optional[dict] = None, raw_name: Optional[str] = None) -> "CobaltLinear":
         """Compress an `nn.Linear` with CoBALT and pack it (the role of `CPRLinear.from_linear`,
         sinq/cprlinear.py:128-171, with the pipeline of src/cobaltkernel/quantize_cobalt.py:424-443).
         Calibration comes as activations X_cal [tokens, in_features] or as H = X^T X; without
-        either, H = I (magnitude pruning, no OBS signal).  The module lands on the linear's device."""
+        either, H = I (magnitude pruning, no OBS signal).  The module lands on the linear's device.
+        `raw_sink[raw_name]` receives the RAW arrays {mask, q, scale, zero, col_scale} on the CPU."""
         from . import compress as Cp
         W = linear.weight.data
         if H is None:
             H = Cp.hessian(X_cal.to(W.device)) if X_cal is not None else torch.eye(W.shape[1], device=W.device)
         raw = Cp.cobalt_compress(W, H.to(W.device), sparsity, bits, group, beta, mask_block)
+        if raw_sink is not None:
+            raw_sink[raw_name or "linear"] = {f: raw[f].detach().cpu() for f in ("mask", "q", "scale", "zero", "col_scale")}
         layout, keep = Cp.layout_for(sparsity, bits, group, mask_block)
         pm = F.pack_raw(raw["mask"], raw["q"], raw["scale"], raw["zero"], raw["col_scale"], layout, bits, group, keep)
         bias = linear.bias.data if getattr(linear, "bias", None) is not None else None

@@ -90,7 +90,8 @@ def compress_model(model: nn.Module, calib_ids: Optional[torch.Tensor] = None, s
                    bits_override: Optional[Dict[str, int]] = None,
                    sparsity_override: Optional[Dict[str, float]] = None, seq_inputs: bool = False,
                    fuse: bool = False,
-                   forward: Optional[Callable[[nn.Module, torch.Tensor], object]] = None) -> Dict[str, dict]:
+                   forward: Optional[Callable[[nn.Module, torch.Tensor], object]] = None,
+                   raw_out: Optional[str] = None) -> Dict[str, dict]:
     """Replace the linears of every decoder block by `CobaltLinear` modules compressed against
     the calibration tokens `calib_ids` [n, seq] (None: no calibration, H = I).  Per-matrix
     `bits_override` / `sparsity_override` are keyed by the names in LINEARS
@@ -98,6 +99,9 @@ def compress_model(model: nn.Module, calib_ids: Optional[torch.Tensor] = None, s
     modules are installed when all blocks are done; with `seq_inputs` every pass of
     `layers_per_pass` blocks is installed at once and later passes calibrate on the compressed
     prefix (quantize_cobalt.py:444-452).  `fuse` row-fuses q|k|v and gate/up afterwards (fuse_model).
+    `raw_out` also writes the RAW artifact of the run (one `layer_XX.safetensors` per block with
+    `<name>.{mask,q,scale,zero,col_scale}` + manifest.json, quantize_cobalt.py:439-467), which
+    `install_raw_artifact` and the reference's packer read.
     Returns {qualified linear name: {shape, layout, bpw,
     bits, sparsity}}."""
     blocks = decoder_blocks(model)
@@ -112,6 +116,8 @@ def compress_model(model: nn.Module, calib_ids: Optional[torch.Tensor] = None, s
     model.eval()
     report: Dict[str, dict] = {}
     pending: List[Tuple[nn.Module, str, nn.Module]] = []
+    raw_layers: List[Dict[str, Dict[str, torch.Tensor]]] = []
+    raw_stats: List[Dict[str, dict]] = []
 
     def install():
         for parent, attr, new in pending:
@@ -128,6 +134,8 @@ def compress_model(model: nn.Module, calib_ids: Optional[torch.Tensor] = None, s
             batches = (calib_ids[i:i + batch_size] for i in range(0, calib_ids.shape[0], batch_size))
             Hs = collect_hessians(model, chunk, batches, forward)
         for bname, blk in chunk:
+            raws: Dict[str, Dict[str, torch.Tensor]] = {}
+            rstats: Dict[str, dict] = {}
             for g, names in HGROUPS.items():
                 H = Hs.pop((bname, g), None)
                 for lname in names:
@@ -138,7 +146,9 @@ def compress_model(model: nn.Module, calib_ids: Optional[torch.Tensor] = None, s
                     nb = bits_override.get(lname, bits)
                     mb = 0 if sp == 0.0 else mask_block
                     new = CobaltLinear.from_linear(lin, H=H, sparsity=sp, bits=nb, group=group, beta=beta,
-                                                   mask_block=mb)
+                                                   mask_block=mb, raw_sink=raws if raw_out else None,
+                                                   raw_name=lname.rsplit(".", 1)[1])
+                    rstats[lname.rsplit(".", 1)[1]] = dict(bits=nb, sparsity_target=sp, mask_block=mb)
                     if device_order and new.blob.is_cuda:
                         new.to_device_order()
                     pending.append((_sub(blk, lname.rsplit(".", 1)[0]), lname.rsplit(".", 1)[1], new))
@@ -146,9 +156,17 @@ def compress_model(model: nn.Module, calib_ids: Optional[torch.Tensor] = None, s
                     report[f"{bname}.{lname}" if bname else lname] = dict(
                         shape=[pm.K, pm.N], layout=pm.layout, bpw=pm.bpw(), bits=nb, sparsity=sp)
                 del H
+            if raw_out:
+                raw_layers.append({n.rsplit(".", 1)[1]: raws[n.rsplit(".", 1)[1]] for n in LINEARS if n.rsplit(".", 1)[1] in raws})
+                raw_stats.append(rstats)
         if seq_inputs:
             install()
     install()
+    if raw_out:
+        from . import container
+        container.write_raw_artifact(raw_out, raw_layers, stats=raw_stats,
+                                     config=dict(sparsity=sparsity, bits=bits, group_size=group, beta=beta,
+                                                 mask_block=mask_block))
     if fuse:
         fuse_model(model, device_order)
     if was_training:
@@ -308,6 +326,45 @@ def fuse_model(model: nn.Module, device_order: bool = True, gated_mlp: bool = Tr
                 if ok and il and gated_mlp:
                     _install_gated_forward(_sub(blk, names[0].rsplit(".", 1)[0]))
     return n
+
+
+def install_raw_artifact(model: nn.Module, path: str, device_order: bool = True, fuse: bool = False) -> Dict[str, dict]:
+    """Install a RAW artifact directory (layer_XX.safetensors per decoder block, the reference
+    compressor's output, src/cobaltkernel/quantize_cobalt.py:439-467) into `model`: every linear
+    of every block is packed (pack_cobalt.py:98-199) and replaced by a `CobaltLinear` that keeps
+    the linear's bias and lands on its device.  Returns the same report as `compress_model`."""
+    from . import container
+    manifest, layers = container.read_raw_artifact(path)
+    blocks = decoder_blocks(model)
+    if len(layers) != len(blocks):
+        raise ValueError(f"the artifact has {len(layers)} layers, the model {len(blocks)} decoder blocks")
+    report: Dict[str, dict] = {}
+    for li, ((bname, blk), mats) in enumerate(zip(blocks, layers)):
+        entries = manifest.get("layers", {}).get(str(li), {})
+        for lname in LINEARS:
+            short = lname.rsplit(".", 1)[1]
+            if short not in mats:
+                raise ValueError(f"layer {li}: no {short} in the artifact")
+            raw = mats[short]
+            lin = _sub(blk, lname)
+            K, N = raw["q"].shape
+            if (lin.out_features, lin.in_features) != (K, N):
+                raise ValueError(f"layer {li} {short}: artifact {K}x{N}, model {lin.out_features}x{lin.in_features}")
+            layout, nb, grp, keep = container.raw_layout(raw, entries.get(short, {}).get("bits"))
+            dev = lin.weight.device if isinstance(lin, nn.Linear) else lin.blob.device
+            t = {f: raw[f].to(dev) for f in container.RAW_FIELDS}
+            bias = lin.bias.data if getattr(lin, "bias", None) is not None else None
+            new = CobaltLinear.from_raw(t["mask"], t["q"], t["scale"], t["zero"], t["col_scale"], bias=bias,
+                                        layout=layout, bits=nb, group=grp, keep=keep)
+            if device_order and new.blob.is_cuda:
+                new.to_device_order()
+            setattr(_sub(blk, lname.rsplit(".", 1)[0]), short, new)
+            pm = new.packed()
+            report[f"{bname}.{lname}" if bname else lname] = dict(shape=[K, N], layout=pm.layout, bpw=pm.bpw(), bits=nb,
+                                                                 sparsity=1.0 - pm.n_survivors / float(K * N))
+    if fuse:
+        fuse_model(model, device_order)
+    return report
 
 
 def dense_twin(model: nn.Module, dtype: Optional[torch.dtype] = None) -> nn.Module:

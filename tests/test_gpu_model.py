@@ -97,3 +97,22 @@ def test_fused_qkv_and_gate_up_match_the_separate_modules():
         ids.copy_(torch.randint(0, 512, (1, 4), generator=g).to(DEV))
         y2 = f(ids).logits
         assert not torch.equal(y1, y2) and float((y2.float() - m(ids).logits.float()).norm()) < 5e-3 * float(y2.float().norm())
+
+
+def test_raw_artifact_installs_on_the_gpu(tmp_path):
+    """The RAW artifact written beside a compression run, installed into a second model on the GPU
+    (fused at installation), gives the logits of the first."""
+    from cobalt_amd import model as Mo
+    m = _tiny_mistral()
+    g = torch.Generator().manual_seed(3)
+    calib = torch.randint(0, 512, (4, 32), generator=g).to(DEV)
+    out = str(tmp_path / "raw")
+    Mo.compress_model(m, calib, raw_out=out)
+    m2 = _tiny_mistral()
+    rep = Mo.install_raw_artifact(m2, out, fuse=True)
+    assert len(rep) == 14 and all(abs(r["bpw"] - 3.1875) < 1e-9 for r in rep.values())
+    for shape in ((1, 40), (2, 1)):
+        ids = torch.randint(0, 512, shape, generator=g).to(DEV)
+        with torch.no_grad():
+            a, b = m(ids).logits.float(), m2(ids).logits.float()
+        assert float((a - b).norm() / a.norm()) < 5e-3, shape

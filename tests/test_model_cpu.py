@@ -138,3 +138,46 @@ def test_fuse_model_structure():
     keys = [k for k in m.state_dict() if k.startswith("layers.0.")]
     assert sum(k.endswith("blob") for k in keys) == 4              # one packed image per fused group
     assert len(Mo.decoder_blocks(m)) == 2
+
+
+def test_raw_artifact_round_trip_installs_the_same_bytes(tmp_path):
+    """compress_model(raw_out=...) writes the compressor's output in the reference's RAW schema
+    (layer_XX.safetensors with <name>.{mask,q,scale,zero,col_scale}, pack_cobalt.py:3-11);
+    installing that directory into a fresh model gives byte-identical packed modules, with the
+    overrides (3-bit down, dense o) found again from the artifact alone."""
+    from cobalt_amd import container as Ct
+    torch.manual_seed(1)
+    m = _Toy(layers=2)
+    ids = torch.randint(0, 64, (4, 16))
+    out = str(tmp_path / "raw")
+    rep = Mo.compress_model(m, ids, sparsity=0.5, bits=4, group=128, layers_per_pass=1,
+                            bits_override={"mlp.down_proj": 3}, sparsity_override={"self_attn.o_proj": 0.0},
+                            raw_out=out)
+    manifest, layers = Ct.read_raw_artifact(out)
+    assert len(layers) == 2 and set(layers[0]) == {n.rsplit(".", 1)[1] for n in Mo.LINEARS}
+    raw = layers[1]["gate_proj"]
+    assert raw["mask"].dtype == torch.uint8 and raw["mask"].shape == (384, 256 // 8)
+    assert raw["q"].dtype == torch.uint8 and raw["q"].shape == (384, 256)
+    assert raw["scale"].dtype == torch.float16 and raw["zero"].dtype == torch.float16 and raw["scale"].shape == (384, 2)
+    assert raw["col_scale"].dtype == torch.float16 and raw["col_scale"].shape == (256,)
+    assert manifest["layers"]["0"]["down_proj"]["bits"] == 3 and manifest["layers"]["0"]["down_proj"]["shape"] == [256, 384]
+    assert manifest["config"]["group_size"] == 128
+    torch.manual_seed(1)
+    m2 = _Toy(layers=2)
+    rep2 = Mo.install_raw_artifact(m2, out)
+    assert set(rep2) == set(rep)
+    for k in rep:
+        assert rep2[k]["layout"] == rep[k]["layout"] and rep2[k]["bits"] == rep[k]["bits"], k
+        assert abs(rep2[k]["bpw"] - rep[k]["bpw"]) < 1e-12
+    for li in range(2):
+        for name in Mo.LINEARS:
+            a, b = Mo._sub(m.layers[li], name), Mo._sub(m2.layers[li], name)
+            assert isinstance(b, CobaltLinear) and torch.equal(a.blob, b.blob), (li, name)
+            assert (a.bias is None) == (b.bias is None)
+    # an artifact of another depth, or a mask no fixed-stride layout holds, is refused
+    with pytest.raises(ValueError):
+        Mo.install_raw_artifact(_Toy(layers=3), out)
+    bad = {f: t.clone() for f, t in layers[0]["q_proj"].items()}
+    bad["mask"][0, 0] ^= 1
+    with pytest.raises(ValueError):
+        Ct.raw_layout(bad)
