@@ -66,6 +66,23 @@ class CobaltLinear(nn.Module):
         return cls(pm, bias, meta)
 
     @classmethod
+    def from_state(cls, blob: torch.Tensor, cbk_meta: torch.Tensor, bias: Optional[torch.Tensor] = None) -> "CobaltLinear":
+        """From the two buffers a saved module holds in a state dict (`<name>.blob`, `<name>.cbk_meta`)."""
+        if blob.dtype != torch.uint8 or cbk_meta.numel() != len(_META_FIELDS):
+            raise ValueError("not the buffers of a CobaltLinear")
+        self = cls.__new__(cls)
+        nn.Module.__init__(self)
+        d = dict(zip(_META_FIELDS, [int(t) for t in cbk_meta.tolist()]))
+        self.in_features, self.out_features = d["N"], d["K"]
+        self.register_buffer("blob", blob)
+        self.register_buffer("cbk_meta", cbk_meta.to("cpu", torch.int64).clone())
+        self.bias = nn.Parameter(bias.detach().clone(), requires_grad=False) if bias is not None else None
+        self.meta = {}
+        self._backend = "hip"
+        self.packed().desc()                                          # raises on an inconsistent description
+        return self
+
+    @classmethod
     def from_sparse_quant_linear(cls, m: nn.Module, layout: Optional[int] = None) -> "CobaltLinear":
         """From the reference's unpacked module: buffers W_q [K,N], scales/zeros [K,G,1], mask [K,N],
         scale2 [1,N] or [N], `bias`, meta{'nbits','group_size'} (benchmark_suite.py:1178-1198,

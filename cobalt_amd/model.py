@@ -367,6 +367,33 @@ def install_raw_artifact(model: nn.Module, path: str, device_order: bool = True,
     return report
 
 
+def load_compressed_state_dict(model: nn.Module, state_dict: Dict[str, torch.Tensor], strict: bool = True):
+    """Load the state dict of a compressed model into a model that still has its dense linears.
+    The module class is picked from the keys, the way the reference's loader does
+    ('W_high_packed' -> CPRLinear, 'W_q' -> SINQLinear, sinq/patch_model.py:1129-1149): a name
+    with `<name>.blob` and `<name>.cbk_meta` becomes a `CobaltLinear` built from those buffers, on
+    the device of the module it replaces; everything else goes through `load_state_dict`."""
+    names = [k[: -len(".cbk_meta")] for k in state_dict if k.endswith(".cbk_meta") and k[: -len(".cbk_meta")] + ".blob" in state_dict]
+    modules = dict(model.named_modules())
+    for name in names:
+        old = modules.get(name)
+        if old is None:
+            if strict:
+                raise KeyError(f"the state dict packs {name}, which the model does not have")
+            continue
+        if isinstance(old, CobaltLinear):
+            continue                                                  # already packed: an ordinary buffer load
+        dev = next((p.device for p in old.parameters()), torch.device("cpu"))
+        bias = state_dict.get(name + ".bias")
+        new = CobaltLinear.from_state(state_dict[name + ".blob"].to(dev), state_dict[name + ".cbk_meta"],
+                                      None if bias is None else bias.to(dev))
+        if isinstance(old, nn.Linear) and (old.in_features, old.out_features) != (new.in_features, new.out_features):
+            raise ValueError(f"{name}: packed {new.out_features}x{new.in_features}, model {old.out_features}x{old.in_features}")
+        parent = modules[name.rsplit(".", 1)[0]] if "." in name else model
+        setattr(parent, name.rsplit(".", 1)[-1], new)
+    return model.load_state_dict(state_dict, strict=strict)
+
+
 def dense_twin(model: nn.Module, dtype: Optional[torch.dtype] = None) -> nn.Module:
     """The same model with every `CobaltLinear` turned back into an `nn.Linear` that holds the
     dequantised weight: what the packed model computes, through the dense library GEMM.  Modifies

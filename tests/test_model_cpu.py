@@ -181,3 +181,29 @@ def test_raw_artifact_round_trip_installs_the_same_bytes(tmp_path):
     bad["mask"][0, 0] ^= 1
     with pytest.raises(ValueError):
         Ct.raw_layout(bad)
+
+
+def test_state_dict_of_a_compressed_model_loads_into_a_dense_one():
+    """The loader picks `CobaltLinear` from the keys `<name>.blob` / `<name>.cbk_meta`
+    (the reference picks its module classes the same way, sinq/patch_model.py:1129-1149)."""
+    torch.manual_seed(2)
+    m = _Toy(layers=2)
+    Mo.compress_model(m, torch.randint(0, 64, (2, 16)), bits_override={"mlp.up_proj": 2})
+    sd = {k: v.clone() for k, v in m.state_dict().items()}
+    torch.manual_seed(3)
+    m2 = _Toy(layers=2)                                              # dense, other weights
+    res = Mo.load_compressed_state_dict(m2, sd)
+    assert not res.missing_keys and not res.unexpected_keys
+    for li in range(2):
+        for name in Mo.LINEARS:
+            a, b = Mo._sub(m.layers[li], name), Mo._sub(m2.layers[li], name)
+            assert isinstance(b, CobaltLinear) and torch.equal(a.blob, b.blob) and torch.equal(a.cbk_meta, b.cbk_meta)
+            assert (a.bias is None and b.bias is None) or torch.equal(a.bias, b.bias)
+            assert b._pm().bits == a._pm().bits
+    assert torch.equal(m2.embed.weight, m.embed.weight) and isinstance(m2.lm_head, nn.Linear)
+    # a truncated blob is caught when the module is built, not at the first launch
+    bad = dict(sd); bad["layers.0.mlp.up_proj.cbk_meta"] = sd["layers.0.mlp.up_proj.cbk_meta"][:5]
+    with pytest.raises(ValueError):
+        Mo.load_compressed_state_dict(_Toy(layers=2), bad)
+    with pytest.raises(KeyError):
+        Mo.load_compressed_state_dict(_Toy(layers=1), sd)
