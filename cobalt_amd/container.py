@@ -114,6 +114,80 @@ def total_stream_bytes(manifest: dict) -> int:
                if not e.get("alias_of"))
 
 
+def check_container(path: str, layers: int = 2, device="cpu", strict: bool = True) -> dict:
+    """Structural and numerical check of a CBK1 directory, the role of the reference's
+    `check_artifact` (src/prod/verify.py:64-152): every array lies inside its blob, the bytes per
+    weight add up, and, for the first `layers` layers, every blocked matrix keeps exactly `keep`
+    columns in every 32-column block.  With a GPU `device` the matrices are also dequantised by the
+    library: all values finite, every pruned position exactly zero.  Returns a report with the
+    list of `problems`; raises ValueError on any of them if `strict`."""
+    with open(os.path.join(path, "manifest.json")) as f:
+        man = json.load(f)
+    problems: List[str] = []
+    rep = {"path": path, "format": man.get("format"), "matrices": {}, "problems": problems}
+    if man.get("format") != FORMAT_NAME:
+        problems.append(f"format is {man.get('format')!r}, want {FORMAT_NAME!r}")
+    sizes: Dict[str, int] = {}
+    for li, entries in enumerate(man.get("layers", [])):
+        for name, e in entries.items():
+            bn = e["blob"]
+            bp = os.path.join(path, bn)
+            if bn not in sizes:
+                if not os.path.exists(bp):
+                    problems.append(f"missing blob {bn}")
+                    sizes[bn] = -1
+                else:
+                    sizes[bn] = os.path.getsize(bp)
+            if sizes[bn] < 0:
+                continue
+            for an, a in e["arrays"].items():
+                if a["off"] % F.ARR_ALIGN:
+                    problems.append(f"{bn}:{name}.{an} starts at {a['off']}, not on a {F.ARR_ALIGN}-byte boundary")
+                if a["off"] + a["bytes"] > sizes[bn]:
+                    problems.append(f"{bn}:{name}.{an} runs past the blob ({a['off']}+{a['bytes']} > {sizes[bn]})")
+    rep["blob_bytes"] = sum(v for v in sizes.values() if v > 0)
+    owned = [e for entries in man.get("layers", []) for e in entries.values() if not e.get("alias_of")]
+    params = sum(e["K"] * e["N"] for e in owned)
+    if params:
+        rep["bpw"] = 8.0 * sum(e["stream_bytes"] for e in owned) / params
+        want = sum(e["bpw"] * e["K"] * e["N"] for e in owned) / params
+        if abs(rep["bpw"] - want) > 1e-6:
+            problems.append(f"bytes per weight recompute to {rep['bpw']:.6f}, the entries say {want:.6f}")
+    if not problems:
+        on_gpu = torch.device(device).type == "cuda"
+        _, mats_by_layer = read_container(path, device=device, include_aliases=False)
+        for li, mats in enumerate(mats_by_layer[:layers]):
+            for name, pm in mats.items():
+                info = {"layout": F.LAYOUT_NAME[pm.layout], "shape": [pm.K, pm.N]}
+                keep = None
+                if pm.layout in (F.BLK1632_4, F.BLK1632_6, F.BLKC):
+                    st = F.row_stride(pm.layout, pm.N, pm.bits, pm.group, pm.keep or None)
+                    rows = pm.array("data")[: pm.K * st].view(pm.K, st)
+                    keep = F.unpack_mask(rows[:, : pm.N // 8], pm.N)
+                    cnt = keep.reshape(pm.K, pm.N // F.BLOCK, F.BLOCK).sum(-1)
+                    lo, hi = int(cnt.min()), int(cnt.max())
+                    info["block_survivors"] = [lo, hi]
+                    if not lo == hi == pm.keep:
+                        problems.append(f"layer {li} {name}: {lo}..{hi} survivors per 32-column block, want exactly {pm.keep}")
+                if on_gpu:
+                    from . import ops
+                    W = ops.dequant(pm, torch.float32)
+                    info["finite"] = bool(torch.isfinite(W).all())
+                    info["zero_fraction"] = float((W == 0).float().mean())
+                    if not info["finite"]:
+                        problems.append(f"layer {li} {name}: non-finite weights")
+                    if keep is not None:
+                        info["pruned_nonzero"] = int((W[~keep] != 0).sum())
+                        info["survivors_on_zero_code"] = int((W[keep] == 0).sum())
+                        if info["pruned_nonzero"]:
+                            problems.append(f"layer {li} {name}: {info['pruned_nonzero']} pruned positions do not decode to zero")
+                rep["matrices"][f"{li}:{name}"] = info
+    rep["ok"] = not problems
+    if problems and strict:
+        raise ValueError("container check failed:\n  " + "\n  ".join(problems))
+    return rep
+
+
 # ------------------------------------------------------------------ RAW artifacts
 RAW_FIELDS = ("mask", "q", "scale", "zero", "col_scale")
 

@@ -85,3 +85,47 @@ def test_alias_entries_point_into_the_fused_matrix(tmp_path):
     # totals skip the aliases
     assert Ct.total_stream_bytes(man2) == fused.stream_bytes()
     assert "q_proj" not in Ct.read_container(str(tmp_path), include_aliases=False)[1][0]
+
+
+def test_check_container_finds_what_is_wrong(tmp_path):
+    """The structural half of the checker (the role of src/prod/verify.py:64-152) on the CPU:
+    a good directory passes; a truncated blob, a wrong byte count and a block with the wrong
+    number of survivors are each reported."""
+    import pytest
+    import shutil
+    layers = [{"q_proj": F.synth_packed(64, 256, F.BLK1632_4, seed=1),
+               "down_proj": F.synth_packed(32, 512, F.BLKC, 3, 64, 10, seed=2)}]
+    good = str(tmp_path / "good")
+    Ct.write_container(good, layers)
+    rep = Ct.check_container(good)
+    assert rep["ok"] and abs(rep["bpw"] - Ct.total_stream_bytes(json.load(open(good + "/manifest.json"))) * 8.0 / (64 * 256 + 32 * 512)) < 1e-9
+    assert rep["matrices"]["0:q_proj"]["block_survivors"] == [16, 16] and rep["matrices"]["0:down_proj"]["block_survivors"] == [10, 10]
+
+    def variant(name):
+        d = str(tmp_path / name)
+        shutil.copytree(good, d)
+        return d
+
+    d = variant("short")
+    with open(d + "/layer_00.bin", "r+b") as f:
+        f.truncate(1000)
+    rep = Ct.check_container(d, strict=False)
+    assert not rep["ok"] and any("runs past the blob" in p for p in rep["problems"])
+    with pytest.raises(ValueError):
+        Ct.check_container(d)
+
+    d = variant("bytes")
+    man = json.load(open(d + "/manifest.json"))
+    man["layers"][0]["q_proj"]["stream_bytes"] += 64
+    json.dump(man, open(d + "/manifest.json", "w"))
+    assert any("bytes per weight" in p for p in Ct.check_container(d, strict=False)["problems"])
+
+    d = variant("mask")
+    man = json.load(open(d + "/manifest.json"))
+    off = man["layers"][0]["q_proj"]["arrays"]["data"]["off"]
+    with open(d + "/layer_00.bin", "r+b") as f:
+        f.seek(off)
+        b = f.read(1)
+        f.seek(off)
+        f.write(bytes([b[0] ^ 1]))                                   # one more or one fewer survivor in block 0 of row 0
+    assert any("survivors per 32-column block" in p for p in Ct.check_container(d, strict=False)["problems"])

@@ -116,3 +116,19 @@ def test_raw_artifact_installs_on_the_gpu(tmp_path):
         with torch.no_grad():
             a, b = m(ids).logits.float(), m2(ids).logits.float()
         assert float((a - b).norm() / a.norm()) < 5e-3, shape
+
+
+def test_check_container_on_the_gpu(tmp_path):
+    """The numerical half of the container checker: blobs on the GPU, dequantised by the library;
+    finite values, every pruned position exactly zero."""
+    from cobalt_amd import container as Ct, format as F
+    layers = [{"q_proj": F.synth_packed(64, 256, F.BLK1632_4, seed=1),
+               "up_proj": F.synth_packed(48, 384, F.BLKC, 2, 64, 23, seed=2),
+               "down_proj": F.synth_packed(32, 512, F.DENSE4, seed=3)}]
+    Ct.write_container(str(tmp_path), layers)
+    rep = Ct.check_container(str(tmp_path), device=DEV)
+    assert rep["ok"]
+    q = rep["matrices"]["0:q_proj"]
+    assert q["finite"] and q["pruned_nonzero"] == 0 and q["zero_fraction"] >= 0.5
+    assert rep["matrices"]["0:up_proj"]["block_survivors"] == [23, 23]
+    assert "pruned_nonzero" not in rep["matrices"]["0:down_proj"] and rep["matrices"]["0:down_proj"]["finite"]
