@@ -64,6 +64,11 @@ __device__ inline uint32_t window(const uint32_t (&s)[NW], uint32_t sh) {
   return w;
 }
 
+// Bitwise select under an all-ones / all-zeros mask (see align_chunk_codes for why not `c ? b : a`).
+__device__ inline uint32_t mask_select(uint32_t mask, uint32_t if_clear, uint32_t if_set) {
+  return (if_set & mask) | (if_clear & ~mask);                   // one v_bfi_b32
+}
+
 // pool bytes holding a code q each  ->  signed bytes q - z   (z <= 128, carried in nz)
 __device__ inline uint32_t bias_pool(uint32_t codes, uint32_t nz) { return (codes + nz) ^ 0x80808080u; }
 
@@ -98,11 +103,18 @@ __device__ inline void align_chunk_codes(const uint32_t (&raw)[C::NL], uint32_t 
 #pragma unroll
     for (int i = 0; i < C::NL; ++i)
       t1[i] = C::ALIGNED ? raw[i] : __builtin_amdgcn_alignbit(i + 1 < C::NL ? raw[i + 1] : 0u, raw[i], skew);
+    // Shift by one and by two dwords with bitwise selects under a sign-extended bit of the skew.
+    // Written as C++ conditionals the compiler turns the two steps into one read of the array at
+    // a run-time index, which puts the array into scratch memory (a store and a load of every
+    // dword per chunk).  Not inline assembly either: the compiler inserts no wait states between
+    // an MFMA and an assembly statement that overwrites one of the MFMA's result registers.
+    const uint32_t m32 = (uint32_t)__builtin_amdgcn_sbfe((int)skew, 5, 1);
+    const uint32_t m64 = (uint32_t)__builtin_amdgcn_sbfe((int)skew, 6, 1);
     uint32_t t2[C::NL];
 #pragma unroll
-    for (int i = 0; i < C::NL; ++i) t2[i] = (skew & 32u) ? (i + 1 < C::NL ? t1[i + 1] : 0u) : t1[i];
+    for (int i = 0; i < C::NL; ++i) t2[i] = mask_select(m32, t1[i], i + 1 < C::NL ? t1[i + 1] : 0u);
 #pragma unroll
-    for (int i = 0; i < C::ND; ++i) cw[i] = (skew & 64u) ? (i + 2 < C::NL ? t2[i + 2] : 0u) : t2[i];
+    for (int i = 0; i < C::ND; ++i) cw[i] = mask_select(m64, t2[i], i + 2 < C::NL ? t2[i + 2] : 0u);
   }
 }
 
