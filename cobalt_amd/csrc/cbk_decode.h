@@ -69,6 +69,22 @@ __device__ inline uint32_t mask_select(uint32_t mask, uint32_t if_clear, uint32_
   return (if_set & mask) | (if_clear & ~mask);                   // one v_bfi_b32
 }
 
+// BLK1632_6: the high two bits of the eight survivors from rank r on, as the two byte pools of
+// decode (even positions of the window, odd positions), already at bits 4-5 of their bytes.
+// Survivor i of a block keeps its high bits at bit i of the block's dword if i is even, at bit
+// i + 15 if it is odd (src/cobaltkernel/dequant_ref.py:61-66).
+__device__ inline uint32_t spread_hi2(uint32_t f) {               // four 2-bit fields -> bits 4-5 of four bytes
+  uint32_t x = f & 0xFFu;
+  x = (x | (x << 12)) & 0x000F000Fu;
+  x = (x | (x << 6)) & 0x03030303u;
+  return x << 4;
+}
+__device__ inline void hi2_pools(uint32_t hw, uint32_t r, uint32_t& h0, uint32_t& h1) {
+  const uint32_t odd = r & 1u;
+  h0 = spread_hi2(hw >> ((r + 15u * odd) & 31u));                 // positions r, r+2, r+4, r+6
+  h1 = spread_hi2(hw >> ((r + 16u - 15u * odd) & 31u));           // positions r+1, r+3, r+5, r+7
+}
+
 // pool bytes holding a code q each  ->  signed bytes q - z   (z <= 128, carried in nz)
 __device__ inline uint32_t bias_pool(uint32_t codes, uint32_t nz) { return (codes + nz) ^ 0x80808080u; }
 
@@ -77,14 +93,18 @@ __device__ inline uint32_t bias_pool(uint32_t codes, uint32_t nz) { return (code
 template <int BITS, int KEEP, int GRP>
 struct CodeCfg {
   static constexpr bool DENSE = KEEP == 0;
-  static constexpr int CB = DENSE ? 32 * BITS : KEEP * BITS;      // code bits per 32-column block
+  // BITS 6 is BLK1632_6: a 4-bit stream of low nibbles exactly like BLK1632_4, and the two high
+  // bits of every survivor in a plane of their own (one dword per block)
+  static constexpr bool HI2 = BITS == 6;
+  static constexpr int PB = HI2 ? 4 : BITS;                       // bits per code in the stream plane
+  static constexpr int CB = DENSE ? 32 * PB : KEEP * PB;          // code bits per 32-column block
   static constexpr int CHB = 4 * CB;                              // per 128-column chunk
   static constexpr bool ALIGNED = CHB % 32 == 0;
   static constexpr int ND = (CHB + 31) / 32;                      // dwords of chunk code bits
   static constexpr bool VEC16 = CHB % 128 == 0;                   // chunks start on 16-byte units
   static constexpr int NL = VEC16 ? ND : 4 * ((CHB + 254) / 128); // dwords loaded: whole units covering any skew
   static constexpr int NIB = DENSE ? 32 : KEEP;                   // codes per block
-  static constexpr int SB = BITS == 3 ? 4 : BITS;                 // stream code width after expansion
+  static constexpr int SB = BITS == 3 ? 4 : PB;                   // stream code width after expansion
   static constexpr int NW = (NIB * SB + 31) / 32;                 // dwords of a block's code stream
   static constexpr int NGC = 128 / GRP;                           // groups per chunk (1 or 2)
   static constexpr int SEL_KIND = (BITS == 2) ? 1 : 0;

@@ -238,7 +238,7 @@ __device__ inline void fetch_selectors(uint32_t mw, const uint2* lut, uint32_t l
 // sel4: the selectors of the block's four mask bytes, read from the table by fetch_selectors.
 template <class C, int BITS>
 __device__ inline void decode_half(const uint32_t (&st)[C::NW], const uint32_t (&rk)[4], const uint2 (&sel4)[4],
-                                   uint32_t nz, int half, uint32_t (&bfrag)[4]) {
+                                   uint32_t nz, int half, uint32_t (&bfrag)[4], uint32_t hw = 0) {
 #pragma unroll
   for (int jj2 = 0; jj2 < 2; ++jj2) {
     const int jj = 2 * half + jj2;                       // mask byte inside the block
@@ -258,7 +258,12 @@ __device__ inline void decode_half(const uint32_t (&st)[C::NW], const uint32_t (
       uint32_t w;
       if (jj == 0) w = st[0];
       else w = window<C::NW>(st, rk[jj] * C::SB);
-      if (C::SB == 4) {
+      if (C::HI2) {
+        uint32_t h0, h1;
+        hi2_pools(hw, jj == 0 ? 0u : rk[jj], h0, h1);
+        p0 = bias_pool((w & 0x0F0F0F0Fu) | h0, nz);
+        p1 = bias_pool(((w >> 4) & 0x0F0F0F0Fu) | h1, nz);
+      } else if (C::SB == 4) {
         p0 = bias_pool(w & 0x0F0F0F0Fu, nz);
         p1 = bias_pool((w >> 4) & 0x0F0F0F0Fu, nz);
       } else {
@@ -281,6 +286,7 @@ struct Loads {
   uint32_t raw[C::NL];
   uint32_t zraw;
   uint32_t sc[C::NGC];        // fp16 bits of the scales of this lane's chunk
+  uint32_t h2[C::HI2 ? 4 : 1];   // BLK1632_6: the chunk's four dwords of high bits
 };
 
 template <int BITS, int KEEP, int GRP, int MP>
@@ -422,6 +428,10 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
           L.raw[4 * i] = v.x; L.raw[4 * i + 1] = v.y; L.raw[4 * i + 2] = v.z; L.raw[4 * i + 3] = v.w;
         }
       }
+      if (C::HI2) {                                                 // unit ch of the plane behind mask and nibbles
+        const uint4 v = *(const uint4*)(m_data + (so_t + ((3u * (uint32_t)NCH + (uint32_t)S4 + chl) << ush) + lane_off));
+        L.h2[0] = v.x; L.h2[1] = v.y; L.h2[2] = v.z; L.h2[3] = v.w;
+      }
       const uint32_t gv = so_g + ((uint32_t)(S4 * C::NGC) << csh) + __umul24(wrc, sz_mul) + ((chl * C::NGC) << csh);
       if (C::NGC == 1) {
         L.zraw = m_zero[gv];
@@ -555,7 +565,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
           for (int half = 0; half < 2; ++half) {
             const int t = 2 * jb + half;                            // fragment index in the chunk
             uint32_t bfrag[4];
-            decode_half<C, BITS>(st, rkc, selc, nz, half, bfrag);
+            decode_half<C, BITS>(st, rkc, selc, nz, half, bfrag, C::HI2 ? cur.h2[C::HI2 ? jb : 0] : 0u);
             const v4i bv = (v4i){(int)bfrag[0], (int)bfrag[1], (int)bfrag[2], (int)bfrag[3]};
 #pragma unroll
             for (int p = 0; p < MP; ++p) {
@@ -672,8 +682,9 @@ bool gemv_fast_takes(const DMat& m, int M) {
   const int fam = family_of(m.layout);
   if (fam == FAM_BLK) { if (!keep_supported(m.keep)) return false; }
   else if (fam == FAM_DENSE) { if (m.bits == 8) return false; }
+  else if (fam == FAM_BLK6) { if (m.bits != 6 || m.keep != 16 || m.group != 128) return false; }
   else return false;
-  if (m.bits != 2 && m.bits != 3 && m.bits != 4) return false;
+  if (m.bits != 2 && m.bits != 3 && m.bits != 4 && fam != FAM_BLK6) return false;
   // 32-bit offsets inside the kernel: every array of the matrix below 4 GB
   if ((uint64_t)((m.K + 15) / 16 * 16) * m.stride + 1024 >= (1ull << 32)) return false;
   if ((uint64_t)((m.K + 15) / 16 * 16) * m.G * 2 >= (1ull << 32)) return false;
@@ -800,6 +811,7 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
   const size_t lds = (size_t)LUT_BYTES + ZERO_BYTES + CNT_BYTES + xq_cap + (size_t)delta_cap * 4 +
                      (size_t)gb.h.red_floats * 4;
   const int bits = gb.mat[0].m.bits;
+  if (bits == 6) return launch_mp<6, 16, 128>(gb, lds, blocks, st);   // BLK1632_6: one configuration
   return bits == 2 ? launch_keep<2>(gb, lds, blocks, st) : bits == 3 ? launch_keep<3>(gb, lds, blocks, st)
        : bits == 4 ? launch_keep<4>(gb, lds, blocks, st) : CBK_ERR_UNSUPPORTED;
 }

@@ -207,8 +207,6 @@ def test_gemv_pruned_columns_contribute_exactly_zero(case, tiled):
                 yh = ops.gemv(pm, xh.expand(M, N).contiguous().to(DEV), out_dtype=torch.float32)
                 assert torch.equal(y0, ym), f"{case_id(case)} zero={zmode} {dtype} M={M}"
                 assert rel_fro(_np(yh)[0], ref[0]) < TOL, f"{case_id(case)} zero={zmode} {dtype} M={M}"
-                if layout == F.BLK1632_6:                      # float row kernel: exact in any case
-                    assert torch.equal(y0, yh)
         assert (_np(ops.dequant(pm))[:, ~pat.reshape(N)] == 0).all()
 
 
