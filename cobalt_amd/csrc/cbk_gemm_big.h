@@ -17,9 +17,9 @@
 //
 // Weight decode.  Each of the 256 threads owns one weight row of the tile and decodes its
 // 64 columns of the stage.  For 2/3/4-bit codes (bitmap layouts with 10, 16 or 23 of 32 kept,
-// and the dense layouts; zero points <= 128) this is the byte-permute decoder of the decode
-// kernel (selector table in LDS) followed by two packed-half operations per column pair; the
-// remaining layouts (6- and 8-bit codes, larger zero points) go through the generic
+// and the dense layouts) and for BLK1632_6, zero points <= 128, this is the byte-permute decoder
+// of the decode kernel (selector table in LDS) followed by two packed-half operations per column
+// pair; the remaining layouts (8-bit codes, larger zero points) go through the generic
 // 32-column reader.
 //
 // Workgroups are ordered so that those running at the same time on one XCD (blockIdx % 8)
@@ -248,6 +248,7 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
     uint32_t z;                          // zero points of the chunk's groups, one per byte
     float s[C::NGC];
     uint32_t ci;                         // chunk index the units were loaded for
+    uint32_t h2[C::HI2 ? 4 : 1];         // BLK1632_6: high bit pairs, one dword per block
   };
   WChunk wA, wB;
   uint32_t st[C::NW];                                             // code stream of the block being decoded
@@ -266,6 +267,10 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
     for (int i = 0; i < C::NL / 4; ++i) {
       const uint4 v = *(const uint4*)rv.unit(u0 + i);
       w.raw[4 * i] = v.x; w.raw[4 * i + 1] = v.y; w.raw[4 * i + 2] = v.z; w.raw[4 * i + 3] = v.w;
+    }
+    if (C::HI2) {                                                   // the plane behind mask and nibbles
+      const uint4 v = *(const uint4*)rv.unit(3u * (uint32_t)nch + (uint32_t)c);
+      w.h2[0] = v.x; w.h2[1] = v.y; w.h2[2] = v.z; w.h2[3] = v.w;
     }
     const size_t mi = meta0 + (size_t)c * C::NGC * meta_step;
     w.z = m.zero[mi];
@@ -326,7 +331,12 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
       const uint32_t mw = w.m[blk];
       const uint32_t r = jj == 0 ? 0u : (uint32_t)__builtin_popcount(mw & ((1u << (8 * jj)) - 1u));
       const uint32_t cwin = jj == 0 ? st[0] : window<C::NW>(st, r * C::SB);
-      if (C::SB == 4) {
+      if (C::HI2) {
+        uint32_t h0, h1;
+        hi2_pools(w.h2[C::HI2 ? blk : 0], r, h0, h1);
+        p0 = bias_pool((cwin & 0x0F0F0F0Fu) | h0, nz);
+        p1 = bias_pool(((cwin >> 4) & 0x0F0F0F0Fu) | h1, nz);
+      } else if (C::SB == 4) {
         p0 = bias_pool(cwin & 0x0F0F0F0Fu, nz);
         p1 = bias_pool((cwin >> 4) & 0x0F0F0F0Fu, nz);
       } else {

@@ -8,6 +8,7 @@ namespace cbk {
 int launch_gemm_big_b2(const GbArgs&, int keep, int group, int blocks, hipStream_t);
 int launch_gemm_big_b3(const GbArgs&, int keep, int group, int blocks, hipStream_t);
 int launch_gemm_big_b4(const GbArgs&, int keep, int group, int blocks, hipStream_t);
+int launch_gemm_big_b6(const GbArgs&, int blocks, hipStream_t);
 
 // ---- X' = fp16(x * col_scale), [Mpad, Npad] row-major; rows M..Mpad-1 and columns N..Npad-1 zero
 __global__ __launch_bounds__(256) void gemm_prep_kernel(const uint16_t* x, int64_t ldx, const uint16_t* cs, int xdt,
@@ -72,10 +73,19 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float* par
 // 32-token blocks per wavefront: calls of at most 64 activation rows take the 64-token tile
 static inline int gb_ti(int M) { return M <= 64 ? 1 : 4; }
 
-static int gb_nsplit(const DMat& m, int M) {
-  const bool le128 = (m.flags & CBK_FLAG_ZERO_LE_128) != 0;
+// the matrices the byte-permute instantiations take (the others go through the generic reader,
+// whose launches are never split)
+static bool gb_fast(const DMat& m) {
   const int fam = family_of(m.layout);
-  if (m.cs_rows > 1 || !le128 || !(fam == FAM_BLK || fam == FAM_DENSE) || m.bits < 2 || m.bits > 4) return 1;
+  if (!(m.flags & CBK_FLAG_ZERO_LE_128) || (m.group != 64 && m.group != 128)) return false;
+  if (fam == FAM_BLK6) return m.bits == 6 && m.keep == 16 && m.group == 128;
+  if (m.bits < 2 || m.bits > 4) return false;
+  if (fam == FAM_BLK) return m.keep == 10 || m.keep == 16 || m.keep == 23;
+  return fam == FAM_DENSE;
+}
+
+static int gb_nsplit(const DMat& m, int M) {
+  if (m.cs_rows > 1 || !gb_fast(m)) return 1;
   const int T = 64 * gb_ti(M);
   const int tiles = ((M + T - 1) / T) * ((m.K + GB_R - 1) / GB_R);
   const int nst = gb_npad(m.N) / GB_K;
@@ -146,6 +156,8 @@ int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, v
     if (m.bits == 2) rc = launch_gemm_big_b2(a, keep, m.group, blocks, st);
     else if (m.bits == 3) rc = launch_gemm_big_b3(a, keep, m.group, blocks, st);
     else if (m.bits == 4) rc = launch_gemm_big_b4(a, keep, m.group, blocks, st);
+  } else if (le128 && fam == FAM_BLK6 && m.bits == 6 && m.keep == 16 && m.group == 128) {
+    rc = launch_gemm_big_b6(a, blocks, st);
   }
   if (rc == CBK_ERR_UNSUPPORTED) {
     if (a.nsplit > 1) return CBK_ERR_UNSUPPORTED;                   // (gb_nsplit only splits what the cases above take)

@@ -1,7 +1,7 @@
 // Reference-shaped decode GEMV for EVERY layout: one wavefront per weight row, lanes stride
 // over 32-column blocks, float32 FMA, butterfly reduction.  It is the path for layouts and
 // parameter combinations the MFMA decode kernel does not take (variable-length SPARSE4*,
-// BLK1632_6, DENSE8, zero points above 127) and the yardstick the fast kernel is checked
+// DENSE8, zero points above 127) and the yardstick the fast kernel is checked
 // against.  Computes, per row k and activation row m,
 //     y[m,k] = sum_g scale[k,g] * sum_{j in g, kept} (q[k,j] - zero[k,g]) * (x[m,j]*cs[j])
 // which is the accumulation order of cbk::gemv_rows in the reference
