@@ -213,7 +213,8 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    layout = F.BLK1632_4 if (a.bits, a.keep, a.group) == (4, 16, 128) else F.BLKC
+    layout = F.BLK1632_4 if (a.bits, a.keep, a.group) == (4, 16, 128) else \
+        F.BLK1632_6 if (a.bits, a.keep, a.group) == (6, 16, 128) else F.BLKC
     dt = torch.float16 if a.dtype == "f16" else torch.bfloat16
     shapes = SHAPES[a.workload]
     M = a.m
