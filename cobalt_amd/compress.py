@@ -152,4 +152,6 @@ def layout_for(sparsity: float, bits: int, group: int, mask_block: int) -> Tuple
     keep = 32 - int(32 * sparsity)
     if (bits, group, keep) == (4, 128, 16):
         return F.BLK1632_4, 16
+    if (bits, group, keep) == (6, 128, 16):
+        return F.BLK1632_6, 16
     return F.BLKC, keep

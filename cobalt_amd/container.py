@@ -255,7 +255,7 @@ def raw_layout(raw: Dict[str, torch.Tensor], bits: Optional[int] = None) -> Tupl
     group = N // raw["scale"].shape[1]
     if bits is None:
         top = int(raw["q"].max())
-        bits = 2 if top < 4 else 3 if top < 8 else 4 if top < 16 else 8
+        bits = 2 if top < 4 else 3 if top < 8 else 4 if top < 16 else 6 if top < 64 else 8
     keep_map = F.unpack_mask(raw["mask"], N)
     if bool(keep_map.all()):
         return (F.DENSE4 if (bits, group) == (4, 128) else F.DENSE8 if (bits, group) == (8, 128) else F.DENSEB), bits, group, None
@@ -264,6 +264,8 @@ def raw_layout(raw: Dict[str, torch.Tensor], bits: Optional[int] = None) -> Tupl
     if bool((cnt == k0).all()):
         if (bits, group, k0) == (4, 128, 16):
             return F.BLK1632_4, 4, 128, 16
+        if (bits, group, k0) == (6, 128, 16):
+            return F.BLK1632_6, 6, 128, 16
         return F.BLKC, bits, group, k0
     raise ValueError("a mask without a fixed number of survivors per 32 columns packs to the variable-length "
                      "layouts, which this package reads but does not produce")

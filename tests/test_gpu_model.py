@@ -43,6 +43,21 @@ def test_hf_decoder_is_compressed_in_place_and_matches_its_dense_twin():
         assert err < 5e-3, (shape, err)                             # fp16 activations through two blocks
 
 
+def test_six_bit_and_three_bit_overrides_match_the_dense_twin():
+    from cobalt_amd import format as F, model as Mo
+    m = _tiny_mistral()
+    g = torch.Generator().manual_seed(5)
+    calib = torch.randint(0, 512, (4, 32), generator=g).to(DEV)
+    rep = Mo.compress_model(m, calib, bits_override={"mlp.down_proj": 6, "self_attn.o_proj": 3})
+    assert rep["model.layers.0.mlp.down_proj"]["layout"] == F.BLK1632_6
+    twin = Mo.dense_twin(copy.deepcopy(m), torch.float16)
+    for shape in ((1, 300), (1, 40), (2, 1)):
+        ids = torch.randint(0, 512, shape, generator=g).to(DEV)
+        with torch.no_grad():
+            a, b = m(ids).logits.float(), twin(ids).logits.float()
+        assert float((a - b).norm() / b.norm()) < 5e-3, shape
+
+
 def test_compressed_model_state_dict_round_trip():
     from cobalt_amd import model as Mo
     m = _tiny_mistral()

@@ -207,3 +207,18 @@ def test_state_dict_of_a_compressed_model_loads_into_a_dense_one():
         Mo.load_compressed_state_dict(_Toy(layers=2), bad)
     with pytest.raises(KeyError):
         Mo.load_compressed_state_dict(_Toy(layers=1), sd)
+
+
+def test_six_bit_override_lands_in_the_reference_layout():
+    """bits 6 at 16 of 32 kept and group 128 is BLK1632_6 (4.1875 bits per weight,
+    docs/FORMAT.md:78-81), not the generic bit-stream layout; the RAW artifact finds it again."""
+    from cobalt_amd import container as Ct
+    torch.manual_seed(0)
+    m = _Toy(layers=1)
+    rep = Mo.compress_model(m, torch.randint(0, 64, (2, 16)), bits_override={"mlp.down_proj": 6})
+    r = rep["layers.0.mlp.down_proj"]
+    assert r["layout"] == F.BLK1632_6 and r["bits"] == 6 and abs(r["bpw"] - 4.1875) < 1e-9
+    pm = m.layers[0].mlp.down_proj.packed()
+    raw = dict(mask=pm.array("data")[: pm.K * (pm.N // 2)].view(pm.K, pm.N // 2)[:, : pm.N // 8].contiguous(),
+               q=torch.full((pm.K, pm.N), 63, dtype=torch.uint8), scale=torch.ones(pm.K, pm.N // 128).half())
+    assert Ct.raw_layout(raw) == (F.BLK1632_6, 6, 128, 16)
