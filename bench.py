@@ -51,7 +51,7 @@ MFMA_PEAK_TFLOPS = 2500.0          # dense bf16 / f16 MFMA peak of MI355X
 # HBM bytes per launch of the decode kernel (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, scaled by
 # the same counters read for a device-to-device copy of known size), keyed by
 # (workload, launch grouping, M); filled from the runs summarised under profiles/.
-MEASURED_TRAFFIC = {("mistral7b", "phase", 1): 22312635}
+MEASURED_TRAFFIC = {("mistral7b", "phase", 1): 22311131}
 
 
 def algorithmic_bytes(pm, M, e_x=2, e_y=2):
