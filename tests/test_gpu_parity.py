@@ -241,7 +241,8 @@ def test_linear_ragged_and_extreme_shapes(case):
 
 
 # ------------------------------------------------------------------ row-fused matrices
-FUSED_CASES = [(F.BLK1632_4, 4, 128, 16), (F.BLKC, 3, 128, 10), (F.BLKC, 2, 64, 23), (F.DENSE4, 4, 128, 0)]
+FUSED_CASES = [(F.BLK1632_4, 4, 128, 16), (F.BLKC, 3, 128, 10), (F.BLKC, 2, 64, 23), (F.DENSE4, 4, 128, 0),
+               (F.BLK1632_6, 6, 128, 16)]
 
 
 def _fused(case, K, N, cs_rows, splits, seed, tiled):
@@ -300,7 +301,7 @@ def test_gemv_fused_rows_equal_their_unfused_parts_bit_for_bit():
     assert torch.equal(y2[:, 0::2], whole[0][:, 0::2]) and torch.equal(y2[:, 1::2], whole[1][:, 1::2])
 
 
-@pytest.mark.parametrize("case", FUSED_CASES[:2], ids=case_id)
+@pytest.mark.parametrize("case", FUSED_CASES[:2] + FUSED_CASES[4:], ids=case_id)
 def test_gemm_fused_col_scale_rows(case):
     """Prefill on fused matrices: q|k|v ranges run the 256 x 256 kernel range by range, gate/up
     (row parity) as workgroups of one parity; ranges off the 16-row grid the 128 x 128 kernel."""
