@@ -24,6 +24,10 @@ the 2.5 PFLOP/s dense bf16/f16 MFMA peak.
 decode workload's MLP shapes; `measured_ceilings` are this GPU's dense f16 MFMA rate and plain
 read rate from two probe kernels.
 
+`lm_head_gemv` is the decode kernel on one large matrix, the model's output projection
+(vocabulary x hidden, dense 4-bit): what the kernel streams when a launch is long enough for
+its fixed costs not to matter.
+
 `cpu_baseline` is the C oracle (dequantise-then-matmul, OpenMP over rows) timed on the host
 cores on the SAME packed bytes as the first layer set, and doubles as a last parity check of
 the GPU outputs.
@@ -138,12 +142,47 @@ def measured_ceilings(torch, dev):
     buf = torch.empty(2**30, dtype=torch.uint8, device=dev)
     buf.random_(0, 256)
     sink4 = torch.zeros(1, dtype=torch.int32, device=dev)
-    ms = timed(lambda: L.cbk_bench_read(buf.data_ptr(), buf.numel(), 16 * cus, sink4.data_ptr(), st.cuda_stream), 10)
-    read = buf.numel() / ms / 1e6
+    read = 0.0
+    for per_cu in (8, 16, 32):                                    # the best of three grid sizes
+        ms = timed(lambda: L.cbk_bench_read(buf.data_ptr(), buf.numel(), per_cu * cus, sink4.data_ptr(), st.cuda_stream), 10)
+        read = max(read, buf.numel() / ms / 1e6)
     del buf, sink, sink4
     return {"mfma_f16_dense_tflops": round(mfma, 1), "hbm_read_gbs": round(read, 1),
             "how": "libcbk_bench.so: 16 independent v_mfma_f32_32x32x16_f16 per wavefront, one wavefront per SIMD; "
-                   "grid-stride 16-byte reads of 1 GiB"}
+                   "grid-stride 16-byte reads of 1 GiB, eight in flight per lane, best of three grid sizes"}
+
+
+VOCAB = {"mistral7b": 32000, "gemma27b": 262144}
+
+
+def lm_head_gemv(torch, F, ops, dev, workload, M, dt, reps=20):
+    """Decode kernel on the output projection of the model the workload is shaped after: dense
+    4-bit codes (DENSE4, the reference packer's default for the tied embedding,
+    src/cobaltkernel/pack_cobalt.py:561-563), vocabulary x hidden, one launch."""
+    N = SHAPES[workload][0][2]
+    K = VOCAB[workload]
+    pm = F.synth_packed(K, N, F.DENSE4, seed=3, device=dev).to_tiled()
+    # successive calls rotate over as many copies of the matrix as exceed twice the 256 MB Infinity Cache
+    copies = [pm]
+    while len(copies) * pm.stream_bytes() < 2 * 256 * 2**20:
+        copies.append(F.synth_packed(K, N, F.DENSE4, seed=3 + len(copies), device=dev).to_tiled())
+    x = torch.randn(M, N, device=dev, generator=torch.Generator(device=dev).manual_seed(1)).to(dt)
+    for i in range(2 * len(copies)):
+        y = ops.gemv(copies[i % len(copies)], x)
+    st = torch.cuda.current_stream()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    reps = -(-reps // len(copies)) * len(copies)
+    e0.record(st)
+    for i in range(reps):
+        y = ops.gemv(copies[i % len(copies)], x)
+    e1.record(st)
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / reps
+    nbytes = algorithmic_bytes(pm, M)
+    out = {"matrix": f"{K}x{N} DENSE4 ({pm.bpw():.4f} bpw), M={M}", "distinct_copies": len(copies), "ms": round(ms, 4), "bytes": nbytes,
+           "gbs": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    del pm, copies, x, y
+    return out
 
 
 def prefill_gemm(torch, F, ops, dev, workload, layout, bits, group, keep, M, dt, reps=20, warm=10):
@@ -196,6 +235,7 @@ def main():
     ap.add_argument("--group", type=int, default=128)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-core baseline")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM measurement")
+    ap.add_argument("--no-lm-head", action="store_true", help="skip the output-projection GEMV measurement")
     ap.add_argument("--prefill-workload", default="gemma27b", choices=list(SHAPES))
     ap.add_argument("--prefill-m", type=int, default=2048)
     ap.add_argument("--prefill-dtype", default="bf16", choices=["f16", "bf16"])
@@ -364,6 +404,8 @@ def main():
         mid = prefill_gemm(torch, F, ops, dev, a.workload, layout, a.bits, a.group, a.keep, 64,
                            torch.float16 if a.dtype == "f16" else torch.bfloat16)
         out["gemm_m64"] = {"workload": mid["workload"], "tflops": mid["tflops"], "per_matrix": mid["per_matrix"]}
+    if not a.no_lm_head:
+        out["lm_head_gemv"] = lm_head_gemv(torch, F, ops, dev, a.workload, M, dt)
     ceil = measured_ceilings(torch, dev)
     if ceil:
         out["measured_ceilings"] = ceil

@@ -31,14 +31,17 @@ __global__ __launch_bounds__(256) void bench_mfma_kernel(float* sink, int iters)
   sink[(size_t)blockIdx.x * 256 + threadIdx.x] = s;
 }
 
-// Grid-stride read of 16 bytes per lane, four loads in flight per lane; the xor keeps the loads.
+// Grid-stride read of 16 bytes per lane, eight loads in flight per lane; the xor keeps the loads.
 __global__ __launch_bounds__(256) void bench_read_kernel(const uint4* __restrict__ p, size_t n16, uint32_t* sink) {
   const size_t stride = (size_t)gridDim.x * 256;
   size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   uint32_t x = 0;
-  for (; i + 3 * stride < n16; i += 4 * stride) {
-    const uint4 a = p[i], b = p[i + stride], c = p[i + 2 * stride], d = p[i + 3 * stride];
-    x ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+  for (; i + 7 * stride < n16; i += 8 * stride) {
+    uint4 v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = p[i + k * stride];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) x ^= v[k].x ^ v[k].y ^ v[k].z ^ v[k].w;
   }
   for (; i < n16; i += stride) {
     const uint4 a = p[i];
