@@ -1,5 +1,6 @@
 // Reference-shaped decode GEMV for EVERY layout: one wavefront per weight row, lanes stride
-// over 32-column blocks, float32 FMA, butterfly reduction.  It is the path for layouts and
+// over 32-column blocks (fixed-stride layouts through the generic reader; the survivor streams
+// with vector loads and a register nibble stream), float32 FMA, butterfly reduction.  It is the path for layouts and
 // parameter combinations the MFMA decode kernel does not take (variable-length SPARSE4*,
 // DENSE8, zero points above 127) and the yardstick the fast kernel is checked
 // against.  Computes, per row k and activation row m,
@@ -17,9 +18,12 @@ __device__ inline float wave_sum(float v) {
   return v;
 }
 
+constexpr int SP4_MAX_G = 512;     // groups per row whose offsets the SPARSE4 path keeps in LDS (N <= 65536)
+
 template <int XDT, int M>
 __global__ __launch_bounds__(256) void gemv_generic_kernel(DMat m, const void* x, int64_t ldx, void* y,
                                                            int ydt, int64_t ldy, const void* bias) {
+  __shared__ uint32_t sp4_goff[4 * SP4_MAX_G];
   const int lane = threadIdx.x & 63;
   const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
   const int nwaves = (gridDim.x * blockDim.x) >> 6;
@@ -52,11 +56,105 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(DMat m, const void* x
 #pragma unroll
         for (int i = 0; i < M; ++i) acc[i] = fmaf(s, part[i], acc[i]);
       }
-    } else {
+    } else if (m.layout != CBK_SPARSE4 || m.G <= SP4_MAX_G) {
+      // The byte offset of every group's codes is in the row's header (SPARSE4X / SPARSE4E) or
+      // is summed up here from the bitmap (SPARSE4: a prefix sum of the groups' byte counts over
+      // the wavefront, kept in LDS), so a lane can take one 32-column block: its survivors'
+      // nibbles start popc(earlier blocks of the group) nibbles into the group.  Activations, column scales and the (at most 17) code
+      // bytes are fetched up front as whole vectors; the nibbles are then shifted out of a
+      // register stream under the mask bits, one mask byte at a time.
       const uint8_t* row = m.data + m.row_off[k];
       const uint32_t* bm = (const uint32_t*)row;
       const bool has_goff = m.layout != CBK_SPARSE4;
       const int hdr = ((m.N >> 3) + (has_goff ? ((m.G * 2 + 15) & ~15) : 0) + 15) & ~15;
+      const uint16_t* goff = (const uint16_t*)(row + (m.N >> 3));
+      uint32_t* lgoff = sp4_goff + (threadIdx.x >> 6) * SP4_MAX_G;
+      if (!has_goff) {
+        uint32_t carry = 0;
+        for (int g0 = 0; g0 < m.G; g0 += 64) {
+          const int g = g0 + lane;
+          uint32_t nb = 0;                                          // bytes of group g: an even number of nibbles
+          if (g < m.G) nb = (uint32_t)(__popc(bm[4 * g]) + __popc(bm[4 * g + 1]) + __popc(bm[4 * g + 2]) + __popc(bm[4 * g + 3]) + 1) >> 1;
+          uint32_t incl = nb;
+#pragma unroll
+          for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t v = (uint32_t)__shfl_up((int)incl, o, 64);
+            incl += lane >= o ? v : 0u;
+          }
+          if (g < m.G) lgoff[g] = carry + incl - nb;
+          carry += (uint32_t)__shfl((int)incl, 63, 64);
+        }
+        __builtin_amdgcn_wave_barrier();
+      }
+      for (int t = lane; t < m.N / BLOCK; t += 64) {
+        const int g = t >> 2, j = t & 3;
+        const uint32_t mw = bm[t];
+        uint32_t pre = 0;                                           // nibbles of the group before this block
+        if (j > 0) pre += __popc(bm[4 * g]);
+        if (j > 1) pre += __popc(bm[4 * g + 1]);
+        if (j > 2) pre += __popc(bm[4 * g + 2]);
+        const uint8_t* cp = row + hdr + (has_goff ? (uint32_t)goff[g] : lgoff[g]) + (pre >> 1);
+        const uintptr_t ca = (uintptr_t)cp & ~(uintptr_t)3;
+        const uint32_t sh = (uint32_t)(((uintptr_t)cp & 3) * 8 + (pre & 1) * 4);   // < 32
+        uint32_t e[6];
+#pragma unroll
+        for (int i = 0; i < 6; ++i) e[i] = ((const uint32_t*)ca)[i];               // 17 bytes + skew; rows end in a readable tail
+        uint32_t w[5];
+#pragma unroll
+        for (int i = 0; i < 5; ++i) w[i] = __builtin_amdgcn_alignbit(e[i + 1], e[i], sh);
+        const float s = h2f(m.scale[(size_t)k * m.G + g]);
+        const float z = (float)m.zero[(size_t)k * m.G + g];
+        float part[M];
+#pragma unroll
+        for (int i = 0; i < M; ++i) part[i] = 0.f;
+#pragma unroll
+        for (int jb = 0; jb < 4; ++jb) {
+          const uint32_t mb = (mw >> (8 * jb)) & 0xFFu;
+          const uint32_t r = jb == 0 ? 0u : (uint32_t)__popc(mw & ((1u << (8 * jb)) - 1u));     // survivors before this byte
+          // 32 bits of the stream from nibble r on: dword r / 8 and the next one, picked by selects
+          const uint32_t idx = r >> 3, bs = (r & 7u) * 4u;
+          uint32_t lo = w[0], hi = w[1];
+#pragma unroll
+          for (int i = 1; i < 4; ++i) { lo = idx == (uint32_t)i ? w[i] : lo; hi = idx == (uint32_t)i ? w[i + 1] : hi; }
+          lo = idx >= 4u ? w[4] : lo; hi = idx >= 4u ? 0u : hi;
+          uint32_t win = __builtin_amdgcn_alignbit(hi, lo, bs);
+          const int c0 = t * BLOCK + 8 * jb;
+          float cf[8];
+          if (cs) {
+            const uint4 cv = *(const uint4*)(cs + c0);
+            const uint32_t cw[4] = {cv.x, cv.y, cv.z, cv.w};
+#pragma unroll
+            for (int p = 0; p < 8; ++p) cf[p] = h2f((uint16_t)(cw[p >> 1] >> (16 * (p & 1))));
+          } else {
+#pragma unroll
+            for (int p = 0; p < 8; ++p) cf[p] = 1.f;
+          }
+          float wv[8];
+#pragma unroll
+          for (int p = 0; p < 8; ++p) {
+            const bool kp = (mb >> p) & 1u;
+            wv[p] = kp ? ((float)(win & 0xFu) - z) * cf[p] : 0.f;
+            win = kp ? win >> 4 : win;
+          }
+#pragma unroll
+          for (int i = 0; i < M; ++i) {
+            const uint4 xv = *(const uint4*)((const uint16_t*)x + (size_t)i * ldx + c0);
+            const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+            for (int p = 0; p < 8; ++p) {
+              const uint16_t hb = (uint16_t)(xw[p >> 1] >> (16 * (p & 1)));
+              part[i] = fmaf(wv[p], XDT == CBK_F16 ? h2f(hb) : bf2f(hb), part[i]);
+            }
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < M; ++i) acc[i] = fmaf(s, part[i], acc[i]);
+      }
+    } else {
+      const uint8_t* row = m.data + m.row_off[k];
+      const uint32_t* bm = (const uint32_t*)row;
+      const bool has_goff = false;
+      const int hdr = ((m.N >> 3) + 15) & ~15;
       for (int g = lane; g < m.G; g += 64) {
         uint32_t off = 0;
         if (has_goff) off = ((const uint16_t*)(row + (m.N >> 3)))[g];

@@ -101,6 +101,21 @@ def test_gemv_matches_oracle(case, dtype, tiled):
             assert np.abs(_np(y) - ref).max() / np.abs(ref).max() < 1e-4
 
 
+@pytest.mark.parametrize("case", SPARSE_CASES, ids=case_id)
+def test_gemv_sparse_streams_on_long_rows(case):
+    """Variable-length layouts with more than 64 groups per row (N = 14336: 112 groups), where the
+    row kernel sums the SPARSE4 group offsets over the wavefront in more than one round."""
+    K, N = 24, 14336
+    raw = make_raw(case, K, N, seed=3 + case[0])
+    pk = oracle_pack(case, raw)
+    pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV)
+    W = R.dequant(pk, K, N, case[0], col_scale=raw["col_scale"], **kw_of(case))
+    for M in (1, 3, 6):
+        x = acts(M, N, torch.float16, seed=M)
+        y = ops.gemv(pm, x.to(DEV), out_dtype=torch.float32)
+        assert rel_fro(_np(y), R.forward_ref(W, _np(x))) < 1e-5, (case_id(case), M)
+
+
 ALL_MFMA_CASES = [(F.BLKC, b, g, k) for b in (2, 3, 4) for g in (64, 128) for k in (10, 16, 23)] + \
                  [(F.DENSEB, b, g, 0) for b in (2, 3, 4) for g in (64, 128)]
 
