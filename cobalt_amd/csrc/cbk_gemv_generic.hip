@@ -33,7 +33,46 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(DMat m, const void* x
 #pragma unroll
     for (int i = 0; i < M; ++i) acc[i] = 0.f;
     const uint16_t* cs = m.cs ? m.cs + (size_t)cs_row_of(m, k) * m.N : nullptr;
-    if (fam != FAM_SPARSE) {
+    if (m.layout == CBK_DENSE8) {
+      // one byte per column: a lane takes a 32-column block as two 16-byte units of codes and
+      // whole vectors of activations and column scales
+      const RowView row = row_view(m, k);
+      for (int t = lane; t < m.N / BLOCK; t += 64) {
+        const uint4 c0 = *(const uint4*)row.unit(2 * t), c1 = *(const uint4*)row.unit(2 * t + 1);
+        const uint32_t cw[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+        const int g = (t * BLOCK) / m.group;
+        const float s = h2f(m.scale[meta_index(m, k, g)]);
+        const float z = (float)m.zero[meta_index(m, k, g)];
+        float part[M];
+#pragma unroll
+        for (int i = 0; i < M; ++i) part[i] = 0.f;
+#pragma unroll
+        for (int o = 0; o < 4; ++o) {                               // eight columns at a time
+          const int col = t * BLOCK + 8 * o;
+          float wv[8];
+#pragma unroll
+          for (int p = 0; p < 8; ++p) wv[p] = (float)((cw[2 * o + (p >> 2)] >> (8 * (p & 3))) & 0xFFu) - z;
+          if (cs) {
+            const uint4 cv = *(const uint4*)(cs + col);
+            const uint32_t sw[4] = {cv.x, cv.y, cv.z, cv.w};
+#pragma unroll
+            for (int p = 0; p < 8; ++p) wv[p] *= h2f((uint16_t)(sw[p >> 1] >> (16 * (p & 1))));
+          }
+#pragma unroll
+          for (int i = 0; i < M; ++i) {
+            const uint4 xv = *(const uint4*)((const uint16_t*)x + (size_t)i * ldx + col);
+            const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+            for (int p = 0; p < 8; ++p) {
+              const uint16_t hb = (uint16_t)(xw[p >> 1] >> (16 * (p & 1)));
+              part[i] = fmaf(wv[p], XDT == CBK_F16 ? h2f(hb) : bf2f(hb), part[i]);
+            }
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < M; ++i) acc[i] = fmaf(s, part[i], acc[i]);
+      }
+    } else if (fam != FAM_SPARSE) {
       const RowView row = row_view(m, k);
       for (int t = lane; t < m.N / BLOCK; t += 64) {
         int q[32];
