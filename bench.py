@@ -1,42 +1,48 @@
 """Headline benchmark of the CBK1 sparse low-bit linear layer on one MI355X.
 
 Decode (the `value` of the JSON line).  One "step" is one pass of the hot path over one
-decoder-layer set: the seven M-row GEMVs of a layer (q, k, v, o, gate, up, down) at sparsity
-0.5, 4-bit codes, group 128 (layout BLK1632_4, 3.1875 bits per weight), launched as the four
-dependency phases of a decoder layer (q,k,v | o | gate,up | down), one batched kernel launch
-per phase, replayed from HIP graphs: one graph holds about 32 steps in a row, as a decoder
-replays all its layers for a token in one graph (a replay boundary costs several microseconds
-on the GPU; single-step graphs serve the remainder, so that exactly K steps are timed).  The
-packed weights of several distinct layer sets are resident in HBM before the timed region;
-successive steps rotate through them so that the streamed set exceeds twice the 256 MB
-Infinity Cache.  `value` is algorithmic bytes (packed
-rows + scales + zeros + col_scale + activations in + outputs out) streamed per second.
+decoder-layer set: the seven M-row GEMVs of a layer (q, k, v, o, gate, up, down), launched as the
+four dependency phases of a decoder layer (q,k,v | o | gate,up | down), one batched kernel launch
+per phase.  The headline workload is the Gemma-3-27B-shaped layer set at sparsity 0.5, 4-bit
+codes, group 128 (layout BLK1632_4, 3.1875 bits per weight), bf16 activations, M=1; the
+Mistral-7B-shaped set (f16) is reported beside it as `decode_mistral7b`.  The packed weights of
+several distinct layer sets are resident in HBM before the timed region and successive steps
+rotate through them, so that the streamed set exceeds twice the 256 MB Infinity Cache.
 
-`roofline` describes the decode kernel: algorithmic bytes per launch over the average launch
-duration, which is the timed region (HIP events recorded on the launch stream) divided by
-the number of launches in it; the gaps between launches are therefore counted as kernel time.
+Launches are replayed from HIP graphs of many steps in a row, as a decoder replays all its layers
+for a token in one graph (a replay boundary costs the GPU several microseconds).  `--steps K` is
+honoured exactly and inside such graphs: K // P replays of a graph of P steps (whole rotations over
+the distinct layer sets, about 32 steps) plus one replay of a graph holding the K % P steps that
+remain.  Warm-up is `--warmup` steps, and never less than 50 ms of replays (the first launches
+of a process run at a lower clock), both graphs included.  The JSON says what was replayed.
 
-`prefill_gemm` reports the prefill kernel at the Gemma-3-27B MLP shapes (M=2048, bf16 by
-default; --prefill-workload / --prefill-m / --prefill-dtype choose others) in TFLOP/s against
-the 2.5 PFLOP/s dense bf16/f16 MFMA peak.
+`value` is algorithmic bytes (packed rows + scales + zeros + col_scale + activations in + outputs
+out) streamed per second.  `roofline` describes the decode kernel: algorithmic bytes per launch
+over the average launch duration, which is the timed region (HIP events recorded on the launch
+stream) divided by the number of launches in it; the gaps between launches are therefore counted
+as kernel time.  `per_matrix` times each distinct matrix of the set on its own (one launch per
+matrix, distinct copies of at least 512 MB in rotation): the kernel's rate without the other
+phases of the step.
 
-`gemm_m64` is the same kernel's 64-token tile at 64 activation rows (batched decoding) on the
-decode workload's MLP shapes; `measured_ceilings` are this GPU's dense f16 MFMA rate and plain
-read rate from two probe kernels.
+`prefill_gemm` reports the prefill kernel at the Gemma-3-27B MLP shapes (M=2048, bf16 by default)
+in TFLOP/s against the 2.5 PFLOP/s dense bf16/f16 MFMA peak, and checks sampled output rows of
+the timed configuration against a float64 matmul with the bit-exact dequantised weights.
 
-`lm_head_gemv` is the decode kernel on one large matrix, the model's output projection
-(vocabulary x hidden, dense 4-bit): what the kernel streams when a launch is long enough for
-its fixed costs not to matter.
+`--grid` runs the nine-cell sweep instead (Gemma-3-27B shapes x 62 layers, sparsity 0.3/0.5/0.7
+as 23/16/10 survivors per 32 columns, 2/3/4-bit codes, group 64): per-token linear time of a
+decode step (M=1) and of a 4096-token prefill, and bits per weight, per cell.
 
-`cpu_baseline` is the C oracle (dequantise-then-matmul, OpenMP over rows) timed on the host
-cores on the SAME packed bytes as the first layer set, and doubles as a last parity check of
-the GPU outputs.
+`cpu_baseline` is the torch restatement of the reference's CPU forward (dequantise the packed
+bytes to float32, then matmul: oracle/torch_ref.py) on the host cores, on the same packed bytes
+as the first layer set; the C oracle checks the GPU outputs of that set.
 
-python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mistral7b|gemma27b] [--m M]
+python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemma27b|mistral7b] [--m M] [--grid]
 """
 import argparse
+import ctypes
 import json
 import os
+import platform
 import sys
 import time
 
@@ -49,12 +55,18 @@ SHAPES = {
     "gemma27b": [("q", 4096, 5376), ("k", 2048, 5376), ("v", 2048, 5376), ("o", 5376, 4096),
                  ("gate", 21504, 5376), ("up", 21504, 5376), ("down", 5376, 21504)],
 }
+WORKLOAD_DTYPE = {"mistral7b": "f16", "gemma27b": "bf16"}          # the activation types the configurations name
+VOCAB = {"mistral7b": 32000, "gemma27b": 262144}
+GEMMA_LAYERS = 62
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = 2500.0          # dense bf16 / f16 MFMA peak of MI355X
+INFINITY_CACHE = 256 * 2**20
+MIN_WARM_MS = 50.0
 
 # HBM bytes per launch of the decode kernel (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, scaled by
 # the same counters read for a device-to-device copy of known size), keyed by
-# (workload, launch grouping, M); filled from the runs summarised under profiles/.
+# (workload, launch grouping, M).  Stored figures from the runs summarised under profiles/, not
+# counters read during a bench run.
 MEASURED_TRAFFIC = {("mistral7b", "phase", 1): 22311131}
 
 
@@ -63,56 +75,303 @@ def algorithmic_bytes(pm, M, e_x=2, e_y=2):
     return pm.stream_bytes() + pm.cs_rows * pm.N * 2 + M * pm.N * e_x + M * pm.K * e_y
 
 
-def cpu_baseline(pms, shapes, xs, ys, M, budget_s=20.0):
-    """C oracle forward over the layer set on the host cores, on the bytes the GPU used."""
-    import numpy as np
-    from oracle import cbk_ref_c as C
-    nthreads = min(16, os.cpu_count() or 1)
-    C.set_threads(nthreads)
-    total_bytes, total_t, worst, done, calls = 0, 0.0, 0.0, [], []
-    t_stop = time.time() + budget_s
-    for pm, (name, K, N) in zip(pms, shapes):
-        if done and time.time() > t_stop:
-            break
-        pk = dict(data=pm.array("data").cpu().numpy(), scale=pm.array("scale").cpu().numpy().reshape(K, -1),
-                  zero=pm.array("zero").cpu().numpy().reshape(K, -1))
-        cs = pm.array("col_scale").cpu().numpy().reshape(pm.cs_rows, N) if pm.cs_rows else None
-        x = xs[N].float().cpu().numpy()
-        call = lambda pk=pk, K=K, N=N, pm=pm, x=x, cs=cs: C.forward(
-            pk, K, N, pm.layout, x, col_scale=cs, bits=pm.bits, group=pm.group, keep_per_block=pm.keep or None)
-        t0 = time.perf_counter()
-        y = call()
-        total_t += time.perf_counter() - t0
-        total_bytes += algorithmic_bytes(pm, M)
-        got = ys[name].float().cpu().numpy()
-        worst = max(worst, float(np.linalg.norm(got - y) / np.linalg.norm(y)))
-        done.append(name)
-        calls.append((call, algorithmic_bytes(pm, M)))
-    # further passes over the same matrices until about one second of wall time on all threads
-    # (10-30 s of CPU work); the first, checked pass counts too
-    passes = 1
-    more = max(0, min(40, int(1.0 / max(total_t, 1e-3))))
-    for _ in range(more):
-        if time.time() > t_stop:
-            break
-        for call, nbytes in calls:
-            t0 = time.perf_counter()
-            call()
-            total_t += time.perf_counter() - t0
-            total_bytes += nbytes
-        passes += 1
-    return dict(value=round(total_bytes / total_t / 1e9, 3), unit="GB/s", cores=nthreads, kind="port",
-                sample=f"C oracle dequantise-then-matmul (OpenMP, {nthreads} threads) over {'+'.join(done)} of the first "
-                       f"layer set, {passes} passes, {total_t:.2f} s wall = {total_t * nthreads:.0f} core-seconds; "
-                       f"same packed bytes as the GPU run",
-                gpu_vs_oracle_rel_fro=worst)
+def layout_of(F, bits, keep, group):
+    return F.BLK1632_4 if (bits, keep, group) == (4, 16, 128) else \
+        F.BLK1632_6 if (bits, keep, group) == (6, 16, 128) else F.BLKC
 
 
+def torch_dtype(torch, name):
+    return torch.float16 if name == "f16" else torch.bfloat16
+
+
+# ------------------------------------------------------------------ decode: layer-set step
+def make_sets(torch, F, dev, shapes, layout, bits, group, keep, min_bytes, keep_first_rowmajor=False):
+    """Distinct layer sets (device order) whose packed bytes add up to at least `min_bytes`."""
+    set_bytes = sum(K * F.row_stride(layout, N, bits, group, keep) + K * (N // group) * 3 for _, K, N in shapes)
+    n_copies = max(2, -(-min_bytes // set_bytes))
+    sets, first = [], None
+    for c in range(n_copies):
+        rm = [F.synth_packed(K, N, layout, bits, group, keep, seed=1000 * c + i, device=dev)
+              for i, (_, K, N) in enumerate(shapes)]
+        if c == 0 and keep_first_rowmajor:
+            first = [p.to("cpu") for p in rm]
+        sets.append([p.to_tiled() for p in rm])
+        del rm
+    return sets, first
+
+
+class GraphTimer:
+    """Replays `step(i)` (i = running step index) from HIP graphs and times exactly K steps."""
+
+    def __init__(self, torch, stream, step, rotation, use_graph=True, target_steps=32):
+        self.torch, self.stream, self.step, self.use_graph = torch, stream, step, use_graph
+        self.per_graph = -(-target_steps // rotation) * rotation       # whole rotations over the distinct sets
+        self.g_all = None
+        self._rem = {}
+        if use_graph:
+            self.g_all = self._capture(self.per_graph)
+
+    def _capture(self, n):
+        g = self.torch.cuda.CUDAGraph()
+        with self.torch.cuda.graph(g, stream=self.stream):
+            for i in range(n):
+                self.step(i)
+        return g
+
+    def _run(self, full, rem):
+        if not self.use_graph:
+            for i in range(full * self.per_graph + rem):
+                self.step(i)
+            return
+        for _ in range(full):
+            self.g_all.replay()
+        if rem:
+            self._rem[rem].replay()
+
+    def measure(self, steps, warmup):
+        torch, stream = self.torch, self.stream
+        full, rem = divmod(steps, self.per_graph)
+        if self.use_graph and rem and rem not in self._rem:
+            self._rem[rem] = self._capture(rem)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        # first replay of every graph (uploads it), then an estimate of a replay's duration
+        self._run(1, rem)
+        stream.synchronize()
+        e0.record(stream)
+        self._run(1, 0)
+        e1.record(stream)
+        stream.synchronize()
+        t_replay = max(e0.elapsed_time(e1), 1e-3)
+        n_warm = max(-(-warmup // self.per_graph), int(MIN_WARM_MS / t_replay) + 1)
+        self._run(n_warm, rem)
+        stream.synchronize()
+        e0.record(stream)
+        self._run(full, rem)
+        e1.record(stream)
+        stream.synchronize()
+        return {"ms_per_step": e0.elapsed_time(e1) / steps, "warmup_steps_run": (n_warm + 2) * self.per_graph + 2 * rem,
+                "graph_replays_timed": (full + (1 if rem else 0)) if self.use_graph else 0,
+                "steps_per_full_graph": self.per_graph if self.use_graph else 0,
+                "steps_in_remainder_graph": rem if self.use_graph else 0}
+
+
+def decode_layer_sets(torch, F, L, dev, shapes, sets, M, dt, launch, steps, warmup, use_graph=True):
+    """Times `steps` layer-set steps over the distinct `sets` in rotation."""
+    n_copies = len(sets)
+    xs = {N: torch.randn(M, N, device=dev, generator=torch.Generator(device=dev).manual_seed(N)).to(dt)
+          for _, _, N in shapes}
+    ys = [torch.empty(M, K, dtype=dt, device=dev) for _, K, _ in shapes]
+    step_bytes = sum(algorithmic_bytes(pm, M) for pm in sets[0])
+    stream = torch.cuda.Stream(dev)
+    sp = stream.cuda_stream
+    xdt = F.dtype_code(dt)
+    groups = {"matrix": [[i] for i in range(len(shapes))],
+              "phase": [[0, 1, 2], [3], [4, 5], [6]],          # qkv | o | gate,up | down
+              "layer": [list(range(len(shapes)))]}[launch]
+    P = ctypes.c_void_p
+    calls, keep_alive = [], []
+    for s in sets:
+        cs = []
+        for g in groups:
+            n = len(g)
+            descs = (F.CbkDesc * n)(*[s[i].desc() for i in g])
+            xp = (P * n)(*[xs[shapes[i][2]].data_ptr() for i in g])
+            yp = (P * n)(*[ys[i].data_ptr() for i in g])
+            ldx = (ctypes.c_int64 * n)(*[shapes[i][2] for i in g])
+            ldy = (ctypes.c_int64 * n)(*[shapes[i][1] for i in g])
+            need = L.cbk_gemv_batch_workspace_bytes(n, descs, M)
+            w = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
+            keep_alive.append((descs, xp, yp, ldx, ldy, w))
+            cs.append((n, descs, xp, ldx, yp, ldy, w.data_ptr(), w.numel()))
+        calls.append(cs)
+
+    def step(i):
+        for n, descs, xp, ldx, yp, ldy, wp, wn in calls[i % n_copies]:
+            rc = L.cbk_gemv_batch(n, descs, xp, ldx, xdt, M, yp, ldy, xdt, None, wp, wn, sp)
+            if rc:
+                raise RuntimeError(L.cbk_strerror(rc).decode())
+
+    torch.cuda.synchronize()                                    # the weights were made on the default stream
+    with torch.cuda.stream(stream):
+        # outputs of layer set 0 in float32, for the parity check (untimed; the timed steps write x's type)
+        y32 = [torch.empty(M, K, dtype=torch.float32, device=dev) for _, K, _ in shapes]
+        for (n, descs, xp, ldx, _, ldy, wp, wn), g in zip(calls[0], groups):
+            yp32 = (P * n)(*[y32[i].data_ptr() for i in g])
+            rc = L.cbk_gemv_batch(n, descs, xp, ldx, xdt, M, yp32, ldy, F.F32, None, wp, wn, sp)
+            if rc:
+                raise RuntimeError(L.cbk_strerror(rc).decode())
+        stream.synchronize()
+        y_first = {name: y for (name, _, _), y in zip(shapes, y32)}
+        for i in range(n_copies):
+            step(i)
+        stream.synchronize()
+        timer = GraphTimer(torch, stream, step, n_copies, use_graph)
+        res = timer.measure(steps, warmup)
+    del timer, calls, keep_alive
+    res.update(step_bytes=step_bytes, launches=len(groups), distinct_layer_sets=n_copies,
+               gbs=step_bytes / (res["ms_per_step"] * 1e-3) / 1e9)
+    return res, xs, y_first
+
+
+def per_matrix(torch, F, L, dev, shapes, layout, bits, group, keep, M, dt, iters=24):
+    """Each distinct matrix of the layer set on its own: one launch per matrix, distinct copies of
+    at least 512 MB in rotation (the protocol of src/cobaltkernel/test_gemv.py:201-202, :521-522),
+    one HIP graph per rotation."""
+    rows, seen = [], set()
+    stream = torch.cuda.Stream(dev)
+    xdt = F.dtype_code(dt)
+    P = ctypes.c_void_p
+    for name, K, N in shapes:
+        if (K, N) in seen:
+            continue
+        seen.add((K, N))
+        one = K * F.row_stride(layout, N, bits, group, keep) + K * (N // group) * 3
+        copies = max(2, -(-2 * INFINITY_CACHE // one))
+        pms = [F.synth_packed(K, N, layout, bits, group, keep, seed=7000 + c, device=dev).to_tiled() for c in range(copies)]
+        x = torch.randn(M, N, device=dev, generator=torch.Generator(device=dev).manual_seed(N)).to(dt)
+        y = torch.empty(M, K, dtype=dt, device=dev)
+        args = []
+        for pm in pms:
+            d = (F.CbkDesc * 1)(pm.desc())
+            args.append((d, (P * 1)(x.data_ptr()), (ctypes.c_int64 * 1)(N), (P * 1)(y.data_ptr()), (ctypes.c_int64 * 1)(K)))
+
+        def rotation():
+            for d, xp, ldx, yp, ldy in args:
+                rc = L.cbk_gemv_batch(1, d, xp, ldx, xdt, M, yp, ldy, xdt, None, None, 0, stream.cuda_stream)
+                if rc:
+                    raise RuntimeError(L.cbk_strerror(rc).decode())
+
+        torch.cuda.synchronize()
+        with torch.cuda.stream(stream):
+            rotation()
+            stream.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                rotation()
+            for _ in range(3):
+                g.replay()
+            stream.synchronize()
+            reps = max(1, -(-iters // copies))
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(reps):
+                g.replay()
+            e1.record(stream)
+            stream.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / (reps * copies)
+        nbytes = algorithmic_bytes(pms[0], M)
+        rows.append({"matrix": f"{name} {K}x{N}", "bytes": nbytes, "distinct_copies": copies, "launches_timed": reps * copies,
+                     "us": round(us, 2), "gbs": round(nbytes / us / 1e3, 1),
+                     "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
+        del pms, args, g, x, y
+        torch.cuda.empty_cache()
+    return rows
+
+
+def lm_head_gemv(torch, F, ops, dev, workload, M, dt, reps=20):
+    """Decode kernel on the output projection of the model the workload is shaped after: dense
+    4-bit codes (DENSE4, the reference packer's default for the tied embedding,
+    src/cobaltkernel/pack_cobalt.py:561-563), vocabulary x hidden, one launch."""
+    N = SHAPES[workload][0][2]
+    K = VOCAB[workload]
+    pm = F.synth_packed(K, N, F.DENSE4, seed=3, device=dev).to_tiled()
+    copies = [pm]
+    while len(copies) * pm.stream_bytes() < 2 * INFINITY_CACHE:
+        copies.append(F.synth_packed(K, N, F.DENSE4, seed=3 + len(copies), device=dev).to_tiled())
+    x = torch.randn(M, N, device=dev, generator=torch.Generator(device=dev).manual_seed(1)).to(dt)
+    for i in range(2 * len(copies)):
+        y = ops.gemv(copies[i % len(copies)], x)
+    st = torch.cuda.current_stream()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    reps = -(-reps // len(copies)) * len(copies)
+    e0.record(st)
+    for i in range(reps):
+        y = ops.gemv(copies[i % len(copies)], x)
+    e1.record(st)
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / reps
+    nbytes = algorithmic_bytes(pm, M)
+    out = {"matrix": f"{K}x{N} DENSE4 ({pm.bpw():.4f} bpw), M={M}", "distinct_copies": len(copies), "ms": round(ms, 4), "bytes": nbytes,
+           "gbs": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    del pm, copies, x, y
+    return out
+
+
+# ------------------------------------------------------------------ prefill
+def prefill_parity(torch, ops, pm, x, nblocks=3, rows_per_block=64):
+    """rel. Frobenius error of sampled output rows (blocks of weight rows at the start, middle and
+    end of the matrix, every token) against a float64 matmul with the bit-exact dequantised
+    weights, float32 output."""
+    y = ops.gemm(pm, x, out_dtype=torch.float32)
+    num = den = 0.0
+    for b in range(nblocks):
+        r0 = (pm.K - rows_per_block) * b // max(1, nblocks - 1)
+        W = ops.dequant(pm, torch.float32, row0=r0, nrows=rows_per_block).double()
+        ref = x.double() @ W.T
+        num += float((y[:, r0:r0 + rows_per_block].double() - ref).pow(2).sum())
+        den += float(ref.pow(2).sum())
+        del W, ref
+    del y
+    return (num / den) ** 0.5
+
+
+def prefill_gemm(torch, F, ops, dev, shapes, names, layout, bits, group, keep, M, dt, reps=20, warm=10, parity=True):
+    """Prefill kernel on matrices `names` of a layer set (each distinct shape timed once, weighted
+    by how often it occurs)."""
+    by_name = {n: (K, N) for n, K, N in shapes}
+    rows, timed = [], {}
+    tot_flop = tot_ms = 0.0
+    worst = 0.0
+    bpw = None
+    for name in names:
+        K, N = by_name[name]
+        if (K, N) not in timed:
+            pm = F.synth_packed(K, N, layout, bits, group, keep, seed=7, device=dev).to_tiled()
+            x = torch.randn(M, N, device=dev, generator=torch.Generator(device=dev).manual_seed(N)).to(dt)
+            ws = ops.workspace_for(pm, M)                             # the caller's scratch, allocated once
+            for _ in range(warm):                                     # the first launches run at a lower clock
+                y = ops.gemm(pm, x, workspace=ws)
+            torch.cuda.synchronize()
+            st = torch.cuda.current_stream()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(st)
+            for _ in range(reps):
+                y = ops.gemm(pm, x, workspace=ws)
+            e1.record(st)
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / reps
+            err = prefill_parity(torch, ops, pm, x) if parity else None
+            if err is not None:
+                worst = max(worst, err)
+                assert err < 1e-3, f"prefill {name} {K}x{N} M={M}: rel. Frobenius error {err} against the dequantised weights"
+            timed[(K, N)] = ms
+            row = {"matrix": f"{name} {K}x{N}", "ms": round(ms, 4), "tflops": round(2.0 * M * K * N / ms / 1e9, 1)}
+            if err is not None:
+                row["rel_fro_vs_dequant_f64"] = float(f"{err:.3g}")
+            rows.append(row)
+            bpw = pm.bpw()
+            del pm, x, y, ws
+        tot_flop += 2.0 * M * K * N
+        tot_ms += timed[(K, N)]
+    ach = tot_flop / tot_ms / 1e9
+    out = {"matrices": "+".join(names), "M": M, "dtype": str(dt)[6:], "layout": F.LAYOUT_NAME[layout], "bits": bits,
+           "keep_per_32": keep, "group": group, "bpw": round(bpw, 4), "ms": round(tot_ms, 4), "tflops": round(ach, 1),
+           "note": "time includes the activation pre-scaling kernel (and the reduction kernel of a split column range)",
+           "per_matrix": rows,
+           "roofline": {"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                        "frac": round(ach / MFMA_PEAK_TFLOPS, 4), "traffic": None, "kernel": "cbk::gemm_big_kernel"}}
+    if parity:
+        out["parity"] = {"worst_rel_fro": float(f"{worst:.3g}"), "tolerance": 1e-3,
+                         "how": "192 sampled weight rows x all tokens of every timed matrix, float32 output against "
+                                "x.double() @ dequant(W).double().T"}
+    return out
+
+
+# ------------------------------------------------------------------ ceilings and CPU baseline
 def measured_ceilings(torch, dev):
     """What this GPU reaches on back-to-back dense f16 MFMAs and on a plain streaming read of
     1 GiB (libcbk_bench.so, built by `python -m cobalt_amd.build`): ceilings to read the kernels'
     figures against, beside the published peaks.  None if the helper library is not built."""
-    import ctypes
     path = os.path.join(ROOT, "cobalt_amd", "libcbk_bench.so")
     if not os.path.exists(path):
         return None
@@ -152,90 +411,146 @@ def measured_ceilings(torch, dev):
                    "grid-stride 16-byte reads of 1 GiB, eight in flight per lane, best of three grid sizes"}
 
 
-VOCAB = {"mistral7b": 32000, "gemma27b": 262144}
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return platform.processor() or "unknown"
 
 
-def lm_head_gemv(torch, F, ops, dev, workload, M, dt, reps=20):
-    """Decode kernel on the output projection of the model the workload is shaped after: dense
-    4-bit codes (DENSE4, the reference packer's default for the tied embedding,
-    src/cobaltkernel/pack_cobalt.py:561-563), vocabulary x hidden, one launch."""
-    N = SHAPES[workload][0][2]
-    K = VOCAB[workload]
-    pm = F.synth_packed(K, N, F.DENSE4, seed=3, device=dev).to_tiled()
-    # successive calls rotate over as many copies of the matrix as exceed twice the 256 MB Infinity Cache
-    copies = [pm]
-    while len(copies) * pm.stream_bytes() < 2 * 256 * 2**20:
-        copies.append(F.synth_packed(K, N, F.DENSE4, seed=3 + len(copies), device=dev).to_tiled())
-    x = torch.randn(M, N, device=dev, generator=torch.Generator(device=dev).manual_seed(1)).to(dt)
-    for i in range(2 * len(copies)):
-        y = ops.gemv(copies[i % len(copies)], x)
-    st = torch.cuda.current_stream()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    reps = -(-reps // len(copies)) * len(copies)
-    e0.record(st)
-    for i in range(reps):
-        y = ops.gemv(copies[i % len(copies)], x)
-    e1.record(st)
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / reps
-    nbytes = algorithmic_bytes(pm, M)
-    out = {"matrix": f"{K}x{N} DENSE4 ({pm.bpw():.4f} bpw), M={M}", "distinct_copies": len(copies), "ms": round(ms, 4), "bytes": nbytes,
-           "gbs": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
-    del pm, copies, x, y
-    return out
+def cpu_baseline(torch, pms, shapes, xs, ys, M, budget_s=25.0):
+    """The reference's CPU forward restated in torch (oracle/torch_ref.py): per distinct shape of
+    the layer set, (i) dequantise-then-matmul per call (the module's low-memory path,
+    benchmarks/benchmark_suite.py:1201-1209) and (ii) matmul with the dequantised weights cached
+    (:1210-1217), float32, all the host cores this process may use; on the packed bytes the GPU
+    used.  The C oracle checks the GPU outputs of the same layer set first."""
+    import numpy as np
+    from oracle import cbk_ref_c as C
+    from oracle import torch_ref as T
+    usable = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    # the GPU boxes share their host: a process is given 16 cores whatever os.cpu_count() shows
+    cores = max(1, min(usable, int(os.environ.get("OMP_NUM_THREADS", usable) or usable)))
+    torch.set_num_threads(cores)
+    C.set_threads(min(16, cores))
+    worst = 0.0
+    t_stop = time.time() + budget_s
+    for pm, (name, K, N) in zip(pms, shapes):                       # parity of the GPU outputs (checker, untimed)
+        pk = dict(data=pm.array("data").numpy(), scale=pm.array("scale").numpy().reshape(K, -1),
+                  zero=pm.array("zero").numpy().reshape(K, -1))
+        cs = pm.array("col_scale").numpy().reshape(pm.cs_rows, N) if pm.cs_rows else None
+        y = C.forward(pk, K, N, pm.layout, xs[N].float().cpu().numpy(), col_scale=cs, bits=pm.bits, group=pm.group,
+                      keep_per_block=pm.keep or None)
+        got = ys[name].float().cpu().numpy()
+        worst = max(worst, float(np.linalg.norm(got - y) / np.linalg.norm(y)))
+    rows, seen = [], set()
+    tot_bytes = tot_a = tot_b = 0.0
+    order = sorted(range(len(shapes)), key=lambda i: shapes[i][1] * shapes[i][2])       # small shapes first
+    for i in order:
+        name, K, N = shapes[i]
+        if (K, N) in seen:
+            continue
+        if rows and time.time() > t_stop:
+            break
+        seen.add((K, N))
+        pm = pms[i]
+        stride = pm.data_bytes // K
+        data = pm.array("data")[: K * stride].reshape(K, stride)
+        scale = pm.array("scale").reshape(K, -1)
+        zero = pm.array("zero").reshape(K, -1)
+        cs = pm.array("col_scale").reshape(pm.cs_rows, N) if pm.cs_rows else None
+        x = xs[N].cpu()
+        deq = lambda: T.dequant(data, scale, zero, cs, K, N, pm.layout, pm.bits, pm.group, pm.keep or 16)
+        W = deq()
+        T.forward(W, x)                                               # warm-up of both parts
+        ta, tb = [], []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            W = deq()
+            y = T.forward(W, x)
+            ta.append(time.perf_counter() - t0)
+            if time.time() > t_stop:
+                break
+        for _ in range(5):
+            t0 = time.perf_counter()
+            y = T.forward(W, x)
+            tb.append(time.perf_counter() - t0)
+        a, b = sorted(ta)[len(ta) // 2], sorted(tb)[len(tb) // 2]
+        nbytes = algorithmic_bytes(pm, M)
+        mult = sum(1 for _, k, n in shapes if (k, n) == (K, N))
+        tot_bytes += nbytes * mult
+        tot_a += a * mult
+        tot_b += b * mult
+        rows.append({"matrix": f"{name} {K}x{N}", "dequant_matmul_ms": round(a * 1e3, 2), "matmul_cached_ms": round(b * 1e3, 3),
+                     "runs": [len(ta), len(tb)]})
+        del W, y
+    done = "+".join(r["matrix"].split()[0] for r in rows)
+    return dict(value=round(tot_bytes / tot_a / 1e9, 4), unit="GB/s", cores=cores, kind="port",
+                sample=f"torch {torch.__version__} float32 dequantise-then-matmul per call at M={M} over the distinct shapes "
+                       f"{done} of the first layer set (same packed bytes as the GPU run), median of up to 3 runs each after one "
+                       f"warm-up, {cores} threads on {cpu_model()} ({os.cpu_count()} logical CPUs visible); `value` is the "
+                       f"algorithmic bytes of those matrices per second of the per-call path; `matmul_cached_gbs` is the "
+                       f"same bytes over the matmul with cached float32 weights (median of 5)",
+                matmul_cached_gbs=round(tot_bytes / tot_b / 1e9, 3), per_matrix=rows,
+                ms_per_layer_set_dequant_matmul=round(tot_a * 1e3, 1), ms_per_layer_set_matmul_cached=round(tot_b * 1e3, 2),
+                gpu_vs_oracle_rel_fro=worst, checker="C oracle (oracle/cbk_ref.c) on every matrix of the first layer set")
 
 
-def prefill_gemm(torch, F, ops, dev, workload, layout, bits, group, keep, M, dt, reps=20, warm=10):
-    """Prefill kernel on the MLP matrices (gate, up, down) of a layer set."""
-    shapes = {n: (K, N) for n, K, N in SHAPES[workload]}
-    rows = []
-    tot_flop, tot_ms = 0.0, 0.0
-    for name in ("gate", "down"):
-        K, N = shapes[name]
-        pm = F.synth_packed(K, N, layout, bits, group, keep, seed=7, device=dev).to_tiled()
-        x = torch.randn(M, N, device=dev, generator=torch.Generator(device=dev).manual_seed(N)).to(dt)
-        ws = ops.workspace_for(pm, M)                             # the caller's scratch, allocated once
-        for _ in range(warm):                                     # the first launches run at a lower clock
-            y = ops.gemm(pm, x, workspace=ws)
-        torch.cuda.synchronize()
-        st = torch.cuda.current_stream()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(st)
-        for _ in range(reps):
-            y = ops.gemm(pm, x, workspace=ws)
-        e1.record(st)
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / reps
-        flop = 2.0 * M * K * N
-        tot_flop += flop * (2 if name == "gate" else 1)         # gate and up have the same shape
-        tot_ms += ms * (2 if name == "gate" else 1)
-        rows.append({"matrix": f"{name} {K}x{N}", "ms": round(ms, 4), "tflops": round(flop / ms / 1e9, 1)})
-        bpw = pm.bpw()
-        del pm, x, y, ws
-    ach = tot_flop / tot_ms / 1e9
-    return {"workload": f"{workload} MLP (gate, up, down), M={M}, {str(dt)[6:]} activations, {F.LAYOUT_NAME[layout]} "
-                        f"{bits}-bit keep {keep}/32 group {group}, {bpw:.4f} bpw; time includes the activation "
-                        "pre-scaling kernel (and the reduction kernel of a split column range)",
-            "tflops": round(ach, 1), "per_matrix": rows,
-            "roofline": {"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                         "frac": round(ach / MFMA_PEAK_TFLOPS, 4), "traffic": None,
-                         "kernel": "cbk::gemm_big_kernel"}}
+# ------------------------------------------------------------------ the nine-cell grid
+def grid(torch, F, ops, L, dev, a):
+    """Gemma-3-27B shapes x 62 layers, sparsity 0.3 / 0.5 / 0.7 as 23 / 16 / 10 survivors per 32
+    columns, 2 / 3 / 4-bit codes, group 64: decode step at M=1 and prefill at M=4096, bf16."""
+    shapes = SHAPES["gemma27b"]
+    dt = torch.bfloat16
+    params = sum(K * N for _, K, N in shapes)
+    cells = []
+    for keep in (23, 16, 10):
+        for bits in (2, 3, 4):
+            sets, _ = make_sets(torch, F, dev, shapes, F.BLKC, bits, 64, keep, 2 * INFINITY_CACHE)
+            res, _, _ = decode_layer_sets(torch, F, L, dev, shapes, sets, 1, dt, "phase", a.steps, a.warmup)
+            bpw = sets[0][0].bpw()
+            del sets
+            torch.cuda.empty_cache()
+            pf = prefill_gemm(torch, F, ops, dev, shapes, [n for n, _, _ in shapes], F.BLKC, bits, 64, keep, a.grid_prefill_m, dt,
+                              reps=5, warm=3, parity=False)
+            cell = {"sparsity": round(1 - keep / 32, 4), "keep_per_32": keep, "bits": bits, "group": 64, "bpw": round(bpw, 4),
+                    "layer_set_bytes": res["step_bytes"],
+                    "decode_ms_per_layer": round(res["ms_per_step"], 5), "decode_gbs": round(res["gbs"], 1),
+                    "decode_frac_of_hbm_peak": round(res["gbs"] / HBM_PEAK_GBS, 4),
+                    "decode_linear_ms_per_token_62_layers": round(res["ms_per_step"] * GEMMA_LAYERS, 3),
+                    "prefill_ms_per_layer": pf["ms"], "prefill_tflops": pf["tflops"],
+                    "prefill_frac_of_mfma_peak": round(pf["tflops"] / MFMA_PEAK_TFLOPS, 4),
+                    "prefill_linear_us_per_token_62_layers": round(pf["ms"] * GEMMA_LAYERS * 1e3 / a.grid_prefill_m, 3)}
+            cells.append(cell)
+            print(json.dumps(cell), file=sys.stderr, flush=True)
+    return {"metric": "decode GEMV HBM GB/s (% of 8 TB/s) at M=1; prefill GEMM TFLOP/s at M=4096", "mode": "grid",
+            "config": {"workload": f"gemma27b 62-layer linear stack ({params} parameters per layer), bf16 activations, group 64, "
+                                   f"sparsity 0.3/0.5/0.7 realised as 23/16/10 survivors per 32 columns, 2/3/4-bit codes; "
+                                   f"decode M=1 (phase-batched launches from HIP graphs, distinct layer sets beyond 2x the "
+                                   f"Infinity Cache in rotation, x62 for the stack), prefill M={a.grid_prefill_m} (all seven "
+                                   f"matrices of a layer, x62)",
+                       "steps": a.steps, "warmup": a.warmup},
+            "n_gpus": 1, "data": "synthetic", "cells": cells}
 
 
+# ------------------------------------------------------------------ main
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=1000)
-    ap.add_argument("--warmup", type=int, default=500)
-    ap.add_argument("--workload", default="mistral7b", choices=list(SHAPES))
+    ap.add_argument("--steps", type=int, default=640)
+    ap.add_argument("--warmup", type=int, default=320)
+    ap.add_argument("--workload", default="gemma27b", choices=list(SHAPES))
     ap.add_argument("--m", type=int, default=1)
-    ap.add_argument("--dtype", default="f16", choices=["f16", "bf16"])
+    ap.add_argument("--dtype", default=None, choices=["f16", "bf16"], help="activation type (default: the workload's)")
     ap.add_argument("--bits", type=int, default=4)
     ap.add_argument("--keep", type=int, default=16)
     ap.add_argument("--group", type=int, default=128)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-core baseline")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM measurement")
     ap.add_argument("--no-lm-head", action="store_true", help="skip the output-projection GEMV measurement")
+    ap.add_argument("--no-secondary", action="store_true", help="skip the other workload's decode step and the per-matrix rows")
     ap.add_argument("--prefill-workload", default="gemma27b", choices=list(SHAPES))
     ap.add_argument("--prefill-m", type=int, default=2048)
     ap.add_argument("--prefill-dtype", default="bf16", choices=["f16", "bf16"])
@@ -244,166 +559,93 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch from the host instead of replaying HIP graphs")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 1 GiB device-to-device copy (reference reading for the HBM traffic counters)")
+    ap.add_argument("--grid", action="store_true", help="the nine-cell sweep of the 62-layer Gemma stack instead of the headline")
+    ap.add_argument("--grid-prefill-m", type=int, default=4096)
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
     import torch
-    from cobalt_amd import format as F, ops
+    from cobalt_amd import _lib, format as F, ops
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    layout = F.BLK1632_4 if (a.bits, a.keep, a.group) == (4, 16, 128) else \
-        F.BLK1632_6 if (a.bits, a.keep, a.group) == (6, 16, 128) else F.BLKC
-    dt = torch.float16 if a.dtype == "f16" else torch.bfloat16
+    L = _lib.lib()
+    if a.grid:
+        print(json.dumps(grid(torch, F, ops, L, dev, a)))
+        return
+    layout = layout_of(F, a.bits, a.keep, a.group)
+    dname = a.dtype or WORKLOAD_DTYPE[a.workload]
+    dt = torch_dtype(torch, dname)
     shapes = SHAPES[a.workload]
     M = a.m
 
-    set_bytes = sum(K * F.row_stride(layout, N, a.bits, a.group, a.keep) + K * (N // a.group) * 3 for _, K, N in shapes)
-    n_copies = max(2, -(-2 * 256 * 2**20 // set_bytes))
-    sets, first_rowmajor = [], None
-    for c in range(n_copies):
-        rm = [F.synth_packed(K, N, layout, a.bits, a.group, a.keep, seed=1000 * c + i, device=dev)
-              for i, (_, K, N) in enumerate(shapes)]
-        if c == 0 and not a.no_cpu:
-            first_rowmajor = [p.to("cpu") for p in rm]
-        sets.append([p.to_tiled() for p in rm])
-        del rm
-    xs = {N: torch.randn(M, N, device=dev, generator=torch.Generator(device=dev).manual_seed(N)).to(dt)
-          for _, _, N in shapes}
-    ys = [torch.empty(M, K, dtype=dt, device=dev) for _, K, _ in shapes]
-    step_bytes = sum(algorithmic_bytes(pm, M) for pm in sets[0])
+    sets, first_rowmajor = make_sets(torch, F, dev, shapes, layout, a.bits, a.group, a.keep, 2 * INFINITY_CACHE,
+                                     keep_first_rowmajor=not a.no_cpu)
+    bpw = sets[0][0].bpw()
+    res, xs, y_first = decode_layer_sets(torch, F, L, dev, shapes, sets, M, dt, a.launch, a.steps, a.warmup, not a.no_graph)
+    if a.copy_calibration:
+        src = torch.empty(2**30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    del sets
+    torch.cuda.empty_cache()
 
-    import ctypes
-    from cobalt_amd import _lib
-    L = _lib.lib()
-    stream = torch.cuda.Stream(dev)
-    sp = stream.cuda_stream
-    xdt = F.dtype_code(dt)
-    groups = {"matrix": [[i] for i in range(len(shapes))],
-              "phase": [[0, 1, 2], [3], [4, 5], [6]],          # qkv | o | gate,up | down
-              "layer": [list(range(len(shapes)))]}[a.launch]
-    P = ctypes.c_void_p
-    calls = []                                                  # per layer set: list of batched calls
-    keep_alive = []
-    for s in sets:
-        cs = []
-        for g in groups:
-            n = len(g)
-            descs = (F.CbkDesc * n)(*[s[i].desc() for i in g])
-            xp = (P * n)(*[xs[shapes[i][2]].data_ptr() for i in g])
-            yp = (P * n)(*[ys[i].data_ptr() for i in g])
-            ldx = (ctypes.c_int64 * n)(*[shapes[i][2] for i in g])
-            ldy = (ctypes.c_int64 * n)(*[shapes[i][1] for i in g])
-            need = L.cbk_gemv_batch_workspace_bytes(n, descs, M)
-            w = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
-            keep_alive.append((descs, xp, yp, ldx, ldy, w))
-            cs.append((n, descs, xp, ldx, yp, ldy, w.data_ptr(), w.numel()))
-        calls.append(cs)
-
-    def launch(c):
-        n, descs, xp, ldx, yp, ldy, wp, wn = c
-        rc = L.cbk_gemv_batch(n, descs, xp, ldx, xdt, M, yp, ldy, xdt, None, wp, wn, sp)
-        if rc:
-            raise RuntimeError(L.cbk_strerror(rc).decode())
-
-    def step(i):
-        for c in calls[i % n_copies]:
-            launch(c)
-
-    launches = len(groups)
-    torch.cuda.synchronize()                                    # the weights were made on the default stream
-    with torch.cuda.stream(stream):
-        step(0)
-        stream.synchronize()
-        y_first = {name: y.clone() for (name, _, _), y in zip(shapes, ys)}   # outputs of layer set 0, for the parity check
-        for i in range(1, n_copies):
-            step(i)
-        stream.synchronize()
-        graphs = None
-        per_graph = 0
-        if not a.no_graph:                                      # one HIP graph per distinct layer set
-            graphs = []
-            for i in range(n_copies):
-                g = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(g, stream=stream):
-                    step(i)
-                graphs.append(g)
-            # and one graph of about 32 layer sets in a row (whole rotations of the distinct sets),
-            # as a decoder replays all its layers per token
-            per_graph = -(-32 // n_copies) * n_copies
-            g_all = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g_all, stream=stream):
-                for i in range(per_graph):
-                    step(i)
-        run = (lambda i: graphs[i % n_copies].replay()) if graphs else step
-
-        def run_steps(first, count):                             # exactly `count` steps, layer sets in rotation
-            i = first
-            while count > 0:
-                if graphs and i % n_copies == 0 and count >= per_graph:
-                    g_all.replay()
-                    i += per_graph
-                    count -= per_graph
-                else:
-                    run(i)
-                    i += 1
-                    count -= 1
-            return i
-
-        nxt = run_steps(0, a.warmup)
-        stream.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(stream)
-        run_steps(nxt, a.steps)
-        e1.record(stream)
-        stream.synchronize()
-        ms_per_step = e0.elapsed_time(e1) / a.steps
-
-        if a.copy_calibration:
-            src = torch.empty(2**30, dtype=torch.uint8, device=dev)
-            dst = torch.empty_like(src)
-            for _ in range(3):
-                dst.copy_(src)
-            stream.synchronize()
-            del src, dst
-
-    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    ms_per_step, step_bytes, launches = res["ms_per_step"], res["step_bytes"], res["launches"]
+    value = res["gbs"]
     # average launch of the decode kernel over the timed region (HIP events on the launch stream);
     # it contains the gap between consecutive launches, so it is an upper bound of the kernel time
     us_per_launch = ms_per_step * 1e3 / launches
     bytes_per_launch = step_bytes / launches
     achieved = bytes_per_launch / (us_per_launch * 1e-6) / 1e9
-    bpw = sets[0][0].bpw()
+    traffic = MEASURED_TRAFFIC.get((a.workload, a.launch, M)) if (a.bits, a.keep, a.group) == (4, 16, 128) else None
     out = {
         "metric": "decode GEMV HBM GB/s (% of 8 TB/s) at M=1; prefill GEMM TFLOP/s at M=2048",
         "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "i8 (int8 MFMA on integer codes and 3-digit block-fixed-point activations, f32 scales)",
         "data": "synthetic",
-        "config": {"workload": f"{a.workload} decode layer set, 7 GEMVs, M={M}, {a.dtype} activations, sparsity "
+        "config": {"workload": f"{a.workload} decode layer set, 7 GEMVs, M={M}, {dname} activations, sparsity "
                                f"{1 - a.keep / 32:.4g}, {a.bits}-bit, group {a.group}, layout {F.LAYOUT_NAME[layout]}, "
                                f"{bpw:.4f} bpw",
-                   "layer_set_bytes": step_bytes, "distinct_layer_sets": n_copies,
+                   "layer_set_bytes": step_bytes, "distinct_layer_sets": res["distinct_layer_sets"],
                    "launches_per_step": launches, "launch_grouping": a.launch,
-                   "hip_graph": not a.no_graph,
-                   "steps_per_graph_replay": (per_graph if not a.no_graph else 0), "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
+                   "hip_graph": not a.no_graph, "graph_replays_timed": res["graph_replays_timed"],
+                   "steps_per_full_graph": res["steps_per_full_graph"],
+                   "steps_in_remainder_graph": res["steps_in_remainder_graph"],
+                   "warmup_steps_run": res["warmup_steps_run"], "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC.get((a.workload, a.launch, M)),
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "traffic_source": ("stored figure of the rocprofv3 counter runs summarised under profiles/, "
+                                        "not read in this run") if traffic else None,
                      "kernel": "cbk::gemv_mfma_kernel", "avg_launch_us": round(us_per_launch, 3),
                      "launches_timed": a.steps * launches, "bytes_per_launch": int(bytes_per_launch)},
     }
-    g_all = None
-    del graphs, sets, calls, keep_alive
-    torch.cuda.empty_cache()
+    if not a.no_secondary:
+        out["per_matrix"] = per_matrix(torch, F, L, dev, shapes, layout, a.bits, a.group, a.keep, M, dt)
+        other = "mistral7b" if a.workload == "gemma27b" else "gemma27b"
+        oshapes, odt = SHAPES[other], torch_dtype(torch, WORKLOAD_DTYPE[other])
+        osets, _ = make_sets(torch, F, dev, oshapes, layout, a.bits, a.group, a.keep, 2 * INFINITY_CACHE)
+        ores, _, _ = decode_layer_sets(torch, F, L, dev, oshapes, osets, M, odt, a.launch, a.steps, a.warmup, not a.no_graph)
+        out[f"decode_{other}"] = {"workload": f"{other} decode layer set, M={M}, {WORKLOAD_DTYPE[other]} activations, same layout",
+                                  "ms_per_step": round(ores["ms_per_step"], 5), "gbs": round(ores["gbs"], 1),
+                                  "frac_of_hbm_peak": round(ores["gbs"] / HBM_PEAK_GBS, 4),
+                                  "layer_set_bytes": ores["step_bytes"], "distinct_layer_sets": ores["distinct_layer_sets"]}
+        del osets
+        torch.cuda.empty_cache()
     if not a.no_prefill:
-        out["prefill_gemm"] = prefill_gemm(torch, F, ops, dev, a.prefill_workload, layout, a.bits, a.group, a.keep,
-                                           a.prefill_m, torch.float16 if a.prefill_dtype == "f16" else torch.bfloat16)
+        pdt = torch_dtype(torch, a.prefill_dtype)
+        out["prefill_gemm"] = prefill_gemm(torch, F, ops, dev, SHAPES[a.prefill_workload], ["gate", "up", "down"], layout,
+                                           a.bits, a.group, a.keep, a.prefill_m, pdt)
+        out["prefill_gemm"]["workload"] = f"{a.prefill_workload} MLP (gate, up, down), M={a.prefill_m}, {a.prefill_dtype} activations"
         # the same kernel's 64-token tile at a batched-decoding row count, on the decode workload's shapes
-        mid = prefill_gemm(torch, F, ops, dev, a.workload, layout, a.bits, a.group, a.keep, 64,
-                           torch.float16 if a.dtype == "f16" else torch.bfloat16)
-        out["gemm_m64"] = {"workload": mid["workload"], "tflops": mid["tflops"], "per_matrix": mid["per_matrix"]}
+        mid = prefill_gemm(torch, F, ops, dev, shapes, ["gate", "up", "down"], layout, a.bits, a.group, a.keep, 64, dt,
+                           parity=False)
+        out["gemm_m64"] = {"workload": f"{a.workload} MLP (gate, up, down), M=64, {dname} activations",
+                           "tflops": mid["tflops"], "per_matrix": mid["per_matrix"]}
     if not a.no_lm_head:
         out["lm_head_gemv"] = lm_head_gemv(torch, F, ops, dev, a.workload, M, dt)
     ceil = measured_ceilings(torch, dev)
@@ -414,8 +656,7 @@ def main():
             out["prefill_gemm"]["roofline"]["frac_of_measured_mfma"] = round(
                 out["prefill_gemm"]["tflops"] / ceil["mfma_f16_dense_tflops"], 4)
     if not a.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(first_rowmajor, shapes, xs, y_first, M)
-        # outputs are rounded to the activation dtype (2^-11 relative) on top of the kernel's own error
+        out["cpu_baseline"] = cpu_baseline(torch, first_rowmajor, shapes, xs, y_first, M)
         assert out["cpu_baseline"]["gpu_vs_oracle_rel_fro"] < 1e-3, "GPU outputs disagree with the oracle"
     print(json.dumps(out))
 

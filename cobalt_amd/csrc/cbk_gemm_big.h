@@ -80,7 +80,7 @@ __device__ inline void dma_x16(const void* base, uint32_t voff, uint32_t lds) {
   const uint64_t sbase = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b64) |
                          ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b64 >> 32)) << 32);
   lds = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds);
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds) : "memory");
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds) : "memory", "m0");
 }
 
 // eight signed bytes (q - z for a kept column, 0 for a pruned one) -> eight halfs times scale

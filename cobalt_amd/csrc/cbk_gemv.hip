@@ -634,9 +634,13 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
           for (int p = 0; p < MP; ++p)
             if (kq == 0 && p < h.M) rs[(part * h.M + p) * 16 + wr] = part_sum[p];
         }
+        // release: this wave's partial sums are in LDS before its arrival is counted; acquire: the
+        // last arriver reads the other waves' sums only after it has seen all their arrivals
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         int old = 0;
         if (lane == 0) old = atomicAdd(&cnt[slot], 1);
         old = __builtin_amdgcn_readfirstlane(old);                 // lane 0 holds it, and every lane is active here
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
         if (old == SK - 1) {                                      // uniform over the wave
           // quarter kq finishes activation row kq (M <= 4); the partial sums are read four at a
           // time (parts past SK re-read the last one and do not count) and added in part order
