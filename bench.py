@@ -234,10 +234,11 @@ def per_matrix(torch, F, L, dev, shapes, layout, bits, group, keep, M, dt, iters
         for pm in pms:
             d = (F.CbkDesc * 1)(pm.desc())
             args.append((d, (P * 1)(x.data_ptr()), (ctypes.c_int64 * 1)(N), (P * 1)(y.data_ptr()), (ctypes.c_int64 * 1)(K)))
+        w = torch.empty(max(L.cbk_gemv_batch_workspace_bytes(1, args[0][0], M), 256), dtype=torch.uint8, device=dev)
 
         def rotation():
             for d, xp, ldx, yp, ldy in args:
-                rc = L.cbk_gemv_batch(1, d, xp, ldx, xdt, M, yp, ldy, xdt, None, None, 0, stream.cuda_stream)
+                rc = L.cbk_gemv_batch(1, d, xp, ldx, xdt, M, yp, ldy, xdt, None, w.data_ptr(), w.numel(), stream.cuda_stream)
                 if rc:
                     raise RuntimeError(L.cbk_strerror(rc).decode())
 
@@ -263,7 +264,7 @@ def per_matrix(torch, F, L, dev, shapes, layout, bits, group, keep, M, dt, iters
         rows.append({"matrix": f"{name} {K}x{N}", "bytes": nbytes, "distinct_copies": copies, "launches_timed": reps * copies,
                      "us": round(us, 2), "gbs": round(nbytes / us / 1e3, 1),
                      "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
-        del pms, args, g, x, y
+        del pms, args, g, x, y, w
         torch.cuda.empty_cache()
     return rows
 

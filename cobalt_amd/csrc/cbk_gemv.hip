@@ -636,11 +636,11 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
         }
         // release: this wave's partial sums are in LDS before its arrival is counted; acquire: the
         // last arriver reads the other waves' sums only after it has seen all their arrivals
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
         int old = 0;
         if (lane == 0) old = atomicAdd(&cnt[slot], 1);
         old = __builtin_amdgcn_readfirstlane(old);                 // lane 0 holds it, and every lane is active here
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
         if (old == SK - 1) {                                      // uniform over the wave
           // quarter kq finishes activation row kq (M <= 4); the partial sums are read four at a
           // time (parts past SK re-read the last one and do not count) and added in part order
