@@ -28,6 +28,7 @@ SIGNATURES = {
                                    ctypes.c_int64, _P]),
     "cbk_gemv": (ctypes.c_int, _MM),
     "cbk_gemm": (ctypes.c_int, _MM),
+    "cbk_gemm_static": (ctypes.c_int, _MM[:9] + [_P]),
     "cbk_gemv_batch_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, _DP, ctypes.c_int]),
     "cbk_gemv_batch": (ctypes.c_int, [ctypes.c_int, _DP, ctypes.POINTER(_P), ctypes.POINTER(ctypes.c_int64),
                                       ctypes.c_int, ctypes.c_int, ctypes.POINTER(_P), ctypes.POINTER(ctypes.c_int64),

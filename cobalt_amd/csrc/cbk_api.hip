@@ -1,5 +1,7 @@
 // extern "C" surface of libcbk_hip.so: host-side descriptor checks and kernel dispatch.
-// No allocation, no host synchronisation, no global state.
+// No allocation, no host synchronisation; the only global state is the scratch array of
+// cbk_gemm_static and its per-device address.
+#include <mutex>
 #include "cbk_device.h"
 
 namespace cbk {
@@ -333,6 +335,48 @@ int cbk_gemm(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ldx,
     return CBK_OK;
   }
   return launch_gemm(m, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, (hipStream_t)stream);
+}
+
+}  // extern "C"
+
+// ------------------------------------------------------------------ cbk_gemm without a workspace argument
+// Scratch of cbk_gemm_static: the pre-scaled activations and the partial output tiles that
+// cbk_gemm keeps in the caller's workspace.  One copy per GPU, at its own address on each; in
+// host code the name of the array is only a handle for hipGetSymbolAddress, never an address.
+static __device__ __align__(256) unsigned char scratch[CBK_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mu;
+void* scratch_ptr[kMaxDevices];          // device address of `scratch` on every GPU seen so far
+
+// The address of this GPU's copy of the array (looked up once per device, with that device
+// current: the caller's), or nullptr if the runtime refuses.
+void* scratch_of_current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> g(scratch_mu);
+  if (!scratch_ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+    scratch_ptr[dev] = p;
+  }
+  return scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" {
+
+int cbk_gemm_static(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ldx, void* y, int y_dtype,
+                    int64_t ldy, const void* bias, void* stream) {
+  if (cbk_workspace_bytes(in, M) > (size_t)CBK_STATIC_SCRATCH_BYTES) {
+    DMat m;
+    const int rc = to_dmat(in, &m, true);
+    return rc ? rc : CBK_ERR_WORKSPACE;                             // more scratch than the array holds
+  }
+  void* ws = scratch_of_current_device();
+  if (!ws) return CBK_ERR_HIP;
+  return cbk_gemm(in, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, ws, (size_t)CBK_STATIC_SCRATCH_BYTES, stream);
 }
 
 int cbk_linear(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ldx, void* y, int y_dtype,

@@ -166,6 +166,21 @@ int cbk_gemm(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
              void* y, int y_dtype, int64_t ldy, const void* bias,
              void* workspace, size_t workspace_bytes, void* stream);
 
+/* cbk_gemm for callers that cannot allocate device memory or pass a workspace: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in
+ * the reference.  Same computation and same results as cbk_gemm, with the scratch (pre-scaled
+ * activations, partial output tiles) in an array of CBK_STATIC_SCRATCH_BYTES that is part of the
+ * library's device image: every GPU the library runs on holds one copy until the process ends.
+ * The call allocates and frees nothing.  A call whose cbk_workspace_bytes() exceeds the array is
+ * refused with CBK_ERR_WORKSPACE before anything is launched (16 MiB hold e.g. 1024 activation
+ * rows of 5376 columns; prompts beyond that go through cbk_gemm).  All calls on one GPU share
+ * that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race;
+ * calls on one stream are safe.  Nothing in the array needs to start at zero and nothing is
+ * carried from one call to the next. */
+#define CBK_STATIC_SCRATCH_BYTES (16u << 20)
+int cbk_gemm_static(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
+                    void* y, int y_dtype, int64_t ldy, const void* bias, void* stream);
+
 /* The layer forward: cbk_gemv for M <= 8, cbk_gemm above (the module seam of
  * benchmarks/benchmark_suite.py:1200-1217). */
 int cbk_linear(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
