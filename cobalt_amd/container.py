@@ -1,19 +1,27 @@
 """CBK1 directories: `manifest.json` plus one `.bin` per decoder layer, each a concatenation of
 256-byte aligned arrays that are, byte for byte, what the kernels read (reference:
 docs/FORMAT.md:1-37 container, :126-151 fused matrices and `alias_of`; writer
-src/cobaltkernel/pack_cobalt.py:390-505; loader src/cobaltkernel/runner.py:413-484).
+src/cobaltkernel/pack_cobalt.py:390-505 and :561-714; loader src/cobaltkernel/runner.py:413-484).
 
-Reading is offset-driven: every matrix entry of the manifest names its blob and the offset and
-length of each of its arrays, so row-fused matrices and the `alias_of` entries that point into
-them need no special case.  A layer's blob is loaded once; the PackedMatrix of every matrix in
-it is a view (offset table) onto that one tensor.  On disk the rows are in the reference's
-row-major order; `to_tiled()` reorders them for the decode kernel after the move to the GPU.
+The manifest is the reference's: `layers[i] = {file, matrices: {name: entry}, norms, bytes}`; an
+entry holds K, N, G, layout, layout_name, arrays{data, row_off?, scale, zero, col_scale?: {off,
+bytes}}, cs_rows, n_survivors, n_zero_fixed, stream_bytes, bpw.  A row-concatenated q|k|v matrix
+carries `fused_from`, `row_ranges` and `cs_row_of`; the entries of its parts carry `alias_of` and
+`alias_row_start`, byte ranges inside the fused arrays (their `data.bytes` has no 64-byte tail,
+pack_cobalt.py:474-503) and a column scale of their own.  The layouts this package adds to the
+reference's (BLKC, DENSEB) put their `bits`, `group` and `keep` into the entry.
+
+Reading is offset-driven: a layer's blob is loaded once; the PackedMatrix of every matrix in it,
+fused, alias or plain, is an offset table onto that one tensor.  On disk the rows are in the
+reference's row-major order; `to_tiled()` reorders them for the decode kernel after the move to
+the GPU.
 """
 from __future__ import annotations
 
 import json
 import os
-from typing import Dict, List, Optional, Tuple
+from collections import Counter
+from typing import Dict, Iterator, List, Optional, Tuple
 
 import numpy as np
 import torch
@@ -22,67 +30,164 @@ from . import format as F
 
 FORMAT_NAME = "CBK1"
 FORMAT_VERSION = 1
+QKV_PARTS = ("q_proj", "k_proj", "v_proj")
+_ARRAYS = ("data", "row_off", "scale", "zero", "col_scale")
 
 
-def _entry(pm: F.PackedMatrix, blob_name: str, base: Dict[str, int]) -> dict:
-    arrays = {}
-    for name in ("data", "row_off", "scale", "zero", "col_scale"):
-        if name in pm.offs and (name != "col_scale" or pm.cs_rows):
-            arrays[name] = {"off": base[name], "bytes": int(pm.array(name).numel() * pm.array(name).element_size())}
-    e = {"K": pm.K, "N": pm.N, "G": pm.G, "layout": pm.layout, "layout_name": F.LAYOUT_NAME[pm.layout],
-         "cs_rows": pm.cs_rows, "n_survivors": pm.n_survivors, "stream_bytes": pm.stream_bytes(),
-         "bpw": pm.bpw(), "blob": blob_name, "arrays": arrays}
-    if pm.layout in (F.BLKC, F.DENSEB) or pm.group != 128:
-        e.update(bits=pm.bits, group=pm.group, keep=pm.keep)       # the extension layouts carry their parameters
-    if pm.cs_rows == 3:
-        e["cs_splits"] = list(pm.cs_splits)
+class _BlobWriter:
+    """Appends arrays to one `.bin`, each on a 256-byte boundary (pack_cobalt.py:389-411)."""
+
+    def __init__(self, path: str):
+        self.f = open(path, "wb")
+        self.pos = 0
+
+    def _pad(self):
+        pad = F._align(self.pos, F.ARR_ALIGN) - self.pos
+        self.f.write(b"\0" * pad)
+        self.pos += pad
+
+    def put(self, t: torch.Tensor) -> dict:
+        self._pad()
+        raw = t.contiguous().reshape(-1).view(torch.uint8).cpu().numpy().tobytes()
+        off = self.pos
+        self.f.write(raw)
+        self.pos += len(raw)
+        return {"off": off, "bytes": len(raw)}
+
+    def close(self) -> int:
+        self._pad()
+        self.f.close()
+        return self.pos
+
+
+def _entry(pm: F.PackedMatrix, bw: _BlobWriter) -> dict:
+    """Write the arrays of one matrix and return its manifest entry (pack_cobalt.py:414-434)."""
+    e = {"K": pm.K, "N": pm.N, "G": pm.G, "layout": pm.layout, "layout_name": F.LAYOUT_NAME[pm.layout], "arrays": {}}
+    for an in _ARRAYS:
+        if an in pm.offs and (an != "col_scale" or pm.cs_rows):
+            e["arrays"][an] = bw.put(pm.array(an))
+    e.update(cs_rows=pm.cs_rows, n_survivors=pm.n_survivors, n_zero_fixed=pm.n_zero_fixed,
+             stream_bytes=pm.stream_bytes(), bpw=pm.bpw())
+    if pm.layout in (F.BLKC, F.DENSEB):
+        e.update(bits=pm.bits, group=pm.group, keep=pm.keep)
     return e
 
 
-def write_container(path: str, layers: List[Dict[str, F.PackedMatrix]], config: Optional[dict] = None) -> dict:
-    """Write `layers[i][name]` (row-major PackedMatrix objects) as layer_%02d.bin + manifest.json.
-    Returns the manifest."""
+def _alias_entry(fused: F.PackedMatrix, fe: dict, fused_name: str, k0: int, k1: int, cs_row: int, bw: _BlobWriter) -> dict:
+    """Entry of rows [k0, k1) of a fused matrix: byte ranges inside the fused arrays, no bytes
+    written but the part's own column scale (pack_cobalt.py:474-503)."""
+    K, G = k1 - k0, fused.G
+    stride = fused.data_bytes // fused.K
+    fa = fe["arrays"]
+    e = {"K": K, "N": fused.N, "G": G, "layout": fused.layout, "layout_name": F.LAYOUT_NAME[fused.layout],
+         "arrays": {"data": {"off": fa["data"]["off"] + k0 * stride, "bytes": K * stride},
+                    "scale": {"off": fa["scale"]["off"] + k0 * G * 2, "bytes": K * G * 2},
+                    "zero": {"off": fa["zero"]["off"] + k0 * G, "bytes": K * G}}}
+    e["arrays"]["col_scale"] = bw.put(fused.array("col_scale").view(fused.cs_rows, fused.N)[cs_row])
+    share = (k1 - k0) / max(fused.K, 1)
+    e.update(cs_rows=1, n_survivors=int(round(fused.n_survivors * share)), n_zero_fixed=0, alias_of=fused_name,
+             alias_row_start=k0, stream_bytes=K * stride + K * G * 3)
+    e["bpw"] = 8.0 * e["stream_bytes"] / (K * fused.N)
+    if fused.layout in (F.BLKC, F.DENSEB):
+        e.update(bits=fused.bits, group=fused.group, keep=fused.keep)
+    return e
+
+
+def write_container(path: str, layers: List[Dict[str, F.PackedMatrix]], config: Optional[dict] = None,
+                    aliases: bool = True) -> dict:
+    """Write `layers[i][name]` (row-major PackedMatrix objects) as layer_%02d.bin + manifest.json in
+    the reference's schema (pack_cobalt.py:561-714) and return the manifest.  A matrix with three
+    column-scale rows is a row-concatenated q|k|v: its entry names the row ranges and, with
+    `aliases`, the layer also gets `alias_of` entries for the three parts."""
     os.makedirs(path, exist_ok=True)
-    manifest = {"format": FORMAT_NAME, "version": FORMAT_VERSION, "config": dict(config or {}), "layers": []}
+    every = [pm for mats in layers for pm in mats.values()]
+    lay = Counter(pm.layout for pm in every).most_common(1)[0][0] if every else F.BLK1632_4
+    bits = Counter(pm.bits for pm in every).most_common(1)[0][0] if every else 4
+    group = Counter(pm.group for pm in every).most_common(1)[0][0] if every else F.GROUP
+    manifest = {"format": FORMAT_NAME, "version": FORMAT_VERSION, "group_size": group, "bits": bits,
+                "layout": F.LAYOUT_NAME[lay], "embed_layout": None, "layout_override": {}, "bits_override": {},
+                "mixed_layout": any((pm.layout, pm.bits) != (lay, bits) for pm in every),
+                "fuse_gateup": any("gateup" in m for m in layers), "fuse_qkv": any("qkv" in m for m in layers),
+                "raw_dir": None, "raw_config": dict(config or {}), "layers": [], "embed": None, "lm_head": None,
+                "misc": None}
+    tot_p = tot_b = 0
     for li, mats in enumerate(layers):
-        blob_name = f"layer_{li:02d}.bin"
-        pos = 0
-        entries = {}
-        with open(os.path.join(path, blob_name), "wb") as f:
+        rec = {"file": f"layer_{li:02d}.bin", "matrices": {}, "norms": {}}
+        bw = _BlobWriter(os.path.join(path, rec["file"]))
+        try:
             for name, pm in mats.items():
                 if pm.tiled:
                     raise ValueError(f"{name}: write the row-major order; the tiled order is a load-time transform")
-                base = {}
-                for an in ("data", "row_off", "scale", "zero", "col_scale"):
-                    if an not in pm.offs or (an == "col_scale" and not pm.cs_rows):
-                        continue
-                    pad = F._align(pos, F.ARR_ALIGN) - pos
-                    f.write(b"\0" * pad)
-                    pos += pad
-                    raw = pm.array(an).contiguous().view(torch.uint8).cpu().numpy().tobytes()
-                    base[an] = pos
-                    f.write(raw)
-                    pos += len(raw)
-                entries[name] = _entry(pm, blob_name, base)
-            f.write(b"\0" * (F._align(pos, F.ARR_ALIGN) - pos))
-        manifest["layers"].append(entries)
+                e = _entry(pm, bw)
+                rec["matrices"][name] = e
+                tot_p += pm.K * pm.N
+                tot_b += e["stream_bytes"]
+                if pm.cs_rows == 3:
+                    s0, s1 = pm.cs_splits
+                    parts = tuple(pm.meta.get("fused_from", QKV_PARTS))
+                    rr = {parts[0]: [0, s0], parts[1]: [s0, s0 + s1], parts[2]: [s0 + s1, pm.K]}
+                    e.update(fused_from=list(parts), row_ranges=rr, cs_row_of={n: i for i, n in enumerate(parts)})
+                    if aliases and not any(n in mats for n in parts):
+                        for i, n in enumerate(parts):
+                            if rr[n][1] > rr[n][0]:
+                                rec["matrices"][n] = _alias_entry(pm, e, name, rr[n][0], rr[n][1], i, bw)
+        finally:
+            rec["bytes"] = bw.close()
+        manifest["layers"].append(rec)
+    manifest["bpw"] = {"params": tot_p, "packed_bytes": tot_b, "bpw_packed": 8.0 * tot_b / max(tot_p, 1)}
     with open(os.path.join(path, "manifest.json"), "w") as f:
         json.dump(manifest, f, indent=1)
     return manifest
 
 
+def layer_records(manifest: dict) -> Iterator[Tuple[int, str, Dict[str, dict]]]:
+    """(index, blob file name, {matrix name: entry}) for every layer of a manifest."""
+    for li, rec in enumerate(manifest.get("layers", [])):
+        if not isinstance(rec, dict) or "file" not in rec or "matrices" not in rec:
+            raise ValueError(f"layer {li} of the manifest has no `file` / `matrices`: not a {FORMAT_NAME} layer record")
+        yield li, rec["file"], rec["matrices"]
+
+
+def _cs_splits(e: dict) -> Tuple[int, int]:
+    """Row counts of the first two column-scale ranges of a q|k|v entry, from its `row_ranges` and
+    `cs_row_of` (pack_cobalt.py:638-640): rows [0, s0) use column-scale row 0, [s0, s0+s1) row 1,
+    the rest row 2."""
+    if int(e.get("cs_rows", 0)) != 3:
+        return (0, 0)
+    rr, co = e.get("row_ranges"), e.get("cs_row_of")
+    if not rr or not co:
+        raise ValueError("an entry with three column-scale rows needs row_ranges and cs_row_of")
+    order = sorted(rr, key=lambda n: co[n])
+    r = [tuple(int(v) for v in rr[n]) for n in order]
+    if len(r) != 3 or [co[n] for n in order] != [0, 1, 2] or r[0][0] != 0 or r[1][0] != r[0][1] or r[2][0] != r[1][1] \
+            or r[2][1] != int(e["K"]):
+        raise ValueError(f"row_ranges {rr} do not tile the rows 0..{e['K']} in column-scale order")
+    return (r[0][1] - r[0][0], r[1][1] - r[1][0])
+
+
 def matrix_from_entry(e: dict, blob: torch.Tensor) -> F.PackedMatrix:
-    """PackedMatrix view of one manifest entry onto its (already loaded) blob."""
+    """PackedMatrix view of one manifest entry onto its (already loaded) blob.  The `data` array of
+    an owning entry ends in the 64-byte tail; that of an `alias_of` entry is rows only."""
     layout = int(e["layout"])
     bits, group, keep = F.canon(layout, e.get("bits"), e.get("group"), e.get("keep"))
     a = e["arrays"]
     offs = {k: int(v["off"]) for k, v in a.items()}
     K, N = int(e["K"]), int(e["N"])
-    data_bytes = int(a["data"]["bytes"]) - F.BLOB_TAIL
-    zero = blob[offs["zero"]: offs["zero"] + int(a["zero"]["bytes"])]
-    flags = F.FLAG_ZERO_LE_128 if int(zero.max()) <= 128 else 0
-    return F.PackedMatrix(blob, offs, K, N, layout, bits, group, keep, int(e.get("cs_rows", 0)),
-                          tuple(e.get("cs_splits", (0, 0))), data_bytes, int(e.get("n_survivors", 0)), flags=flags)
+    data_bytes = int(a["data"]["bytes"]) - (0 if e.get("alias_of") else F.BLOB_TAIL)
+    for an, want in (("scale", K * (N // group) * 2), ("zero", K * (N // group))):
+        if int(a[an]["bytes"]) != want:
+            raise ValueError(f"{an} holds {a[an]['bytes']} bytes, want {want} for {K}x{N} with groups of {group}")
+    cs_rows = int(e.get("cs_rows", 0))
+    if cs_rows and int(a["col_scale"]["bytes"]) != cs_rows * N * 2:
+        raise ValueError(f"col_scale holds {a['col_scale']['bytes']} bytes, want {cs_rows} rows of {N} halves")
+    pm = F.PackedMatrix(blob, offs, K, N, layout, bits, group, keep, cs_rows, _cs_splits(e), data_bytes,
+                        int(e.get("n_survivors", 0)), int(e.get("n_zero_fixed", 0)))
+    pm.validate(deep=blob.device.type == "cpu")
+    if int(pm.array("zero").max()) <= 128:
+        pm.flags |= F.FLAG_ZERO_LE_128
+    if e.get("fused_from"):
+        pm.meta["fused_from"] = list(e["fused_from"])
+    return pm
 
 
 def read_container(path: str, device="cpu", include_aliases: bool = True) -> Tuple[dict, List[Dict[str, F.PackedMatrix]]]:
@@ -91,18 +196,17 @@ def read_container(path: str, device="cpu", include_aliases: bool = True) -> Tup
         manifest = json.load(f)
     if manifest.get("format") != FORMAT_NAME:
         raise ValueError(f"{path}: not a {FORMAT_NAME} directory")
-    blobs: Dict[str, torch.Tensor] = {}
     layers = []
-    for entries in manifest["layers"]:
+    for li, fn, entries in layer_records(manifest):
+        blob = torch.from_numpy(np.fromfile(os.path.join(path, fn), dtype=np.uint8)).to(device)
         mats = {}
         for name, e in entries.items():
             if e.get("alias_of") and not include_aliases:
                 continue
-            bn = e["blob"]
-            if bn not in blobs:
-                raw = np.fromfile(os.path.join(path, bn), dtype=np.uint8)
-                blobs[bn] = torch.from_numpy(raw).to(device)
-            mats[name] = matrix_from_entry(e, blobs[bn])
+            try:
+                mats[name] = matrix_from_entry(e, blob)
+            except (ValueError, KeyError) as err:
+                raise ValueError(f"{path}: layer {li} {name}: {err}") from err
         layers.append(mats)
     return manifest, layers
 
@@ -110,7 +214,7 @@ def read_container(path: str, device="cpu", include_aliases: bool = True) -> Tup
 def total_stream_bytes(manifest: dict) -> int:
     """Weight bytes one pass over the model streams; entries with `alias_of` are views into a
     fused matrix and are not counted twice (docs/FORMAT.md:146-151)."""
-    return sum(int(e["stream_bytes"]) for entries in manifest["layers"] for e in entries.values()
+    return sum(int(e["stream_bytes"]) for _, _, entries in layer_records(manifest) for e in entries.values()
                if not e.get("alias_of"))
 
 
@@ -128,25 +232,31 @@ def check_container(path: str, layers: int = 2, device="cpu", strict: bool = Tru
     if man.get("format") != FORMAT_NAME:
         problems.append(f"format is {man.get('format')!r}, want {FORMAT_NAME!r}")
     sizes: Dict[str, int] = {}
-    for li, entries in enumerate(man.get("layers", [])):
+    owned: List[dict] = []
+    try:
+        records = list(layer_records(man))
+    except ValueError as err:
+        problems.append(str(err))
+        records = []
+    for li, bn, entries in records:
+        bp = os.path.join(path, bn)
+        if not os.path.exists(bp):
+            problems.append(f"missing blob {bn}")
+            continue
+        sizes[bn] = os.path.getsize(bp)
         for name, e in entries.items():
-            bn = e["blob"]
-            bp = os.path.join(path, bn)
-            if bn not in sizes:
-                if not os.path.exists(bp):
-                    problems.append(f"missing blob {bn}")
-                    sizes[bn] = -1
-                else:
-                    sizes[bn] = os.path.getsize(bp)
-            if sizes[bn] < 0:
-                continue
+            alias = bool(e.get("alias_of"))
+            if alias and e["alias_of"] not in entries:
+                problems.append(f"{bn}:{name} is an alias of {e['alias_of']}, which the layer does not hold")
+            if not alias:
+                owned.append(e)
             for an, a in e["arrays"].items():
-                if a["off"] % F.ARR_ALIGN:
+                # an alias points into the fused arrays, on a row boundary rather than an array boundary
+                if a["off"] % F.ARR_ALIGN and not (alias and an != "col_scale"):
                     problems.append(f"{bn}:{name}.{an} starts at {a['off']}, not on a {F.ARR_ALIGN}-byte boundary")
                 if a["off"] + a["bytes"] > sizes[bn]:
                     problems.append(f"{bn}:{name}.{an} runs past the blob ({a['off']}+{a['bytes']} > {sizes[bn]})")
-    rep["blob_bytes"] = sum(v for v in sizes.values() if v > 0)
-    owned = [e for entries in man.get("layers", []) for e in entries.values() if not e.get("alias_of")]
+    rep["blob_bytes"] = sum(sizes.values())
     params = sum(e["K"] * e["N"] for e in owned)
     if params:
         rep["bpw"] = 8.0 * sum(e["stream_bytes"] for e in owned) / params
@@ -155,7 +265,11 @@ def check_container(path: str, layers: int = 2, device="cpu", strict: bool = Tru
             problems.append(f"bytes per weight recompute to {rep['bpw']:.6f}, the entries say {want:.6f}")
     if not problems:
         on_gpu = torch.device(device).type == "cuda"
-        _, mats_by_layer = read_container(path, device=device, include_aliases=False)
+        try:
+            _, mats_by_layer = read_container(path, device=device, include_aliases=False)
+        except ValueError as err:
+            problems.append(str(err))
+            mats_by_layer = []
         for li, mats in enumerate(mats_by_layer[:layers]):
             for name, pm in mats.items():
                 info = {"layout": F.LAYOUT_NAME[pm.layout], "shape": [pm.K, pm.N]}

@@ -281,6 +281,59 @@ class PackedMatrix:
             return v.view(torch.int32)
         return v
 
+    def validate(self, deep: bool = False) -> "PackedMatrix":
+        """Raise ValueError unless the integers describe arrays that lie inside the image and agree
+        with each other: the checks a kernel launch relies on, made where a description enters from
+        outside (a manifest entry, a state dict).  `deep` also reads the row offsets of a
+        variable-length matrix (a device-to-host copy when the image is on a GPU)."""
+        def bad(msg):
+            raise ValueError(f"packed matrix {self.K}x{self.N} {LAYOUT_NAME.get(self.layout, self.layout)}: {msg}")
+        if self.blob.dtype != torch.uint8 or self.blob.dim() != 1:
+            bad("the image is not a flat uint8 tensor")
+        if self.layout not in LAYOUT_NAME or self.layout == BF16:
+            bad("unknown layout")
+        try:
+            want = canon(self.layout, self.bits, self.group, self.keep)
+        except (ValueError, TypeError) as e:
+            bad(str(e))
+        if (self.bits, self.group, self.keep) != want:
+            bad(f"bits/group/keep {(self.bits, self.group, self.keep)} do not fit the layout (want {want})")
+        if self.K < 1 or self.N < 1 or self.N % GROUP:
+            bad(f"K >= 1 and N a positive multiple of {GROUP} are required")
+        if not 0 <= self.cs_rows <= 3:
+            bad(f"cs_rows {self.cs_rows} outside 0..3")
+        if self.cs_rows == 3:
+            s0, s1 = self.cs_splits
+            if s0 < 0 or s1 < 0 or s0 + s1 > self.K:
+                bad(f"row ranges {self.cs_splits} of the three column-scale rows do not fit K")
+        sparse = self.layout in _SPARSE
+        if sparse and self.tiled:
+            bad("a variable-length layout cannot be in tiled order")
+        if self.data_bytes < 0:
+            bad("negative data_bytes")
+        if not sparse:
+            st = row_stride(self.layout, self.N, self.bits, self.group, self.keep or None)
+            if self.data_bytes != self._krows() * st:
+                bad(f"data_bytes {self.data_bytes} is not rows x stride = {self._krows()} x {st}")
+        need = ["data", "scale", "zero"] + (["row_off"] if sparse else []) + (["col_scale"] if self.cs_rows else [])
+        align = {"data": 16, "scale": 4, "zero": 4, "col_scale": 16, "row_off": 4}     # what the library asks of the pointers
+        kr, n = self._krows(), self.blob.numel()
+        size = {"data": self.data_bytes + (TILED_TAIL if self.tiled else BLOB_TAIL), "scale": kr * self.G * 2,
+                "zero": kr * self.G, "col_scale": self.cs_rows * self.N * 2, "row_off": (self.K + 1) * 4}
+        for name in need:
+            if name not in self.offs:
+                bad(f"no offset for the {name} array")
+            off = self.offs[name]
+            if off < 0 or off % align[name]:
+                bad(f"{name} starts at {off}, not on a {align[name]}-byte boundary")
+            if off + size[name] > n:
+                bad(f"{name} runs past the image ({off} + {size[name]} > {n})")
+        if sparse and deep:
+            ro = self.array("row_off").cpu().to(torch.int64)
+            if int(ro[0]) != 0 or bool((ro[1:] < ro[:-1]).any()) or bool((ro % 16 != 0).any()) or int(ro[-1]) > self.data_bytes:
+                bad("row offsets are not an increasing sequence of multiples of 16 from 0 to at most data_bytes")
+        return self
+
     def stream_bytes(self) -> int:
         """Weight bytes one pass streams: rows + scale + zero (pack_cobalt.py:431-433)."""
         return self.data_bytes + self._krows() * self.G * 3

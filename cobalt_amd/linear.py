@@ -79,7 +79,7 @@ class CobaltLinear(nn.Module):
         self.bias = nn.Parameter(bias.detach().clone(), requires_grad=False) if bias is not None else None
         self.meta = {}
         self._backend = "hip"
-        self.packed().desc()                                          # raises on an inconsistent description
+        self.packed()                                                 # raises on an inconsistent description
         return self
 
     @classmethod
@@ -121,7 +121,7 @@ class CobaltLinear(nn.Module):
             offs["col_scale"] = d["off_col_scale"]
         return F.PackedMatrix(self.blob, offs, d["K"], d["N"], d["layout"], d["bits"], d["group"], d["keep"],
                               d["cs_rows"], (d["cs_split0"], d["cs_split1"]), d["data_bytes"], d["n_survivors"],
-                              flags=d["flags"])
+                              flags=d["flags"]).validate()
 
     def _apply(self, fn, recurse=True):
         out = super()._apply(fn, recurse)

@@ -147,3 +147,41 @@ def test_check_container_on_the_gpu(tmp_path):
     assert q["finite"] and q["pruned_nonzero"] == 0 and q["zero_fraction"] >= 0.5
     assert rep["matrices"]["0:up_proj"]["block_survivors"] == [23, 23]
     assert "pruned_nonzero" not in rep["matrices"]["0:down_proj"] and rep["matrices"]["0:down_proj"]["finite"]
+
+
+def test_directory_written_by_the_reference_loads_and_runs():
+    """tests/golden/cbk1_dir was written by the reference's `pack_artifact` with fused qkv and
+    gate/up (tests/golden/make_container_vectors.py); cbk1_dir_expect.npz holds the reference's own
+    decode.  Loaded onto the GPU, every matrix (fused, alias, plain) dequantises bit for bit to
+    that decode, and the fused matrices multiply like their parts, through the row-major bytes as
+    read and through the tiled order."""
+    import hashlib
+    import os
+    from cobalt_amd import container as Ct, ops
+    gold = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    exp = np.load(os.path.join(gold, "cbk1_dir_expect.npz"))
+    man, layers = Ct.read_container(os.path.join(gold, "cbk1_dir"), device=DEV)
+    mats = layers[0]
+    W = {}
+    for name, pm in mats.items():
+        W[name] = ops.dequant(pm, torch.float32)
+        w = W[name].cpu().numpy() + np.float32(0.0)
+        assert np.array_equal(w[exp[f"{name}.rows"]], exp[f"{name}.values"] + np.float32(0.0)), name
+        assert hashlib.sha256(np.ascontiguousarray(w).tobytes()).hexdigest() == bytes(exp[f"{name}.sha256"]).decode(), name
+        if "alias_of" not in man["layers"][0]["matrices"][name]:
+            assert torch.equal(ops.dequant(pm.to_tiled(), torch.float32), W[name]), name
+    g = torch.Generator(device=DEV).manual_seed(3)
+    for M in (1, 3, 40):
+        x = torch.randn(M, 256, device=DEV, generator=g).half()
+        for fused in (mats["qkv"], mats["qkv"].to_tiled()):
+            y = ops.linear(fused, x, out_dtype=torch.float32)
+            parts = torch.cat([ops.linear(mats[n], x, out_dtype=torch.float32) for n in ("q_proj", "k_proj", "v_proj")], 1)
+            ref = x.double() @ W["qkv"].double().T
+            tol = 2e-5 if M < 8 else 2e-3
+            assert float((y.double() - ref).abs().max() / ref.abs().max()) < tol
+            assert float((parts.double() - ref).abs().max() / ref.abs().max()) < tol
+        gu = ops.linear(mats["gateup"].to_tiled(), x, out_dtype=torch.float32).double()
+        ref = x.double() @ W["gateup"].double().T
+        assert float((gu - ref).abs().max() / ref.abs().max()) < (2e-5 if M < 8 else 2e-3)
+    rep = Ct.check_container(os.path.join(gold, "cbk1_dir"), device=DEV)
+    assert rep["ok"] and rep["matrices"]["0:gateup"]["pruned_nonzero"] == 0

@@ -193,3 +193,34 @@ def test_state_dict_roundtrip_and_patch_model():
     assert done == ["0"] and net[0] is cl2
     with pytest.raises(TypeError):
         F.dtype_code(torch.float64)
+
+
+def test_packed_matrix_validate_refuses_descriptions_that_do_not_fit_the_image():
+    """A description from a state dict or a manifest is outside input: offsets past the image,
+    misaligned arrays, a byte count that is not rows x stride, row ranges beyond K, parameters the
+    layout does not take and row offsets that are not increasing multiples of 16 all raise."""
+    import dataclasses
+    pm = F.synth_packed(48, 256, F.BLK1632_4, seed=1)
+    assert pm.validate() is pm and pm.to_tiled().validate().tiled
+    for change in (dict(offs={**pm.offs, "scale": pm.blob.numel()}), dict(offs={**pm.offs, "data": 8}),
+                   dict(offs={k: v for k, v in pm.offs.items() if k != "zero"}), dict(data_bytes=pm.data_bytes - 96),
+                   dict(K=pm.K + 1), dict(cs_rows=4), dict(cs_rows=3, cs_splits=(40, 16)), dict(bits=3), dict(keep=8),
+                   dict(layout=4), dict(N=192), dict(blob=pm.blob[:-256])):
+        with pytest.raises(ValueError):
+            dataclasses.replace(pm, **change).validate()
+    import os
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "sparse_stream.npz"))
+    sp = F.from_arrays(z["c0_SPARSE4X_data"], z["c0_SPARSE4X_scale"], z["c0_SPARSE4X_zero"], None, 5, 256, F.SPARSE4X,
+                       row_off=z["c0_SPARSE4X_row_off"].astype(np.int32))
+    assert sp.validate(deep=True) is sp
+    ro = sp.array("row_off").clone()
+    ro[3] += 8
+    broken = sp.clone()
+    broken.array("row_off")[:] = ro
+    with pytest.raises(ValueError):
+        broken.validate(deep=True)
+    cl = CobaltLinear(pm)
+    meta = cl.cbk_meta.clone()
+    meta[12] = pm.blob.numel()                                         # off_scale past the image
+    with pytest.raises(ValueError):
+        CobaltLinear.from_state(pm.blob, meta)
