@@ -40,8 +40,11 @@ the reference's formula, their byte layout is defined here:
 Parity status: every function here is pinned by tests/test_oracle_*.py through hand
 vectors, the reference documentation's known answers, an independent per-position
 decoder and round trips, except where a docstring says "parity unpinned"; the zero-point
-repair and the variable-length layouts (SPARSE4, SPARSE4X, SPARSE4E) in addition by bytes and
-values the reference's own packer wrote (tests/golden/fix_zero_range.npz, sparse_stream.npz).
+repair, the variable-length layouts (SPARSE4, SPARSE4X, SPARSE4E), the fixed-stride layouts
+(DENSE4, DENSE8, BLK1632_4, BLK1632_6), the interleaved gate/up fusion with two column-scale
+rows and the row-concatenated q|k|v with three in addition by bytes and values the reference's
+own packer and decoder wrote (tests/golden/fix_zero_range.npz, sparse_stream.npz,
+fixed_stride.npz, cbk1_dir/ with cbk1_dir_expect.npz).
 """
 from __future__ import annotations
 
