@@ -22,6 +22,8 @@ int launch_gemm(const DMat&, const void*, int, int, int64_t, void*, int, int64_t
 int launch_gemm_big(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*, void*, size_t,
                     hipStream_t);
 size_t gemm_big_workspace(const DMat&, int M);
+int launch_pack(const DMat&, const void* mask, const void* q, const void* scale, const void* zero, int zero_f16,
+                int fix_zero, int* status, hipStream_t);
 // The 256 x 256 tile kernel takes every call of the fixed-stride layouts: below 256 activation
 // rows part of its token tile is padding, and it is still several times faster than the
 // 128 x 128 kernel, which decodes through the generic reader (14336 x 4096 at 64 rows: 54 us
@@ -231,6 +233,19 @@ int cbk_dequant(const cbk_desc* in, int row0, int nrows, int with_col_scale, voi
   if (row0 < 0 || nrows < 0 || row0 + nrows > m.K || ld_out < m.N) return CBK_ERR_SHAPE;
   if (out_dtype != CBK_F32 && out_dtype != CBK_F16 && out_dtype != CBK_BF16T) return CBK_ERR_DTYPE;
   return launch_dequant(m, row0, nrows, with_col_scale, out, out_dtype, ld_out, (hipStream_t)stream);
+}
+
+int cbk_pack(const cbk_desc* dst, const void* mask_bits, const void* q, const void* scale, const void* zero,
+             int zero_dtype, int fix_zero, int* status, void* stream) {
+  DMat m;
+  const int rc = to_dmat(dst, &m, true);
+  if (rc) return rc;
+  if (!q || !scale || !zero) return CBK_ERR_NULL;
+  if (zero_dtype != CBK_F16 && zero_dtype != CBK_U8) return CBK_ERR_DTYPE;
+  if (((uintptr_t)q & 15) || ((uintptr_t)mask_bits & 3) || ((uintptr_t)scale & 1) || ((uintptr_t)status & 3) ||
+      (zero_dtype == CBK_F16 && ((uintptr_t)zero & 1)))
+    return CBK_ERR_ALIGN;
+  return launch_pack(m, mask_bits, q, scale, zero, zero_dtype == CBK_F16, fix_zero != 0, status, (hipStream_t)stream);
 }
 
 int cbk_gemv_batch(int n, const cbk_desc* descs, const void* const* xs, const int64_t* ldxs, int x_dtype, int M,

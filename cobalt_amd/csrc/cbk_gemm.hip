@@ -5,9 +5,11 @@
 //
 // Numerics.  The weight tile is fp16(W_hat): the float32 value of the dequant formula,
 // rounded once to 11 significant bits (relative error <= 2^-12).  bf16 activations are
-// widened to fp16 exactly (8 significant bits fit; magnitudes above 65504 saturate), so a
-// bf16 call loses nothing on the activation side and carries the same 2^-12 weight rounding
-// as an fp16 call.  Feeding the bf16 matrix pipe instead would round W_hat to 8 bits
+// widened to fp16 exactly (8 significant bits fit), so a bf16 call loses nothing on the
+// activation side and carries the same 2^-12 weight rounding as an fp16 call.  A token whose
+// largest bf16 magnitude is beyond 2^15 is first divided by a power of two that brings it into
+// [2^14, 2^15) and its outputs are multiplied back: exact, and nothing saturates at fp16's
+// 65504.  Feeding the bf16 matrix pipe instead would round W_hat to 8 bits
 // (2^-9), which alone exceeds the 1e-3 relative-Frobenius budget of this layer; the f16 and
 // bf16 MFMA rates are identical on gfx950.
 //
@@ -39,6 +41,24 @@ __global__ __launch_bounds__(256) void gemm_kernel(DMat m, const uint16_t* __res
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
+  // ---- bf16 only: power-of-two scale per token, two threads scan one token's row
+  __shared__ float tok_scale[BT];
+  if (XDT == CBK_BF16T) {
+    const int row = tid >> 1, tok = t0 + row;
+    float mx = 0.f;
+    if (tok < M)
+      for (int c = (tid & 1) * 8; c < m.N; c += 16) {
+        const uint4 v = *(const uint4*)(x + (size_t)tok * ldx + c);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          mx = fmaxf(mx, fmaxf(fabsf(bf2f((uint16_t)(w[e] & 0xffffu))), fabsf(bf2f((uint16_t)(w[e] >> 16)))));
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 1));
+    tok_scale[row] = token_scale(mx);
+    __syncthreads();
+  }
+
   // this thread's weight block: row r0 + tid/2, 32-column block (c0/32 + tid%2)
   const int wrow = r0 + (tid >> 1);
   const bool wrow_ok = wrow < m.K;
@@ -56,10 +76,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(DMat m, const uint16_t* __res
       if (tok < M) v = *(const uint4*)(x + (size_t)tok * ldx + c0 + ch * 8);
       if (XDT == CBK_BF16T) {
         uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        const float inv = 1.f / tok_scale[row];                       // a power of two: exact
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          float lo = fminf(fmaxf(bf2f((uint16_t)(w[e] & 0xffffu)), -65504.f), 65504.f);
-          float hi = fminf(fmaxf(bf2f((uint16_t)(w[e] >> 16)), -65504.f), 65504.f);
+          const float lo = bf2f((uint16_t)(w[e] & 0xffffu)) * inv, hi = bf2f((uint16_t)(w[e] >> 16)) * inv;
           w[e] = (uint32_t)f2h(lo) | ((uint32_t)f2h(hi) << 16);
         }
         v = make_uint4(w[0], w[1], w[2], w[3]);
@@ -130,7 +150,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(DMat m, const uint16_t* __res
       for (int r = 0; r < 16; ++r) {
         const int tok = t0 + 64 * wt + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         if (tok >= M) continue;
-        const float v = acc[i][j][r] + bv;
+        const float ts = XDT == CBK_BF16T ? tok_scale[tok - t0] : 1.f;
+        const float v = acc[i][j][r] * ts + bv;
         const size_t o = (size_t)tok * ldy + k;
         if (ydt == CBK_F32) ((float*)y)[o] = v;
         else if (ydt == CBK_F16) ((uint16_t*)y)[o] = f2h(v);

@@ -7,9 +7,12 @@
 // dequantise the weights of stage s + 1 into the other buffer, and the activation tile is
 // copied there from global memory without passing through registers.
 //
-// Operands.  The activation side is X' = fp16(x * col_scale), written once per call into the
-// caller's workspace by a small elementwise kernel (bf16 inputs are widened exactly; the
-// product is rounded once to fp16, magnitudes above 65504 saturate).  The weight side is
+// Operands.  The activation side is X' = fp16(x * col_scale / s_m), written once per call into
+// the caller's workspace by a small row-wise kernel (bf16 inputs are widened exactly; the
+// product is rounded once to fp16).  s_m is 1 unless token m holds a product of magnitude 2^15
+// or more; then it is the power of two that brings the token's largest below 2^15, and the
+// epilogue multiplies the token's outputs by it, so nothing saturates at fp16's 65504 and the
+// scaling itself is exact.  The weight side is
 // fp16((q - zero) * scale) for a kept column and exactly 0 for a pruned one, so
 // Y = sum_j X'[m,j] * W'[k,j] carries two roundings of relative size 2^-12.  Feeding bf16
 // operands instead would round to 2^-9, which alone exceeds the 1e-3 relative-Frobenius
@@ -47,6 +50,8 @@ typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
 struct GbArgs {
   DMat m;
   const uint16_t* xp;      // X' fp16 [Mpad, Npad]
+  const float* row_scale;  // [Mpad] per X': power of two each of its rows was divided by
+  int rss;                 // elements between the row scales of two X'
   int M, Npad;
   void* y;
   int ydt;
@@ -107,7 +112,7 @@ __device__ inline uint4 bytes_to_halfs(uint32_t b0, uint32_t b1, h2_t s2) {
 // per element: the 256 accumulators make this straight-line code, and it has to stay small.
 template <int YDT, int kstep, int TI>                            // local row i is output column row0 + kstep * i
 __device__ inline void gb_epilogue(const GbArgs& a, v16f (&acc)[TI][4], uint8_t* smem, int lane, int wave, int tok0,
-                                   int row0) {
+                                   int row0, const float* rs) {   // rs: the row scales of this tile's X'
   constexpr int ESZ = YDT == CBK_F32 ? 4 : 2;
   constexpr int PITCH = 128 * ESZ + 16;                          // bytes per token row in LDS
   constexpr int EPP = 16 / ESZ, PPR = 128 / EPP;                 // elements per 16-byte piece, pieces per row
@@ -124,11 +129,14 @@ __device__ inline void gb_epilogue(const GbArgs& a, v16f (&acc)[TI][4], uint8_t*
   const bool vec_ok = ((a.ldy * ESZ) & 15) == 0 && (((uintptr_t)a.y) & 15) == 0;
 #pragma unroll
   for (int i = 0; i < TI; ++i) {
+    float ts[16];                                                  // token of register r: see above
+#pragma unroll
+    for (int r = 0; r < 16; ++r) ts[r] = rs[tok0 + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float v = acc[i][j][r] + bv[j];
+        const float v = acc[i][j][r] * ts[r] + bv[j];
         uint8_t* d = epl + (8 * (r >> 2) + (r & 3)) * PITCH + 32 * j * ESZ;
         if (YDT == CBK_F32) *(float*)d = v;
         else if (YDT == CBK_F16) *(uint16_t*)d = f2h(v);
@@ -472,17 +480,18 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
   __syncthreads();
 
   const int tok0 = t0 + 32 * TI * wt, row0 = r0 + kstep * 128 * wr;
+  const float* rs = a.row_scale + (size_t)xv * a.rss;
   if (SPLIT) {                                                    // float32 partial tile, no bias
     GbArgs b = a;
     b.y = a.part + (size_t)part * a.part_stride;
     b.ldy = a.part_ld;
     b.bias = nullptr;
-    gb_epilogue<CBK_F32, 1, TI>(b, acc, smem, lane, wave, tok0, row0);
+    gb_epilogue<CBK_F32, 1, TI>(b, acc, smem, lane, wave, tok0, row0, rs);
     return;
   }
-  if (a.ydt == CBK_F32) gb_epilogue<CBK_F32, kstep, TI>(a, acc, smem, lane, wave, tok0, row0);
-  else if (a.ydt == CBK_F16) gb_epilogue<CBK_F16, kstep, TI>(a, acc, smem, lane, wave, tok0, row0);
-  else gb_epilogue<CBK_BF16T, kstep, TI>(a, acc, smem, lane, wave, tok0, row0);
+  if (a.ydt == CBK_F32) gb_epilogue<CBK_F32, kstep, TI>(a, acc, smem, lane, wave, tok0, row0, rs);
+  else if (a.ydt == CBK_F16) gb_epilogue<CBK_F16, kstep, TI>(a, acc, smem, lane, wave, tok0, row0, rs);
+  else gb_epilogue<CBK_BF16T, kstep, TI>(a, acc, smem, lane, wave, tok0, row0, rs);
 }
 
 template <int BITS, int KEEP, int GRP, int PAR, int TI>

@@ -10,29 +10,59 @@ int launch_gemm_big_b3(const GbArgs&, int keep, int group, int blocks, hipStream
 int launch_gemm_big_b4(const GbArgs&, int keep, int group, int blocks, hipStream_t);
 int launch_gemm_big_b6(const GbArgs&, int blocks, hipStream_t);
 
-// ---- X' = fp16(x * col_scale), [Mpad, Npad] row-major; rows M..Mpad-1 and columns N..Npad-1 zero
-__global__ __launch_bounds__(256) void gemm_prep_kernel(const uint16_t* x, int64_t ldx, const uint16_t* cs, int xdt,
-                                                        int M, int Mpad, int N, int Npad, uint16_t* out) {
-  const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;     // one thread = 8 columns
-  const int n8 = Npad >> 3;
-  if (id >= (int64_t)Mpad * n8) return;
-  const int row = (int)(id / n8), c8 = (int)(id % n8);
-  if (row >= M || c8 * 8 >= N) { *(uint4*)(out + (size_t)row * Npad + c8 * 8) = make_uint4(0, 0, 0, 0); return; }
-  const uint4 v = *(const uint4*)(x + (size_t)row * ldx + c8 * 8);
-  uint4 c = make_uint4(0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u);
-  if (cs) c = *(const uint4*)(cs + c8 * 8);
+// ---- X' = fp16(x * col_scale / s_row), [Mpad, Npad] row-major, and s_row, one workgroup per row.
+// s_row is the power of two that brings the row's largest |x * col_scale| below 2^15 (1 for
+// nearly every row: only magnitudes beyond fp16's range need it); the GEMM kernel multiplies the
+// row's outputs by it.  Rows M..Mpad-1 and columns N..Npad-1 are zero.
+__device__ inline void prep8(const uint4 v, const uint4 c, int xdt, float (&a)[8]) {
   const uint32_t xw[4] = {v.x, v.y, v.z, v.w}, cw[4] = {c.x, c.y, c.z, c.w};
-  uint32_t o[4];
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    float a0, a1;
-    if (xdt == CBK_F16) { a0 = h2f((uint16_t)(xw[e] & 0xffffu)); a1 = h2f((uint16_t)(xw[e] >> 16)); }
-    else { a0 = bf2f((uint16_t)(xw[e] & 0xffffu)); a1 = bf2f((uint16_t)(xw[e] >> 16)); }
-    a0 *= h2f((uint16_t)(cw[e] & 0xffffu)); a1 *= h2f((uint16_t)(cw[e] >> 16));
-    a0 = fminf(fmaxf(a0, -65504.f), 65504.f); a1 = fminf(fmaxf(a1, -65504.f), 65504.f);
-    o[e] = (uint32_t)f2h(a0) | ((uint32_t)f2h(a1) << 16);
+    if (xdt == CBK_F16) { a[2 * e] = h2f((uint16_t)(xw[e] & 0xffffu)); a[2 * e + 1] = h2f((uint16_t)(xw[e] >> 16)); }
+    else { a[2 * e] = bf2f((uint16_t)(xw[e] & 0xffffu)); a[2 * e + 1] = bf2f((uint16_t)(xw[e] >> 16)); }
+    a[2 * e] *= h2f((uint16_t)(cw[e] & 0xffffu)); a[2 * e + 1] *= h2f((uint16_t)(cw[e] >> 16));
   }
-  *(uint4*)(out + (size_t)row * Npad + c8 * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+__global__ __launch_bounds__(256) void gemm_prep_kernel(const uint16_t* x, int64_t ldx, const uint16_t* cs, int xdt,
+                                                        int M, int N, int Npad, uint16_t* out, float* row_scale) {
+  __shared__ float red[4];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const int n8 = Npad >> 3, nv = N >> 3;                           // N is a multiple of 128
+  uint16_t* orow = out + (size_t)row * Npad;
+  if (row >= M) {
+    for (int c8 = tid; c8 < n8; c8 += 256) *(uint4*)(orow + c8 * 8) = make_uint4(0, 0, 0, 0);
+    if (tid == 0) row_scale[row] = 1.f;
+    return;
+  }
+  const uint16_t* xr = x + (size_t)row * ldx;
+  const uint4 one = make_uint4(0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u);
+  float mx = 0.f;
+  for (int c8 = tid; c8 < nv; c8 += 256) {
+    float a[8];
+    prep8(*(const uint4*)(xr + c8 * 8), cs ? *(const uint4*)(cs + c8 * 8) : one, xdt, a);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) mx = fmaxf(mx, fabsf(a[e]));
+  }
+#pragma unroll
+  for (int o = 32; o; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+  if ((tid & 63) == 0) red[tid >> 6] = mx;
+  __syncthreads();
+  const float s = token_scale(fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])));
+  const float inv = 1.f / s;                                       // a power of two: exact
+  if (tid == 0) row_scale[row] = s;
+  for (int c8 = tid; c8 < n8; c8 += 256) {
+    uint4 o4 = make_uint4(0, 0, 0, 0);
+    if (c8 < nv) {
+      float a[8];
+      prep8(*(const uint4*)(xr + c8 * 8), cs ? *(const uint4*)(cs + c8 * 8) : one, xdt, a);
+      uint32_t o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = (uint32_t)f2h(a[2 * e] * inv) | ((uint32_t)f2h(a[2 * e + 1] * inv) << 16);
+      o4 = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+    *(uint4*)(orow + c8 * 8) = o4;
+  }
 }
 
 static inline int gb_npad(int N) { return (N + 255) / 256 * 256; }
@@ -109,7 +139,9 @@ static inline size_t gb_kpad(int K) { return (size_t)(K + 7) / 8 * 8; }
 
 size_t gemm_big_workspace(const DMat& m, int M) {
   const size_t T = 64 * gb_ti(M), mpad = (size_t)(M + T - 1) / T * T;
-  size_t b = ((m.cs_rows > 1 ? m.cs_rows : 1) * mpad * gb_npad(m.N) * 2 + 255) & ~(size_t)255;
+  const size_t nv = m.cs_rows > 1 ? m.cs_rows : 1;
+  size_t b = (nv * mpad * gb_npad(m.N) * 2 + 255) & ~(size_t)255;     // X', one per col_scale vector
+  b += (nv * mpad * 4 + 255) & ~(size_t)255;                          // and its row scales
   const int ns = gb_nsplit(m, M);
   if (ns > 1) b += ((size_t)ns * M * gb_kpad(m.K) * 4 + 255) & ~(size_t)255;
   return b;
@@ -126,15 +158,19 @@ int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, v
   const int T = 64 * gb_ti(M);
   const int Mpad = (M + T - 1) / T * T;
   const int Npad = gb_npad(m.N);
-  const int64_t items = (int64_t)Mpad * (Npad / 8);
   const int par = m.cs_rows == 2 ? 1 : 0;
-  for (int v = 0; v < (m.cs_rows > 1 ? m.cs_rows : 1); ++v)       // one X' per col_scale vector
-    hipLaunchKernelGGL(gemm_prep_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st,
-                       (const uint16_t*)x, ldx, m.cs ? m.cs + (size_t)v * m.N : nullptr, xdt, M, Mpad, m.N, Npad,
-                       (uint16_t*)ws + (size_t)v * Mpad * Npad);
+  const int nv = m.cs_rows > 1 ? m.cs_rows : 1;
+  const size_t xbytes = ((size_t)nv * Mpad * Npad * 2 + 255) & ~(size_t)255;
+  const size_t sbytes = ((size_t)nv * Mpad * 4 + 255) & ~(size_t)255;
+  float* row_scale = (float*)((uint8_t*)ws + xbytes);
+  for (int v = 0; v < nv; ++v)                                     // one X' per col_scale vector
+    hipLaunchKernelGGL(gemm_prep_kernel, dim3((unsigned)Mpad), dim3(256), 0, st,
+                       (const uint16_t*)x, ldx, m.cs ? m.cs + (size_t)v * m.N : nullptr, xdt, M, m.N, Npad,
+                       (uint16_t*)ws + (size_t)v * Mpad * Npad, row_scale + (size_t)v * Mpad);
   GbArgs a;
   a.m = m; a.xp = (const uint16_t*)ws; a.M = M; a.Npad = Npad; a.y = y; a.ydt = ydt; a.ldy = ldy; a.bias = bias;
   a.par = par; a.xps = (size_t)Mpad * Npad;
+  a.row_scale = row_scale; a.rss = Mpad;
   a.vs0 = m.cs_rows == 3 ? m.cs_split0 : 0x7fffffff;
   a.vs1 = m.cs_rows == 3 ? m.cs_split0 + m.cs_split1 : 0x7fffffff;
   const int nst_all = Npad / GB_K;
@@ -142,7 +178,7 @@ int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, v
   a.nst_part = ((nst_all + a.nsplit - 1) / a.nsplit + 3) / 4 * 4;
   a.part_ld = (int64_t)gb_kpad(m.K);
   a.part_stride = (size_t)M * gb_kpad(m.K);
-  a.part = (float*)((uint8_t*)ws + (((size_t)(m.cs_rows > 1 ? m.cs_rows : 1) * Mpad * Npad * 2 + 255) & ~(size_t)255));
+  a.part = (float*)((uint8_t*)ws + xbytes + sbytes);
   a.ti = gb_ti(M);
   a.tiles_t = (M + T - 1) / T;
   a.tiles_r = par ? 2 * ((m.K + 2 * GB_R - 1) / (2 * GB_R)) : (m.K + GB_R - 1) / GB_R;

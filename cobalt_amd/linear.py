@@ -36,18 +36,28 @@ class CobaltLinear(nn.Module):
              o["scale"], o["zero"], o.get("col_scale", -1), packed.n_survivors, packed.flags], dtype=torch.int64)
 
     # ---- construction ------------------------------------------------------------------
+    @staticmethod
+    def _pack(mask, q, scale, zero, col_scale, layout, bits, group, keep, cs_splits=(0, 0), tiled=False) -> F.PackedMatrix:
+        """RAW arrays on a GPU are packed there by the library's kernel, others by the torch packer."""
+        if q.is_cuda:
+            from . import ops
+            return ops.pack_raw(mask, q, scale, zero, col_scale, layout, bits, group, keep, cs_splits=cs_splits, tiled=tiled)
+        pm = F.pack_raw(mask, q, scale, zero, col_scale, layout, bits, group, keep, cs_splits=cs_splits)
+        return pm.to_tiled() if tiled else pm
+
     @classmethod
     def from_raw(cls, mask, q, scale, zero, col_scale, bias=None, layout=F.BLK1632_4, bits=None, group=None,
-                 keep=None, meta=None, cs_splits=(0, 0)) -> "CobaltLinear":
+                 keep=None, meta=None, cs_splits=(0, 0), tiled=False) -> "CobaltLinear":
         """From the RAW per-matrix schema `<name>.{mask,q,scale,zero,col_scale}`
-        (src/cobaltkernel/pack_cobalt.py:3-11)."""
-        return cls(F.pack_raw(mask, q, scale, zero, col_scale, layout, bits, group, keep, cs_splits=cs_splits),
-                   bias, meta)
+        (src/cobaltkernel/pack_cobalt.py:3-11); `tiled` asks for the decode kernel's byte order
+        at once instead of the reference's row-major order."""
+        return cls(cls._pack(mask, q, scale, zero, col_scale, layout, bits, group, keep, cs_splits, tiled), bias, meta)
 
     @classmethod
     def from_linear(cls, linear: nn.Module, X_cal: Optional[torch.Tensor] = None, H: Optional[torch.Tensor] = None,
                     sparsity: float = 0.5, bits: int = 4, group: int = 128, beta: float = 0.5, mask_block: int = 32,
-                    meta=None, raw_sink: Optional[dict] = None, raw_name: Optional[str] = None) -> "CobaltLinear":
+                    meta=None, raw_sink: Optional[dict] = None, raw_name: Optional[str] = None,
+                    tiled: bool = False) -> "CobaltLinear":
         """Compress an `nn.Linear` with CoBALT and pack it (the role of `CPRLinear.from_linear`,
         sinq/cprlinear.py:128-171, with the pipeline of src/cobaltkernel/quantize_cobalt.py:424-443).
         Calibration comes as activations X_cal [tokens, in_features] or as H = X^T X; without
@@ -61,7 +71,8 @@ class CobaltLinear(nn.Module):
         if raw_sink is not None:
             raw_sink[raw_name or "linear"] = {f: raw[f].detach().cpu() for f in ("mask", "q", "scale", "zero", "col_scale")}
         layout, keep = Cp.layout_for(sparsity, bits, group, mask_block)
-        pm = F.pack_raw(raw["mask"], raw["q"], raw["scale"], raw["zero"], raw["col_scale"], layout, bits, group, keep)
+        pm = cls._pack(raw["mask"], raw["q"], raw["scale"], raw["zero"], raw["col_scale"], layout, bits, group, keep,
+                       tiled=tiled)
         bias = linear.bias.data if getattr(linear, "bias", None) is not None else None
         return cls(pm, bias, meta)
 
@@ -106,8 +117,8 @@ class CobaltLinear(nn.Module):
             else:
                 layout = F.DENSE4 if (bits, group) == (4, 128) else F.DENSEB
         bias = m.bias.data if getattr(m, "bias", None) is not None else None
-        pm = F.pack_raw(F.pack_mask(keepm), torch.round(W_q.float()).to(torch.int32), scales.reshape(K, G),
-                        zeros.reshape(K, G), m.scale2.reshape(-1, N), layout, bits, group, c0 if uniform else None)
+        pm = cls._pack(F.pack_mask(keepm), torch.round(W_q.float()).to(torch.int32), scales.reshape(K, G),
+                       zeros.reshape(K, G), m.scale2.reshape(-1, N), layout, bits, group, c0 if uniform else None)
         return cls(pm, bias, getattr(m, "meta", None))
 
     # ---- the packed view ----------------------------------------------------------------

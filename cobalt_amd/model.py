@@ -147,7 +147,8 @@ def compress_model(model: nn.Module, calib_ids: Optional[torch.Tensor] = None, s
                     mb = 0 if sp == 0.0 else mask_block
                     new = CobaltLinear.from_linear(lin, H=H, sparsity=sp, bits=nb, group=group, beta=beta,
                                                    mask_block=mb, raw_sink=raws if raw_out else None,
-                                                   raw_name=lname.rsplit(".", 1)[1])
+                                                   raw_name=lname.rsplit(".", 1)[1],
+                                                   tiled=device_order and lin.weight.is_cuda)
                     rstats[lname.rsplit(".", 1)[1]] = dict(bits=nb, sparsity_target=sp, mask_block=mb)
                     if device_order and new.blob.is_cuda:
                         new.to_device_order()
@@ -219,7 +220,7 @@ def _fuse_group(blk: nn.Module, names: Sequence[str], interleave: bool, device_o
     mods = [_sub(blk, n) for n in names]
     if not all(isinstance(m, CobaltLinear) for m in mods):
         return False
-    pms = [m.packed() for m in mods]
+    pms = [m.packed().to_rowmajor() for m in mods]
     try:
         fused_pm = F.fuse_rows(pms, interleave=interleave)
     except ValueError:
@@ -355,7 +356,8 @@ def install_raw_artifact(model: nn.Module, path: str, device_order: bool = True,
             t = {f: raw[f].to(dev) for f in container.RAW_FIELDS}
             bias = lin.bias.data if getattr(lin, "bias", None) is not None else None
             new = CobaltLinear.from_raw(t["mask"], t["q"], t["scale"], t["zero"], t["col_scale"], bias=bias,
-                                        layout=layout, bits=nb, group=grp, keep=keep)
+                                        layout=layout, bits=nb, group=grp, keep=keep,
+                                        tiled=device_order and dev.type == "cuda")
             if device_order and new.blob.is_cuda:
                 new.to_device_order()
             setattr(_sub(blk, lname.rsplit(".", 1)[0]), short, new)

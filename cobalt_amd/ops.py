@@ -171,3 +171,63 @@ def gemv_batch(pms, xs, biases=None, out_dtype=None):
                           _stream_ptr(pms[0].blob.device))
     _lib.check(rc, "cbk_gemv_batch")
     return [y.reshape(*x.shape[:-1], pm.K) for y, x, pm in zip(ys, xs, pms)]
+
+
+def pack_raw(mask_bits, q, scale, zero, col_scale, layout, bits=None, group=None, keep=None, fix_zero=True,
+             cs_splits=(0, 0), tiled=True) -> PackedMatrix:
+    """RAW arrays on the GPU -> PackedMatrix on the GPU, written by the library's packing kernel
+    (rows, scale, zero point, and the re-derivation of zero points that are off the code grid,
+    src/cobaltkernel/pack_cobalt.py:55-87), in the tiled order the decode kernel streams (`tiled`)
+    or the reference's row-major order.  Same arguments and same bytes as `format.pack_raw`
+    (which is torch and runs anywhere)."""
+    from . import format as F
+    bits, group, kpb = F.canon(layout, bits, group, keep)
+    if layout in F._SPARSE:
+        raise NotImplementedError("the variable-length SPARSE4* layouts are read, not produced, by this package")
+    if q.device.type != "cuda":
+        raise _lib.CbkError("ops.pack_raw packs on the GPU; use format.pack_raw for tensors on the CPU")
+    dev = q.device
+    K, N = q.shape
+    if N % 128 or N % group:
+        raise ValueError(f"N={N} must be a multiple of 128 and of the group size")
+    G = N // group
+    nl = (1 << bits) - 1
+    mb = None if mask_bits is None else mask_bits.to(dev).reshape(K, N // 8).contiguous()
+    q8 = (q if q.dtype == torch.uint8 else q.clamp(0, 255).to(torch.uint8)).contiguous()
+    sc16 = scale.to(dev).to(torch.float16).reshape(K, G).contiguous()
+    z = zero.to(dev).reshape(K, G)
+    z = (z if z.dtype == torch.uint8 else z.to(torch.float16)).contiguous()
+    stride = F.row_stride(layout, N, bits, group, kpb or None)
+    kr = F._align(K, 16) if tiled else K
+    sizes = {"data": kr * stride + (F.TILED_TAIL if tiled else F.BLOB_TAIL), "scale": kr * G * 2, "zero": kr * G}
+    cs = None
+    if col_scale is not None:
+        cs = col_scale.to(dev).to(torch.float16).reshape(-1, N).contiguous()
+        sizes["col_scale"] = cs.numel() * 2
+    offs, pos = {}, 0
+    for name, n in sizes.items():
+        pos = F._align(pos, F.ARR_ALIGN)
+        offs[name] = pos
+        pos += n
+    blob = torch.zeros(F._align(pos, F.ARR_ALIGN), dtype=torch.uint8, device=dev)
+    if cs is not None:
+        blob[offs["col_scale"]: offs["col_scale"] + sizes["col_scale"]] = cs.reshape(-1).view(torch.uint8)
+    if layout in F._DENSE:
+        n_surv = K * N if mb is None else int(F.unpack_mask(mb, N).sum())
+    else:
+        n_surv = K * (N // F.BLOCK) * kpb
+    pm = PackedMatrix(blob, offs, K, N, layout, bits, group, kpb, 0 if cs is None else cs.shape[0], tuple(cs_splits),
+                      kr * stride, n_surv, 0, (F.FLAG_TILED16 if tiled else 0))
+    status = torch.zeros(2, dtype=torch.int32, device=dev)
+    d = pm.desc()
+    rc = _lib.lib().cbk_pack(ctypes.byref(d), mb.data_ptr() if mb is not None else None, q8.data_ptr(), sc16.data_ptr(),
+                             z.data_ptr(), 3 if z.dtype == torch.uint8 else F.F16, int(bool(fix_zero)), status.data_ptr(),
+                             _stream_ptr(dev))
+    _lib.check(rc, "cbk_pack")
+    wrong, pm.n_zero_fixed = (int(v) for v in status.tolist())
+    if wrong:
+        raise ValueError(f"{F.LAYOUT_NAME[layout]} needs exactly {kpb} survivors in every aligned block of "
+                         f"{F.BLOCK} columns; the mask has a block with another count")
+    if int(pm.array("zero").max()) <= 128:
+        pm.flags |= F.FLAG_ZERO_LE_128
+    return pm.validate()

@@ -46,7 +46,7 @@ enum cbk_layout {
 #define CBK_FLAG_ZERO_LE_128 1
 #define CBK_FLAG_TILED16 2
 
-enum cbk_dtype { CBK_F32 = 0, CBK_F16 = 1, CBK_BF16T = 2 };
+enum cbk_dtype { CBK_F32 = 0, CBK_F16 = 1, CBK_BF16T = 2, CBK_U8 = 3 /* cbk_pack's zero points only */ };
 
 /* gate activations of cbk_linear_act (cobalt_gemm.cuh:216-220: tanh-GELU, x / (1 + exp(-x))) */
 enum cbk_act { CBK_ACT_GELU_TANH = 0, CBK_ACT_SILU = 1 };
@@ -127,8 +127,9 @@ size_t cbk_stream_bytes(const cbk_desc* d, size_t sparse_data_bytes);
 /* Device scratch needed by cbk_gemv / cbk_gemm / cbk_linear for M activation rows (0 for the
  * decode kernels; the prefill kernel keeps its pre-scaled fp16 activations there:
  * ceil(M/256)*256 * ceil(N/256)*256 * 2 bytes per col_scale vector, i.e. times cs_rows for a
- * fused matrix, plus float32 partial outputs when the library splits the column range of a
- * launch that would not fill the chip).  Ask, do not compute.  256-byte aligned. */
+ * fused matrix, one float32 scale per activation row and col_scale vector, plus float32 partial
+ * outputs when the library splits the column range of a launch that would not fill the chip).
+ * Ask, do not compute.  256-byte aligned. */
 size_t cbk_workspace_bytes(const cbk_desc* d, int M);
 
 /* Rows [row0, row0+nrows) of W_hat -> out[nrows, ld_out] in out_dtype, bit-exact float32
@@ -137,6 +138,26 @@ size_t cbk_workspace_bytes(const cbk_desc* d, int M);
  * harness entry `dequant_rows`, test_gemv.cu:223-235). */
 int cbk_dequant(const cbk_desc* d, int row0, int nrows, int with_col_scale,
                 void* out, int out_dtype, int64_t ld_out, void* stream);
+
+/* RAW arrays -> the data, scale and zero arrays of the CBK1 image `dst` describes (dst->data,
+ * dst->scale, dst->zero point at device memory of the sizes the layout implies; CBK_FLAG_TILED16
+ * in dst->flags selects the 16-row tiled order, else the reference's row-major order; padding
+ * and tail bytes are written as zero).  Fixed-stride layouts only.
+ *   mask_bits  uint8 [K, N/8], LSB first, 1 = survivor; NULL = nothing pruned
+ *   q          uint8 [K, N] codes (clamped to [0, 2^bits) here)
+ *   scale      fp16  [K, N/group]
+ *   zero       [K, N/group], zero_dtype CBK_F16 (an integer value, rounded here) or CBK_U8
+ * A dense layout stores the group's zero point at a pruned column; a bitmap layout stores the
+ * survivors of each 32-column block in column order.  With fix_zero != 0 a group whose zero
+ * point lies outside [0, 2^bits - 1] gets scale, zero point and codes re-derived from the hull of
+ * its dequantised survivors and 0, as _fix_zero_range does (src/cobaltkernel/pack_cobalt.py:55-87),
+ * in correctly rounded float32 steps in that function's order.  `status`, if given, is two device
+ * ints the caller has set to 0: status[0] becomes 1 when a block does not hold exactly `keep`
+ * survivors (the bytes written for such a block are then meaningless), status[1] counts the
+ * groups re-derived.  The byte layouts are the ones `pack_matrix` (pack_cobalt.py:98-250) writes
+ * with torch operations. */
+int cbk_pack(const cbk_desc* dst, const void* mask_bits, const void* q, const void* scale,
+             const void* zero, int zero_dtype, int fix_zero, int* status, void* stream);
 
 /* Decode path, 1 <= M <= 16: y[m, k] = sum_j x[m, j] * W_hat[k, j] (+ bias[k]).
  * x is [M, ldx] fp16 or bf16, y is [M, ldy] in y_dtype (f32 / f16 / bf16), bias is NULL or

@@ -1,0 +1,164 @@
+"""The producer side on the GPU: the library's packing kernel (RAW arrays -> CBK1 rows, row-major
+or tiled) bit for bit against the oracle's packer, the torch packer and the reference's own bytes;
+the compressor run on the GPU against the reference's vectors."""
+import os
+import time
+
+import numpy as np
+import pytest
+import torch
+
+from cobalt_amd import compress as C, format as F, ops
+from cobalt_amd.linear import CobaltLinear
+from oracle import cbk_ref as R
+from helpers import FIXED_CASES, case_id, make_raw, oracle_pack
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _t(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def _same_arrays(a, b, names=("data", "scale", "zero", "col_scale")):
+    for n in names:
+        if n == "col_scale" and not a.cs_rows:
+            continue
+        assert torch.equal(a.array(n), b.array(n)), n
+
+
+@pytest.mark.parametrize("case", FIXED_CASES, ids=case_id)
+def test_hip_packer_writes_the_oracle_bytes(case):
+    """K not a multiple of 16 (tile padding), N an odd and an even multiple of 128 (a last
+    128-column unit), zero points off the grid (the repair path), two column-scale rows."""
+    layout, bits, group, keep = case
+    for K, N, seed in ((37, 384, 1), (48, 1024, 2)):
+        raw = make_raw(case, K, N, seed=seed)
+        zero = raw["zero"].astype(np.float16).copy()
+        if seed == 1:
+            zero[3, 0] = -2.0
+            zero[5, -1] = float((1 << bits) + 1)
+        pk = R.pack_matrix(raw["mask"], raw["q"], raw["scale"], zero, layout,
+                           **({"bits": bits, "group": group, "keep_per_block": keep or None} if layout in (F.BLKC, F.DENSEB) else {}))
+        cs = np.stack([raw["col_scale"], raw["col_scale"][::-1]], 0) if seed == 2 else raw["col_scale"]
+        host = (raw["mask"], raw["q"], raw["scale"], zero, cs)
+        args = tuple(_t(a) for a in host) + (layout, bits, group, keep or None)
+        # the torch packer on the CPU: its divisions on the GPU round differently in the zero-point repair
+        torch_pm = F.pack_raw(*[torch.from_numpy(np.ascontiguousarray(a)) for a in host], layout, bits, group, keep or None).to(DEV)
+        rm = ops.pack_raw(*args, tiled=False)
+        a, c = rm.array("data").cpu().numpy(), pk["data"]
+        assert np.array_equal(a, c), f"row bytes against the oracle: {np.nonzero(a != c)[0][:8]} of {(a != c).sum()}, K={K} N={N}"
+        assert np.array_equal(rm.array("scale").cpu().numpy().reshape(K, -1), pk["scale"])
+        assert np.array_equal(rm.array("zero").cpu().numpy().reshape(K, -1), pk["zero"])
+        assert (rm.offs, rm.data_bytes, rm.flags, rm.n_survivors, rm.n_zero_fixed, rm.cs_rows) == \
+               (torch_pm.offs, torch_pm.data_bytes, torch_pm.flags, torch_pm.n_survivors, torch_pm.n_zero_fixed, torch_pm.cs_rows)
+        assert torch.equal(rm.blob, torch_pm.blob)
+        tl, want = ops.pack_raw(*args, tiled=True), torch_pm.to_tiled()
+        assert (tl.offs, tl.data_bytes, tl.flags) == (want.offs, want.data_bytes, want.flags) and torch.equal(tl.blob, want.blob)
+        W = R.dequant(pk, K, N, layout, col_scale=np.asarray(cs, np.float16).reshape(-1, N),
+                      **({"bits": bits, "group": group, "keep_per_block": keep or None} if layout in (F.BLKC, F.DENSEB) else {}))
+        assert np.array_equal(ops.dequant(tl, torch.float32).cpu().numpy() + np.float32(0), W + np.float32(0))
+
+
+def test_hip_packer_writes_the_reference_bytes():
+    """tests/golden/fixed_stride.npz: bytes of the reference's own pack_matrix."""
+    fix = np.load(os.path.join(GOLD, "fixed_stride.npz"))
+    for name in ("DENSE4", "DENSE8", "BLK1632_4", "BLK1632_6"):
+        p = name + "_"
+        pm = ops.pack_raw(_t(fix[p + "mask"]), _t(fix[p + "q"]), _t(fix[p + "scale_in"]), _t(fix[p + "zero_in"]),
+                          _t(fix[p + "col_scale"]), getattr(F, name), tiled=False)
+        assert np.array_equal(pm.array("data").cpu().numpy(), fix[p + "data"]), name
+        assert np.array_equal(pm.array("scale").cpu().numpy().reshape(6, -1), fix[p + "scale"])
+        assert np.array_equal(pm.array("zero").cpu().numpy().reshape(6, -1), fix[p + "zero"])
+        assert pm.n_zero_fixed == 2
+
+
+def test_hip_packer_refuses_a_mask_with_the_wrong_block_count():
+    raw = make_raw((F.BLK1632_4, 4, 128, 16), 32, 256, seed=3)
+    mask = raw["mask"].copy()
+    mask[7, 4] ^= 1
+    with pytest.raises(ValueError):
+        ops.pack_raw(_t(mask), _t(raw["q"]), _t(raw["scale"]), _t(raw["zero"]), _t(raw["col_scale"]), F.BLK1632_4)
+    with pytest.raises(Exception):
+        ops.pack_raw(torch.from_numpy(mask), torch.from_numpy(raw["q"]), torch.from_numpy(raw["scale"]),
+                     torch.from_numpy(raw["zero"]), None, F.BLK1632_4)                       # CPU tensors: not this packer
+
+
+def test_modules_built_on_the_gpu_use_the_hip_packer_and_match_the_cpu_build():
+    raw = make_raw((F.BLK1632_4, 4, 128, 16), 80, 512, seed=4)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a))
+    cpu = CobaltLinear.from_raw(t(raw["mask"]), t(raw["q"]), t(raw["scale"]), t(raw["zero"]), t(raw["col_scale"]))
+    gpu = CobaltLinear.from_raw(*[_t(raw[k]) for k in ("mask", "q", "scale", "zero", "col_scale")])
+    assert gpu.blob.is_cuda and torch.equal(gpu.blob.cpu(), cpu.blob) and torch.equal(gpu.cbk_meta, cpu.cbk_meta)
+    tiled = CobaltLinear.from_raw(*[_t(raw[k]) for k in ("mask", "q", "scale", "zero", "col_scale")], tiled=True)
+    assert tiled._pm().tiled and torch.equal(tiled.blob.cpu(), cpu._pm().to_tiled().blob)
+
+
+def _golden_case(fix, i):
+    p = f"c{i}_"
+    c = {k[len(p):]: fix[k] for k in fix.files if k.startswith(p)}
+    X = c["X"].astype(np.float64)
+    c["H"] = (X.T @ X).astype(np.float32)
+    sp, beta, bits, group, mb = c["cfg"]
+    c["args"] = (float(sp), float(beta), int(bits), int(group), int(mb))
+    c["keep"] = np.unpackbits(c["mask"], axis=-1, bitorder="little")[:, : c["W"].shape[1]].astype(bool)
+    return c
+
+
+def test_compressor_on_the_gpu_against_the_reference_vectors():
+    """`cobalt_compress` with its tensors on the GPU against the vectors the reference's
+    `cobalt_math.cobalt_quantize` wrote (tests/golden/cobalt_quantize.npz; bit for bit on the CPU).
+    The mask is computed before any matrix product and has to be identical.  The Cholesky inverse
+    and the compensation matmul are other libraries on the GPU and sum in another order, so what
+    follows them agrees to rounding: scales and column scales within one fp16 step, zero points
+    within one code, at most 2 % of the codes differ and never by more than one, and the
+    reconstruction error equals the reference's to 1e-3 of itself."""
+    fix = np.load(os.path.join(GOLD, "cobalt_quantize.npz"))
+    for i in range(4):
+        c = _golden_case(fix, i)
+        sp, beta, bits, group, mb = c["args"]
+        r = C.cobalt_compress(_t(c["W"]), _t(c["H"]), sp, bits, group, beta, mb)
+        assert r["q"].is_cuda
+        keep = c["keep"]
+        assert np.array_equal(r["mask"].cpu().numpy(), c["mask"]), f"case {i}: mask bytes"
+        q = r["q"].cpu().numpy().astype(np.int32)
+        dq = np.abs(q[keep] - c["q"][keep].astype(np.int32))
+        assert dq.max() <= 1 and (dq != 0).mean() <= 0.02, f"case {i}: {(dq != 0).mean():.4f} of the codes differ, max {dq.max()}"
+        assert (q[~keep] == 0).all()
+        for name in ("scale", "col_scale"):
+            a, b = r[name].cpu().numpy().astype(np.float32), c[name].astype(np.float16).astype(np.float32)
+            assert np.all(np.abs(a - b) <= np.abs(b) * 2.0 ** -10), f"case {i}: {name}"
+            assert (a != b).mean() <= 0.05, f"case {i}: {name} differs in {(a != b).mean():.3f} of its entries"
+        assert np.abs(r["zero"].float().cpu().numpy() - c["zero"]).max() <= 1
+        W_hat = r["W_hat"].cpu().numpy()
+        rel = np.linalg.norm(W_hat - c["W"]) / np.linalg.norm(c["W"])
+        assert abs(rel - float(c["relerr"])) < 1e-3 * float(c["relerr"]), f"case {i}: {rel} vs {float(c['relerr'])}"
+
+
+def test_compress_and_pack_one_full_size_matrix_on_the_gpu():
+    """14336 x 4096 (the reference's bandwidth-test shape) through the whole producer path on the
+    GPU: Hessian, compressor, HIP packer; the packed module multiplies like its own W_hat.  Prints
+    the seconds each stage took."""
+    K, N = 14336, 4096
+    g = torch.Generator(device=DEV).manual_seed(0)
+    W = torch.randn(K, N, device=DEV, generator=g) * 0.02
+    X = torch.randn(2048, N, device=DEV, generator=g)
+    torch.cuda.synchronize(); t0 = time.time()
+    H = C.hessian(X)
+    raw = C.cobalt_compress(W, H, 0.5, 4, 128, 0.5, 32)
+    torch.cuda.synchronize(); t1 = time.time()
+    pm = ops.pack_raw(raw["mask"], raw["q"], raw["scale"], raw["zero"], raw["col_scale"], F.BLK1632_4, tiled=True)
+    torch.cuda.synchronize(); t2 = time.time()
+    ref = F.pack_raw(*[raw[k].cpu() for k in ("mask", "q", "scale", "zero", "col_scale")], F.BLK1632_4).to_tiled()
+    t3 = time.time()
+    print(f"\n14336x4096: compress {t1 - t0:.3f} s, HIP pack {t2 - t1:.4f} s ({pm.n_zero_fixed} zero points re-derived), "
+          f"torch pack + tile on the CPU {t3 - t2:.2f} s", flush=True)
+    assert torch.equal(pm.blob.cpu(), ref.blob) and abs(pm.bpw() - 3.1875) < 1e-9 and pm.n_zero_fixed == ref.n_zero_fixed
+    x = torch.randn(2, N, device=DEV, generator=g).half()
+    y = ops.gemv(pm, x, out_dtype=torch.float32).double()
+    want = x.double() @ ops.dequant(pm, torch.float32).double().T
+    assert float((y - want).abs().max() / want.abs().max()) < 2e-5
+    loose = x.double() @ raw["W_hat"].double().T                        # scales not yet rounded to fp16
+    assert float((y - loose).norm() / loose.norm()) < 1e-3

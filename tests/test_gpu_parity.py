@@ -507,6 +507,36 @@ def test_gemm_bias_dtype_and_prune_zero():
     assert torch.equal(ops.gemm(pm, x0.to(DEV), out_dtype=torch.float32), ops.gemm(pm, xh.to(DEV), out_dtype=torch.float32))
 
 
+def test_gemm_activations_beyond_fp16_range():
+    """bf16 activations (and fp16 ones under a column scale) whose products leave fp16's range:
+    the prefill kernels feed the fp16 matrix pipe, so such a token is scaled by a power of two on
+    the way in and back on the way out.  Tokens 1, 70 and 299 carry values up to 1e36 / 1e9 / 7e4;
+    every token, large or not, meets the float64 product to the usual tolerance, and the small
+    tokens give the same bits as in a call without the large ones."""
+    case = (F.BLK1632_4, 4, 128, 16)
+    K, N, M = 512, 1024, 300
+    for cs_rows, splits in ((1, (0, 0)), (2, (0, 0)), (3, (256, 128)), (3, (40, 24))):
+        pm, W = _fused(case, K, N, cs_rows, splits, seed=31 + cs_rows + splits[0], tiled=splits[0] % 16 == 0)
+        for dtype, big in ((torch.bfloat16, (1.0e36, 1.0e9, 7.0e4)), (torch.float16, (6.5e4, 4.0e4, 3.3e4))):
+            x = acts(M, N, dtype, seed=M + cs_rows)
+            small = ops.gemm(pm, x.to(DEV), out_dtype=torch.float32)
+            xb = x.clone()
+            for tok, top in zip((1, 70, 299), big):
+                xb[tok] = (x[tok].float() * (top / float(x[tok].float().abs().max()))).to(dtype)
+                xb[tok, 5] = top
+            y = ops.gemm(pm, xb.to(DEV), out_dtype=torch.float32)
+            assert bool(torch.isfinite(y).all())
+            ref = R.forward_ref(W, _np(xb))
+            for tok in (0, 1, 70, 150, 299):
+                err = rel_fro(_np(y[tok:tok + 1]), ref[tok:tok + 1])
+                assert err < TOL, f"cs_rows={cs_rows} splits={splits} {dtype} token {tok}: {err}"
+            keep = [t for t in range(M) if t not in (1, 70, 299)]
+            assert torch.equal(y[keep], small[keep])
+            y64 = ops.gemm(pm, xb[:40].to(DEV), out_dtype=torch.float32)          # the 64-token instantiation
+            small64 = ops.gemm(pm, x[:40].to(DEV), out_dtype=torch.float32)
+            assert rel_fro(_np(y64[1:2]), ref[1:2]) < TOL and torch.equal(y64[2:], small64[2:])
+
+
 # ------------------------------------------------------------------ the module seam
 def test_cobalt_linear_forward_matches_reference_module_math():
     K, N = 256, 1024
