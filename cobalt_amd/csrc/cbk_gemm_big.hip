@@ -24,44 +24,77 @@ __device__ inline void prep8(const uint4 v, const uint4 c, int xdt, float (&a)[8
   }
 }
 
-__global__ __launch_bounds__(256) void gemm_prep_kernel(const uint16_t* x, int64_t ldx, const uint16_t* cs, int xdt,
-                                                        int M, int N, int Npad, uint16_t* out, float* row_scale) {
-  __shared__ float red[4];
+// One workgroup of 1024 threads per row.  CH: 16-byte pieces of the row a thread keeps in
+// registers between the two passes (the row is read from memory once); 0 = any row length, the
+// second pass reads the row again.
+template <int CH>
+__global__ __launch_bounds__(1024) void gemm_prep_kernel(const uint16_t* x, int64_t ldx, const uint16_t* cs, int xdt,
+                                                         int M, int N, int Npad, uint16_t* out, float* row_scale) {
+  constexpr int T = 1024;
+  __shared__ float red[T / 64];
   const int row = blockIdx.x, tid = threadIdx.x;
   const int n8 = Npad >> 3, nv = N >> 3;                           // N is a multiple of 128
   uint16_t* orow = out + (size_t)row * Npad;
   if (row >= M) {
-    for (int c8 = tid; c8 < n8; c8 += 256) *(uint4*)(orow + c8 * 8) = make_uint4(0, 0, 0, 0);
+    for (int c8 = tid; c8 < n8; c8 += T) *(uint4*)(orow + c8 * 8) = make_uint4(0, 0, 0, 0);
     if (tid == 0) row_scale[row] = 1.f;
     return;
   }
   const uint16_t* xr = x + (size_t)row * ldx;
   const uint4 one = make_uint4(0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u);
+  uint4 xv[CH ? CH : 1], cv[CH ? CH : 1];
   float mx = 0.f;
-  for (int c8 = tid; c8 < nv; c8 += 256) {
-    float a[8];
-    prep8(*(const uint4*)(xr + c8 * 8), cs ? *(const uint4*)(cs + c8 * 8) : one, xdt, a);
+  if (CH) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) mx = fmaxf(mx, fabsf(a[e]));
+    for (int i = 0; i < CH; ++i) {
+      const int c8 = tid + T * i;
+      xv[i] = make_uint4(0, 0, 0, 0); cv[i] = one;
+      if (c8 < nv) { xv[i] = *(const uint4*)(xr + c8 * 8); if (cs) cv[i] = *(const uint4*)(cs + c8 * 8); }
+    }
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      float a[8];
+      prep8(xv[i], cv[i], xdt, a);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) mx = fmaxf(mx, fabsf(a[e]));
+    }
+  } else {
+    for (int c8 = tid; c8 < nv; c8 += T) {
+      float a[8];
+      prep8(*(const uint4*)(xr + c8 * 8), cs ? *(const uint4*)(cs + c8 * 8) : one, xdt, a);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) mx = fmaxf(mx, fabsf(a[e]));
+    }
   }
 #pragma unroll
   for (int o = 32; o; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
   if ((tid & 63) == 0) red[tid >> 6] = mx;
   __syncthreads();
-  const float s = token_scale(fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])));
+  float all = red[0];
+#pragma unroll
+  for (int w = 1; w < T / 64; ++w) all = fmaxf(all, red[w]);
+  const float s = token_scale(all);
   const float inv = 1.f / s;                                       // a power of two: exact
   if (tid == 0) row_scale[row] = s;
-  for (int c8 = tid; c8 < n8; c8 += 256) {
+  auto emit = [&](int c8, const uint4 xq, const uint4 cq) {
     uint4 o4 = make_uint4(0, 0, 0, 0);
     if (c8 < nv) {
       float a[8];
-      prep8(*(const uint4*)(xr + c8 * 8), cs ? *(const uint4*)(cs + c8 * 8) : one, xdt, a);
+      prep8(xq, cq, xdt, a);
       uint32_t o[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) o[e] = (uint32_t)f2h(a[2 * e] * inv) | ((uint32_t)f2h(a[2 * e + 1] * inv) << 16);
       o4 = make_uint4(o[0], o[1], o[2], o[3]);
     }
     *(uint4*)(orow + c8 * 8) = o4;
+  };
+  if (CH) {
+#pragma unroll
+    for (int i = 0; i < CH; ++i)
+      if (tid + T * i < n8) emit(tid + T * i, xv[i], cv[i]);
+  } else {
+    for (int c8 = tid; c8 < n8; c8 += T)
+      emit(c8, c8 < nv ? *(const uint4*)(xr + c8 * 8) : one, (cs && c8 < nv) ? *(const uint4*)(cs + c8 * 8) : one);
   }
 }
 
@@ -163,8 +196,10 @@ int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, v
   const size_t xbytes = ((size_t)nv * Mpad * Npad * 2 + 255) & ~(size_t)255;
   const size_t sbytes = ((size_t)nv * Mpad * 4 + 255) & ~(size_t)255;
   float* row_scale = (float*)((uint8_t*)ws + xbytes);
+  const int ch = (Npad / 8 + 1023) / 1024;                         // 16-byte pieces per thread of the row kernel
+  auto prep = ch <= 1 ? gemm_prep_kernel<1> : ch <= 3 ? gemm_prep_kernel<3> : gemm_prep_kernel<0>;
   for (int v = 0; v < nv; ++v)                                     // one X' per col_scale vector
-    hipLaunchKernelGGL(gemm_prep_kernel, dim3((unsigned)Mpad), dim3(256), 0, st,
+    hipLaunchKernelGGL(prep, dim3((unsigned)Mpad), dim3(1024), 0, st,
                        (const uint16_t*)x, ldx, m.cs ? m.cs + (size_t)v * m.N : nullptr, xdt, M, m.N, Npad,
                        (uint16_t*)ws + (size_t)v * Mpad * Npad, row_scale + (size_t)v * Mpad);
   GbArgs a;
