@@ -67,7 +67,7 @@ MIN_WARM_MS = 50.0
 # the same counters read for a device-to-device copy of known size), keyed by
 # (workload, launch grouping, M).  Stored figures from the runs summarised under profiles/, not
 # counters read during a bench run.
-MEASURED_TRAFFIC = {("mistral7b", "phase", 1): 22311131}
+MEASURED_TRAFFIC = {("mistral7b", "phase", 1): 22311131, ("gemma27b", "phase", 1): 43089816}
 
 
 def algorithmic_bytes(pm, M, e_x=2, e_y=2):
