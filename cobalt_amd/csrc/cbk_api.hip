@@ -272,10 +272,10 @@ int cbk_gemv_batch(int n, const cbk_desc* descs, const void* const* xs, const in
     if (k == 0 || nc + k > kMaxBatch) { fast = false; continue; }
     for (int j = 0; j < k; ++j) calls[nc++] = sub[j];
   }
-  // activation rows per pass: as many (4, 2 or 1) as the digits of every matrix fit in LDS with;
-  // a gate/up matrix stages two scaled copies of every activation row
+  // activation rows per pass: as many (8, 4, 2 or 1) as the kernel takes for every matrix and
+  // their digits fit in LDS with; a gate/up matrix stages two scaled copies of every activation row
   const int vm = fast && calls[0].par ? 2 : 1;
-  int mc = M * vm >= 4 ? 4 / vm : (M * vm >= 2 ? 2 / vm : 1);
+  int mc = M * vm > 4 ? 8 / vm : (M * vm >= 4 ? 4 / vm : (M * vm >= 2 ? 2 / vm : 1));
   for (int i = 0; fast && i < nc; ++i) {
     while (mc > 1 && !gemv_fast_takes(calls[i].m, mc * vm) && gemv_fast_takes(calls[i].m, vm)) mc >>= 1;
     fast = gemv_fast_takes(calls[i].m, vm) && gemv_same_config(calls[0].m, calls[i].m) && calls[i].par == calls[0].par;

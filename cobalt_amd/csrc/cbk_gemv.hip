@@ -22,10 +22,10 @@
 // to 16 column parts and the (tile, part) items are dealt round-robin to the wavefronts.  There
 // is no barrier per tile: the partial sums of a tile meet in an LDS slot and the wavefront that
 // arrives last adds them in part order, so results are run-to-run identical.
-// For 2 <= M <= 4 the headline configurations put the lane quarters on the four 32-column
+// For 2 <= M <= 8 the headline configurations put the lane quarters on the four 32-column
 // blocks of one chunk instead of on four chunks (see block_split_capable below), so that
-// every MFMA serves all activation rows; sums are formed in the same order as for M = 1, so
-// a row's result does not depend on M.
+// every MFMA serves four activation rows (M = 5..8: two MFMAs per decoded fragment, one weight
+// pass); sums are formed in the same order as for M = 1, so a row's result does not depend on M.
 // The activation digits and the byte-permute selector table live in LDS for the whole launch.
 //
 // Expansion of the bitmap.  For one mask byte (8 columns, r survivors before it in its
@@ -53,7 +53,7 @@ constexpr int CNT_SLOTS = 64;                 // most reduction slots (arrival c
 constexpr int CNT_BYTES = CNT_SLOTS * 4;       // at a fixed place: zeroed before the arguments are read
 constexpr int X_LDS_BUDGET = 112 * 1024;      // activation digits: M * 3 * N bytes (of 160 KB LDS)
 constexpr int NDIG = 3;                       // int8 digits per activation
-constexpr int GV_MAX_M = 4;
+constexpr int GV_MAX_M = 8;                     // 5..8 only in the block-per-quarter arrangement
 constexpr int GV_MAX_BATCH = 8;               // matrices per launch
 
 // ------------------------------------------------------------------ kernel configuration
@@ -292,7 +292,9 @@ struct Loads {
 template <int BITS, int KEEP, int GRP, int MP>
 __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
   using C = Cfg<BITS, KEEP, GRP, MP>;
-  constexpr bool QB = MP == 4 && block_split_capable(BITS, KEEP, GRP);
+  constexpr bool QB = (MP == 4 || MP == 8) && block_split_capable(BITS, KEEP, GRP);
+  constexpr int NG = MP == 8 ? 2 : 1;                  // groups of four activation rows, one MFMA each per fragment
+  static_assert(MP <= 4 || QB, "more than four activation rows need the block-per-quarter arrangement");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // in a scalar register: positions are scalar work
@@ -503,13 +505,23 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
         uint32_t zs[4];                                             // zero | scale << 8 of the groups 4S .. 4S+3
 #pragma unroll
         for (int c = 0; c < 4; ++c) zs[c] = (uint32_t)__shfl((int)cur.zraw, wr + 16 * c, 64);
-        const bool a_on = a_dig < NDIG && a_m < h.M;
-        const uint32_t a_base = xq_off + (uint32_t)((a_m * NDIG + a_dig) * N + kq * 32);
-        const int dm = kq < h.M ? kq : 0;                           // the activation row this quarter sums
+        // row group g holds activation rows 4g .. 4g+3: its A operand, and in the result lane
+        // quarter kq the three digit sums of activation row 4g + kq
+        bool a_on[NG];
+        uint32_t a_base[NG];
+        int dm[NG];                                                 // the activation rows this quarter sums
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+          a_on[g] = a_dig < NDIG && a_m + 4 * g < h.M;
+          a_base[g] = xq_off + (uint32_t)(((a_m + 4 * g) * NDIG + a_dig) * N + kq * 32);
+          dm[g] = kq + 4 * g < h.M ? kq + 4 * g : 0;
+        }
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
           const int chunk = 4 * S + c;
-          const uint32_t aaddr = (a_on && chunk < NCH) ? a_base + (uint32_t)chunk * 128u : z_off;
+          uint32_t aaddr[NG];
+#pragma unroll
+          for (int g = 0; g < NG; ++g) aaddr[g] = (a_on[g] && chunk < NCH) ? a_base[g] + (uint32_t)chunk * 128u : z_off;
           uint32_t rkc[4];
           uint2 selc[4];
           fetch_selectors<C>(cur.mk[c], lut, l16, rkc, selc);
@@ -518,21 +530,29 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
           for (int k = 0; k < C::NW; ++k) st[k] = cur.raw[c * C::NW + k];
           const uint32_t z = zs[c] & 0xFFu;
           const uint32_t nz = 0x80808080u - z * 0x01010101u;
-          v4i acc = (v4i){0, 0, 0, 0};
+          v4i acc[NG];
+#pragma unroll
+          for (int g = 0; g < NG; ++g) acc[g] = (v4i){0, 0, 0, 0};
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
-            const v4i av = *(const v4i*)(smem + aaddr + 16 * half);
             uint32_t bfrag[4];
             decode_half<C, BITS>(st, rkc, selc, nz, half, bfrag);
             const v4i bv = (v4i){(int)bfrag[0], (int)bfrag[1], (int)bfrag[2], (int)bfrag[3]};
-            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bv, acc, 0, 0, 0);
-            asm("s_nop 1" : "+v"(acc));                             // see the other decode path
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+              const v4i av = *(const v4i*)(smem + aaddr[g] + 16 * half);
+              acc[g] = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bv, acc[g], 0, 0, 0);
+              asm("s_nop 1" : "+v"(acc[g]));                        // see the other decode path
+            }
           }
           // the 128 columns of group `chunk` are complete: rows 4 kq .. 4 kq + 2 of the result
-          // are the three digit sums of activation row kq
-          const float dl = delta[dm * (NCH + 4) + chunk];           // 0 past the last chunk
-          const float f = fmaf((float)(acc[0] * 256 + acc[1]), 256.f, (float)acc[2]);
-          ysum[c] = fmaf(f, h2f((uint16_t)(zs[c] >> 8)) * dl, ysum[c]);
+          // are the three digit sums of activation row 4g + kq
+#pragma unroll
+          for (int g = 0; g < NG; ++g) {
+            const float dl = delta[dm[g] * (NCH + 4) + chunk];      // 0 past the last chunk
+            const float f = fmaf((float)(acc[g][0] * 256 + acc[g][1]), 256.f, (float)acc[g][2]);
+            ysum[4 * g + c] = fmaf(f, h2f((uint16_t)(zs[c] >> 8)) * dl, ysum[4 * g + c]);
+          }
         }
       } else
       {
@@ -597,7 +617,11 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       for (int p = 0; p < MP; ++p) {
         // quarter kq holds activation row kq, one running sum per chunk position; added in the
         // order of the other decode path, so a row's result does not depend on M
-        if (QB) { part_sum[p] = (ysum[0] + ysum[MP > 1 ? 1 : 0]) + (ysum[MP > 2 ? 2 : 0] + ysum[MP > 3 ? 3 : 0]); continue; }
+        if (QB) {                                                   // (p: row group; only p < NG is used)
+          const int q = p < NG ? 4 * p : 0;
+          part_sum[p] = (ysum[q] + ysum[q + 1]) + (ysum[q + 2] + ysum[q + 3]);
+          continue;
+        }
         part_sum[p] = quarter_sum(ysum[p]);
       }
       auto store = [&](int om, int r, float v) {
@@ -616,7 +640,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       };
       if (SK == 1) {
         if (QB) {
-          if (kq < h.M) store(kq, wr, part_sum[0]);
+#pragma unroll
+          for (int g = 0; g < NG; ++g)
+            if (kq + 4 * g < h.M) store(kq + 4 * g, wr, part_sum[g]);
         } else {
 #pragma unroll
           for (int p = 0; p < MP; ++p)
@@ -628,7 +654,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
         const int slot = tl & (h.nslot - 1);
         float* rs = red + (size_t)slot * h.sk_cap * h.M * 16;
         if (QB) {
-          if (kq < h.M) rs[(part * h.M + kq) * 16 + wr] = part_sum[0];
+#pragma unroll
+          for (int g = 0; g < NG; ++g)
+            if (kq + 4 * g < h.M) rs[(part * h.M + kq + 4 * g) * 16 + wr] = part_sum[g];
         } else {
 #pragma unroll
           for (int p = 0; p < MP; ++p)
@@ -642,18 +670,22 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
         old = __builtin_amdgcn_readfirstlane(old);                 // lane 0 holds it, and every lane is active here
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
         if (old == SK - 1) {                                      // uniform over the wave
-          // quarter kq finishes activation row kq (M <= 4); the partial sums are read four at a
-          // time (parts past SK re-read the last one and do not count) and added in part order
-          if (kq < h.M) {
-            float v = 0.f;
-            for (int j0 = 0; j0 < SK; j0 += 4) {
-              float pv[4];
+          // the partial sums are read four at a time (parts past SK re-read the last one and do
+          // not count) and added in part order
 #pragma unroll
-              for (int j = 0; j < 4; ++j) pv[j] = rs[((j0 + j < SK ? j0 + j : SK - 1) * h.M + kq) * 16 + wr];
+          for (int g = 0; g < NG; ++g) {
+            const int am = kq + 4 * g;                              // quarter kq finishes activation rows kq and 4 + kq
+            if (am < h.M) {
+              float v = 0.f;
+              for (int j0 = 0; j0 < SK; j0 += 4) {
+                float pv[4];
 #pragma unroll
-              for (int j = 0; j < 4; ++j) v += j0 + j < SK ? pv[j] : 0.f;
+                for (int j = 0; j < 4; ++j) pv[j] = rs[((j0 + j < SK ? j0 + j : SK - 1) * h.M + am) * 16 + wr];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v += j0 + j < SK ? pv[j] : 0.f;
+              }
+              store(am, wr, v);
             }
-            store(kq, wr, v);
           }
           if (lane == 0) cnt[slot] = 0;
         }
@@ -681,6 +713,7 @@ static bool keep_supported(int keep) { return keep == 10 || keep == 16 || keep =
 
 bool gemv_fast_takes(const DMat& m, int M) {
   if (M < 1 || M > GV_MAX_M) return false;
+  if (M > 4 && !block_split_capable(m.bits, family_of(m.layout) == FAM_DENSE ? 0 : m.keep, m.group)) return false;
   if (m.cs_rows == 3) return false;                              // the caller splits q|k|v into its ranges
   if (!(m.flags & CBK_FLAG_ZERO_LE_128)) return false;
   const int fam = family_of(m.layout);
@@ -731,6 +764,11 @@ static int launch_mp(const GvBatch& b, size_t lds, int blocks, hipStream_t st) {
   if constexpr (!block_split_capable(BITS, KEEP, GRP)) {
     if (b.h.M == 2) return launch_cfg<BITS, KEEP, GRP, 2>(b, lds, blocks, st);
   }
+  if constexpr (block_split_capable(BITS, KEEP, GRP)) {
+    if (b.h.M > 4) return launch_cfg<BITS, KEEP, GRP, 8>(b, lds, blocks, st);
+  } else {
+    if (b.h.M > 4) return CBK_ERR_UNSUPPORTED;
+  }
   return launch_cfg<BITS, KEEP, GRP, 4>(b, lds, blocks, st);
 }
 
@@ -752,7 +790,8 @@ static int launch_keep(const GvBatch& b, size_t lds, int blocks, hipStream_t st)
   }
 }
 
-// All matrices share one kernel configuration (checked by the caller) and 1 <= M <= 4.
+// All matrices share one kernel configuration (checked by the caller) and 1 <= M <= 8 (more than
+// four only where gemv_fast_takes says so).
 int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, void* workspace, size_t ws_bytes,
                            hipStream_t st) {
   if (n < 1 || n > GV_MAX_BATCH) return CBK_ERR_SHAPE;

@@ -236,6 +236,25 @@ def test_gemv_rows_are_independent_of_batch_and_run_to_run_identical():
     assert torch.equal(ops.gemv(pm, x, out_dtype=torch.float32), y4)
 
 
+@pytest.mark.parametrize("case", [(F.BLK1632_4, 4, 128, 16), (F.DENSE4, 4, 128, 0), (F.BLKC, 2, 128, 16), (F.BLKC, 4, 64, 23)], ids=case_id)
+def test_gemv_five_to_eight_rows_equal_single_rows(case):
+    """M = 5..8: where the arrangement allows it (group 128, block code streams of whole bytes) and
+    the digits of all rows fit in LDS (N = 4096) the weights are streamed once, with two matrix
+    instructions per decoded fragment; elsewhere in passes of at most four rows.  Either way row m
+    of the result is the M = 1 result of row m bit for bit, also for a gate/up matrix (two scaled
+    copies of every activation row), with a bias, and for a tile split into parts."""
+    for (K, N, cs_rows) in ((80, 4096, 1), (48, 4096, 2), (16, 14336, 1)):
+        pm, W = _fused(case, K, N, cs_rows, (0, 0), seed=K + N + cs_rows, tiled=True)
+        bias = acts(1, K, torch.float32, seed=2)[0].to(DEV)
+        for M in (5, 6, 7, 8):
+            x = acts(M, N, torch.bfloat16, seed=10 * M).to(DEV)
+            y = ops.gemv(pm, x, bias=bias, out_dtype=torch.float32)
+            assert rel_fro(_np(y), R.forward_ref(W, _np(x)) + _np(bias)[None, :]) < TOL
+            for i in range(M):
+                assert torch.equal(ops.gemv(pm, x[i:i + 1], bias=bias, out_dtype=torch.float32)[0], y[i]), (K, N, cs_rows, M, i)
+            assert torch.equal(ops.gemv(pm, x, bias=bias, out_dtype=torch.float32), y)
+
+
 @pytest.mark.parametrize("case", [(F.BLK1632_4, 4, 128, 16), (F.BLKC, 3, 64, 10), (F.DENSE4, 4, 128, 0)], ids=case_id)
 def test_linear_ragged_and_extreme_shapes(case):
     """One row, one chunk, row counts off the 16-row and 256-row tiles, column counts off the
