@@ -123,6 +123,18 @@ def test_entry_points_reject_bad_arguments_before_any_launch():
     d.data, d.cs_rows = 0x1000, 1
     assert L.cbk_gemv(ctypes.byref(d), 0x4000, 1, 1, 256, 0x5000, 0, 16, None, None, 0, None) == -1
     assert b"aligned" in L.cbk_strerror(-4)
+    # the packing and the static-scratch entry points check before they launch, too
+    d = F.CbkDesc(K=16, N=256, layout=F.BLK1632_4)
+    assert L.cbk_pack(ctypes.byref(d), None, 0x4000, 0x5000, 0x6000, 1, 1, None, None) == -1      # no destination arrays
+    d.data, d.scale, d.zero = 0x1000, 0x2000, 0x3000
+    assert L.cbk_pack(ctypes.byref(d), None, None, 0x5000, 0x6000, 1, 1, None, None) == -1
+    assert L.cbk_pack(ctypes.byref(d), None, 0x4000, 0x5000, 0x6000, 0, 1, None, None) == -5      # zero points are fp16 or uint8
+    assert L.cbk_pack(ctypes.byref(d), None, 0x4004, 0x5000, 0x6000, 1, 1, None, None) == -4
+    assert L.cbk_pack(ctypes.byref(d), 0x7001, 0x4000, 0x5000, 0x6000, 3, 1, None, None) == -4
+    ds = F.CbkDesc(K=16, N=256, layout=F.SPARSE4, data=0x1000, scale=0x2000, zero=0x3000, row_off=0x8000)
+    assert L.cbk_pack(ctypes.byref(ds), None, 0x4000, 0x5000, 0x6000, 1, 1, None, None) == -8     # variable-length layouts are not produced
+    big = F.CbkDesc(K=256, N=21504, layout=F.BLK1632_4, data=0x1000, scale=0x2000, zero=0x3000)
+    assert L.cbk_gemm_static(ctypes.byref(big), 0x4000, 2, 4096, 21504, 0x5000, 2, 256, None, None) == -6
 
 
 def test_ops_refuse_to_run_without_gpu_tensors():
