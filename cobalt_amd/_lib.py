@@ -25,6 +25,7 @@ SIGNATURES = {
     "cbk_stream_bytes": (ctypes.c_size_t, [_DP, ctypes.c_size_t]),
     "cbk_workspace_bytes": (ctypes.c_size_t, [_DP, ctypes.c_int]),
     "cbk_pack": (ctypes.c_int, [_DP, _P, _P, _P, _P, ctypes.c_int, ctypes.c_int, _P, _P]),
+    "cbk_unpack": (ctypes.c_int, [_DP, _P, _P, _P]),
     "cbk_dequant": (ctypes.c_int, [_DP, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P, ctypes.c_int,
                                    ctypes.c_int64, _P]),
     "cbk_gemv": (ctypes.c_int, _MM),

@@ -24,6 +24,7 @@ int launch_gemm_big(const DMat&, const void*, int, int, int64_t, void*, int, int
 size_t gemm_big_workspace(const DMat&, int M);
 int launch_pack(const DMat&, const void* mask, const void* q, const void* scale, const void* zero, int zero_f16,
                 int fix_zero, int* status, hipStream_t);
+int launch_unpack(const DMat&, void* q, void* mask, hipStream_t);
 // The 256 x 256 tile kernel takes every call of the fixed-stride layouts: below 256 activation
 // rows part of its token tile is padding, and it is still several times faster than the
 // 128 x 128 kernel, which decodes through the generic reader (14336 x 4096 at 64 rows: 54 us
@@ -161,6 +162,37 @@ static int check_io(const void* x, int xdt, int M, int64_t ldx, const void* y, i
   return CBK_OK;
 }
 
+// A survivor-stream matrix (SPARSE4, SPARSE4X, SPARSE4E: rows of different lengths) has no
+// matrix-core kernel of its own.  A prefill call re-packs it, in the caller's workspace and for
+// the duration of the call, as the dense 4-bit layout in tiled order (pruned columns hold the
+// zero point, so every weight dequantises to the same value) and runs the prefill kernel on that:
+// two small kernels (image -> codes and bitmap, codes -> rows) in front of the matrix product.
+struct Transient {
+  size_t q, mask, data, scale, zero, end;   // byte offsets in the workspace, 256-byte aligned
+};
+static Transient transient_dense4(const DMat& m) {
+  const size_t K16 = ((size_t)m.K + 15) / 16 * 16, stride = (size_t)m.N / 2;
+  auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  Transient t;
+  t.q = 0;
+  t.mask = up((size_t)m.K * m.N);
+  t.data = t.mask + up((size_t)m.K * (m.N / 8));
+  t.scale = t.data + up(K16 * stride + 512);
+  t.zero = t.scale + up(K16 * m.G * 2);
+  t.end = t.zero + up(K16 * m.G);
+  return t;
+}
+static DMat dense4_view(const DMat& m, uint8_t* ws, const Transient& t) {
+  DMat d = m;
+  d.data = ws + t.data; d.row_off = nullptr;
+  d.scale = (const uint16_t*)(ws + t.scale); d.zero = ws + t.zero;
+  d.layout = CBK_DENSE4; d.bits = 4; d.group = 128; d.keep = 0; d.G = m.N / 128;
+  d.flags = (m.flags & ~CBK_FLAG_TILED16) | CBK_FLAG_TILED16 | CBK_FLAG_ZERO_LE_128;   // 4-bit zero points are at most 15
+  d.tiled = 1;
+  d.stride = (uint32_t)(m.N / 2); d.code_off = 0;
+  return d;
+}
+
 }  // namespace cbk
 
 using namespace cbk;
@@ -203,6 +235,11 @@ size_t cbk_stream_bytes(const cbk_desc* in, size_t sparse_data_bytes) {
 size_t cbk_workspace_bytes(const cbk_desc* in, int M) {
   DMat m;
   if (to_dmat(in, &m, false)) return 0;
+  if (family_of(m.layout) == FAM_SPARSE) {                          // cbk_gemm / cbk_linear above 16 rows: see Transient
+    if (M <= 16) return 0;
+    const Transient t = transient_dense4(m);
+    return t.end + gemm_big_workspace(dense4_view(m, nullptr, t), M);
+  }
   // the most any of the three entry points asks for (cbk_gemm runs the prefill kernel at any M)
   size_t need = (M >= 1 && M <= 16 && gemv_fast_takes(m, 1)) ? gemv_fast_workspace(m, 1) : 0;
   if (gemm_big_takes(m, M)) {
@@ -246,6 +283,15 @@ int cbk_pack(const cbk_desc* dst, const void* mask_bits, const void* q, const vo
       (zero_dtype == CBK_F16 && ((uintptr_t)zero & 1)))
     return CBK_ERR_ALIGN;
   return launch_pack(m, mask_bits, q, scale, zero, zero_dtype == CBK_F16, fix_zero != 0, status, (hipStream_t)stream);
+}
+
+int cbk_unpack(const cbk_desc* in, void* q, void* mask_bits, void* stream) {
+  DMat m;
+  const int rc = to_dmat(in, &m, true);
+  if (rc) return rc;
+  if (!q) return CBK_ERR_NULL;
+  if (((uintptr_t)q & 15) || ((uintptr_t)mask_bits & 3)) return CBK_ERR_ALIGN;
+  return launch_unpack(m, q, mask_bits, (hipStream_t)stream);
 }
 
 int cbk_gemv_batch(int n, const cbk_desc* descs, const void* const* xs, const int64_t* ldxs, int x_dtype, int M,
@@ -331,6 +377,22 @@ int cbk_gemm(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ldx,
   if (rc) return rc;
   rc = check_io(x, x_dtype, M, ldx, y, y_dtype, ldy, m.N, m.K);
   if (rc) return rc;
+  if (family_of(m.layout) == FAM_SPARSE) {
+    if (M <= 16)                                                    // not worth re-packing: the row kernel
+      return cbk_gemv(in, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, workspace, workspace_bytes, stream);
+    if (m.cs_rows > 1) return CBK_ERR_UNSUPPORTED;                  // row fusion needs a fixed row stride
+    const Transient t = transient_dense4(m);
+    if (!workspace || workspace_bytes < t.end) return CBK_ERR_WORKSPACE;
+    if ((uintptr_t)workspace & 255) return CBK_ERR_ALIGN;
+    uint8_t* ws = (uint8_t*)workspace;
+    const DMat d = dense4_view(m, ws, t);
+    rc = launch_unpack(m, ws + t.q, ws + t.mask, (hipStream_t)stream);
+    if (rc) return rc;
+    rc = launch_pack(d, ws + t.mask, ws + t.q, m.scale, m.zero, 0, 0, nullptr, (hipStream_t)stream);
+    if (rc) return rc;
+    return launch_gemm_big(d, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, ws + t.end, workspace_bytes - t.end,
+                           (hipStream_t)stream);
+  }
   if (gemm_big_takes(m, M))
     return launch_gemm_big(m, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, workspace, workspace_bytes,
                            (hipStream_t)stream);
@@ -400,8 +462,9 @@ int cbk_linear(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ld
   // prefill kernel's 64-token tile decodes them (14336 x 4096: 28 us against 31 us; 54 us at 16 rows)
   if (M <= 8) return cbk_gemv(in, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, workspace, workspace_bytes, stream);
   cbk_desc d;
-  if (in && canon(in, &d) == CBK_OK && family_of(d.layout) == FAM_SPARSE) {
-    // the variable-length layouts have no MFMA path: run the row GEMV in slices of 16 rows
+  if (in && canon(in, &d) == CBK_OK && family_of(d.layout) == FAM_SPARSE && (M <= 16 || d.cs_rows > 1)) {
+    // the variable-length layouts have no MFMA path of their own: up to 16 rows the row GEMV (more
+    // rows go through cbk_gemm, which re-packs the matrix for the call)
     for (int m0 = 0; m0 < M; m0 += 16) {
       const int mc = M - m0 < 16 ? M - m0 : 16;
       int rc = cbk_gemv(in, (const uint8_t*)x + (size_t)m0 * ldx * 2, x_dtype, mc, ldx,

@@ -170,6 +170,78 @@ static void clear16(void* p, size_t bytes, hipStream_t st) {
   hipLaunchKernelGGL(pack_clear_kernel, dim3((unsigned)((bytes / 16 + 255) / 256)), dim3(256), 0, st, (uint4*)p, bytes / 16);
 }
 
+// ------------------------------------------------------------------ the way back: image -> RAW
+// Codes (0 at a pruned column of a bitmap or survivor-stream layout, the stored code, i.e. the
+// zero point, at a pruned column of a dense layout) and the keep bitmap of any layout.
+// Fixed-stride layouts: one thread per (row, 32-column block); survivor streams: one thread
+// per (row, group), as in the dequantiser.
+__global__ __launch_bounds__(256) void unpack_fixed_kernel(DMat m, uint8_t* q, uint8_t* mask) {
+  const int NB = m.N / BLOCK;
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= (int64_t)m.K * NB) return;
+  const int k = (int)(gid / NB), t = (int)(gid % NB);
+  int c[32];
+  const uint32_t keep = decode_block32(m, row_view(m, k), t, c);
+  uint32_t w[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    w[i] = (uint32_t)c[4 * i] | ((uint32_t)c[4 * i + 1] << 8) | ((uint32_t)c[4 * i + 2] << 16) | ((uint32_t)c[4 * i + 3] << 24);
+  uint4* dst = (uint4*)(q + (size_t)k * m.N + t * BLOCK);
+  dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
+  dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
+  if (mask) *(uint32_t*)(mask + (size_t)k * (m.N >> 3) + t * 4) = keep;
+}
+
+__global__ __launch_bounds__(256) void unpack_sparse_kernel(DMat m, uint8_t* q, uint8_t* mask) {
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= (int64_t)m.K * m.G) return;
+  const int k = (int)(gid / m.G), g = (int)(gid % m.G);
+  const uint8_t* row = m.data + m.row_off[k];
+  const uint32_t* bm = (const uint32_t*)row;
+  const bool has_goff = m.layout != CBK_SPARSE4;
+  const int hdr = ((m.N >> 3) + (has_goff ? ((m.G * 2 + 15) & ~15) : 0) + 15) & ~15;
+  uint32_t off = 0;
+  if (has_goff) {
+    off = ((const uint16_t*)(row + (m.N >> 3)))[g];
+  } else {
+    for (int gg = 0; gg < g; ++gg) {
+      int c = 0;
+      for (int i = 0; i < 4; ++i) c += __popc(bm[gg * 4 + i]);
+      off += (uint32_t)(c + 1) >> 1;
+    }
+  }
+  const uint8_t* codes = row + hdr + off;
+  int nib = 0;
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t keep = bm[g * 4 + i];
+    uint32_t w[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) w[e] = 0;
+#pragma unroll
+    for (int p = 0; p < 32; ++p) {
+      if ((keep >> p) & 1u) {
+        const uint32_t by = codes[nib >> 1];
+        const uint32_t c = (nib & 1) ? (by >> 4) : (by & 0xFu);
+        ++nib;
+        w[p >> 2] |= c << (8 * (p & 3));
+      }
+    }
+    uint4* dst = (uint4*)(q + (size_t)k * m.N + g * 128 + i * 32);
+    dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
+    dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
+    if (mask) *(uint32_t*)(mask + (size_t)k * (m.N >> 3) + g * 16 + i * 4) = keep;
+  }
+}
+
+int launch_unpack(const DMat& m, void* q, void* mask, hipStream_t st) {
+  const bool sparse = family_of(m.layout) == FAM_SPARSE;
+  const int64_t items = (int64_t)m.K * (sparse ? m.G : m.N / BLOCK);
+  const dim3 grid((unsigned)((items + 255) / 256)), blk(256);
+  if (sparse) hipLaunchKernelGGL(unpack_sparse_kernel, grid, blk, 0, st, m, (uint8_t*)q, (uint8_t*)mask);
+  else hipLaunchKernelGGL(unpack_fixed_kernel, grid, blk, 0, st, m, (uint8_t*)q, (uint8_t*)mask);
+  return hipGetLastError() == hipSuccess ? CBK_OK : CBK_ERR_HIP;
+}
+
 int launch_pack(const DMat& m, const void* mask, const void* q, const void* scale, const void* zero, int zero_f16,
                 int fix_zero, int* status, hipStream_t st) {
   const int fam = family_of(m.layout);

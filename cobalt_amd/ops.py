@@ -231,3 +231,30 @@ def pack_raw(mask_bits, q, scale, zero, col_scale, layout, bits=None, group=None
     if int(pm.array("zero").max()) <= 128:
         pm.flags |= F.FLAG_ZERO_LE_128
     return pm.validate()
+
+
+def unpack(pm: PackedMatrix):
+    """(mask_bits uint8 [K, N/8], q uint8 [K, N]) of a packed matrix of any layout on the GPU: the
+    inverse of `pack_raw` up to the zero-point repair (a dense layout returns its stored codes,
+    the zero point at pruned columns, and an all-ones mask)."""
+    _require_gpu(pm)
+    q = torch.empty(pm.K, pm.N, dtype=torch.uint8, device=pm.blob.device)
+    mask = torch.empty(pm.K, pm.N // 8, dtype=torch.uint8, device=pm.blob.device)
+    d = pm.desc()
+    _lib.check(_lib.lib().cbk_unpack(ctypes.byref(d), q.data_ptr(), mask.data_ptr(), _stream_ptr(pm.blob.device)), "cbk_unpack")
+    return mask, q
+
+
+def transcode(pm: PackedMatrix, layout: int, bits=None, group=None, keep=None, tiled=True) -> PackedMatrix:
+    """The same weights in another fixed-stride layout (same codes, scales, zero points and column
+    scales; every weight dequantises to the same value).  The use: a survivor-stream matrix
+    (SPARSE4*, which the row kernel serves at about a tenth of the matrix-core kernels' rate)
+    as DENSE4, one bit per weight more for the fast kernels."""
+    from . import format as F
+    mask, q = unpack(pm)
+    rm = pm.to_rowmajor() if pm.tiled else pm
+    cs = rm.array("col_scale").view(rm.cs_rows, rm.N) if rm.cs_rows else None
+    out = pack_raw(None if pm.layout in F._DENSE else mask, q, rm.array("scale").view(rm.K, rm.G), rm.array("zero").view(rm.K, rm.G),
+                   cs, layout, bits, group, keep, fix_zero=False, cs_splits=rm.cs_splits, tiled=tiled)
+    out.n_survivors = pm.n_survivors
+    return out

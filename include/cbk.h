@@ -159,6 +159,14 @@ int cbk_dequant(const cbk_desc* d, int row0, int nrows, int with_col_scale,
 int cbk_pack(const cbk_desc* dst, const void* mask_bits, const void* q, const void* scale,
              const void* zero, int zero_dtype, int fix_zero, int* status, void* stream);
 
+/* The way back: the codes and the keep bitmap of a packed image of any layout, as uint8 [K, N]
+ * (0 at a pruned column of a bitmap or survivor-stream layout; a dense layout returns what it
+ * stores there, the group's zero point) and, if mask_bits is not NULL, uint8 [K, N/8] LSB first
+ * (all ones for a dense layout).  The decode side of `dequant_reference`
+ * (src/cobaltkernel/pack_cobalt.py:277-334) without the arithmetic; with cbk_pack it re-packs a
+ * matrix into another layout, which is how cbk_gemm serves the survivor-stream layouts. */
+int cbk_unpack(const cbk_desc* d, void* q, void* mask_bits, void* stream);
+
 /* Decode path, 1 <= M <= 16: y[m, k] = sum_j x[m, j] * W_hat[k, j] (+ bias[k]).
  * x is [M, ldx] fp16 or bf16, y is [M, ldy] in y_dtype (f32 / f16 / bf16), bias is NULL or
  * K values of y_dtype.  Replaces the harness entry `gemv` (test_gemv.cu:187-199) and
@@ -180,9 +188,13 @@ int cbk_gemv_batch(int n, const cbk_desc* descs, const void* const* xs, const in
                    int x_dtype, int M, void* const* ys, const int64_t* ldys, int y_dtype,
                    const void* const* biases, void* workspace, size_t workspace_bytes, void* stream);
 
-/* Prefill path, any M >= 1 (256-token tiles; a 64-token tile up to 64 rows).  Same contract as cbk_gemv; bf16 activations
- * are carried as fp16 inside (magnitudes above 65504 saturate).  Replaces the
- * harness entry `gemm` (test_gemm.cu:151-165) and cbk::gemm_tile (cobalt_gemm.cuh:243-609). */
+/* Prefill path, any M >= 1 (256-token tiles; a 64-token tile up to 64 rows).  Same contract as
+ * cbk_gemv; activations are carried as fp16 inside, a token whose values leave fp16's range
+ * scaled by a power of two on the way in and back on the way out.  The survivor-stream layouts
+ * (SPARSE4, SPARSE4X, SPARSE4E) are re-packed for the call, above 16 rows, into the dense 4-bit
+ * layout inside the workspace (cbk_workspace_bytes counts it) and go to the row kernel below
+ * that.  Replaces the harness entry `gemm` (test_gemm.cu:151-165) and cbk::gemm_tile
+ * (cobalt_gemm.cuh:243-609). */
 int cbk_gemm(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
              void* y, int y_dtype, int64_t ldy, const void* bias,
              void* workspace, size_t workspace_bytes, void* stream);

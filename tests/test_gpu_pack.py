@@ -162,3 +162,72 @@ def test_compress_and_pack_one_full_size_matrix_on_the_gpu():
     assert float((y - want).abs().max() / want.abs().max()) < 2e-5
     loose = x.double() @ raw["W_hat"].double().T                        # scales not yet rounded to fp16
     assert float((y - loose).norm() / loose.norm()) < 1e-3
+
+
+# ------------------------------------------------------------------ the way back, and re-packing
+from helpers import SPARSE_CASES, packed_from_oracle, kw_of, rel_fro, acts
+
+
+@pytest.mark.parametrize("case", FIXED_CASES + SPARSE_CASES, ids=case_id)
+def test_unpack_returns_the_codes_and_the_bitmap(case):
+    """cbk_unpack on every layout, both byte orders, against the oracle's decoder: the codes of
+    the kept columns, zeros (bitmap / survivor-stream layouts) or the zero point (dense layouts)
+    at the pruned ones, and the keep bitmap."""
+    layout, bits, group, keep = case
+    K, N = 37, 640
+    raw = make_raw(case, K, N, seed=9)
+    pk = oracle_pack(case, raw)
+    q_ref, keep_ref = R.unpack_codes(pk, K, N, layout, bits, group, keep or None)
+    for tiled in ((False, True) if layout not in (F.SPARSE4, F.SPARSE4X, F.SPARSE4E) else (False,)):
+        pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV, tiled=tiled)
+        mask, q = ops.unpack(pm)
+        q, keepm = q.cpu().numpy(), F.unpack_mask(mask.cpu(), N).numpy()
+        dense = layout in (F.DENSE4, F.DENSE8, F.DENSEB)
+        assert np.array_equal(keepm, np.ones_like(keepm) if dense else keep_ref != 0), tiled
+        assert np.array_equal(q[keep_ref != 0], np.asarray(q_ref)[keep_ref != 0]), tiled
+        if not dense:
+            assert (q[keep_ref == 0] == 0).all()
+
+
+@pytest.mark.parametrize("case", SPARSE_CASES, ids=case_id)
+def test_survivor_streams_repacked_as_dense_rows(case):
+    """A survivor-stream matrix re-packed as DENSE4 (`ops.transcode`) dequantises to the same
+    values bit for bit and runs on the matrix-core kernels; and `ops.linear` above 16 rows, which
+    re-packs inside the call's workspace, meets the oracle like every other layout."""
+    layout = case[0]
+    K, N = 300, 1152
+    raw = R.synth_raw_matrix(K, N, 0.55, 4, seed=21)
+    pk = oracle_pack(case, raw)
+    W = R.dequant(pk, K, N, layout, col_scale=raw["col_scale"])
+    pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV)
+    d4 = ops.transcode(pm, F.DENSE4)
+    assert d4.tiled and d4.layout == F.DENSE4 and abs(d4.bpw() - (4 + 24 / 128) * (304 / 300)) < 1e-9
+    assert np.array_equal(ops.dequant(d4, torch.float32).cpu().numpy() + np.float32(0), W + np.float32(0))
+    for M in (1, 8, 17, 64, 300):
+        x = acts(M, N, torch.bfloat16, seed=M)
+        ref = R.forward_ref(W, x.float().numpy())
+        for p in (pm, d4):
+            y = ops.linear(p, x.to(DEV), out_dtype=torch.float32).cpu().numpy()
+            assert rel_fro(y, ref) < 1e-3, (case_id(case), M, p.layout)
+    y = ops.gemm(pm, acts(5, N, torch.float16, seed=5).to(DEV), out_dtype=torch.float32)       # few rows: the row kernel
+    assert rel_fro(y.cpu().numpy(), R.forward_ref(W, acts(5, N, torch.float16, seed=5).float().numpy())) < 1e-3
+
+
+def test_module_with_a_survivor_stream_matrix_can_be_repacked_at_load():
+    case = (F.SPARSE4E, 4, 128, 0)
+    K, N = 96, 1024
+    raw = R.synth_raw_matrix(K, N, 0.5, 4, seed=4)
+    pk = oracle_pack(case, raw)
+    W = R.dequant(pk, K, N, F.SPARSE4E, col_scale=raw["col_scale"])
+    lin = CobaltLinear(packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV))
+    assert lin.to_device_order()._pm().layout == F.SPARSE4E                      # unchanged unless asked
+    lin.to_device_order(repack_sparse=True)
+    pm = lin._pm()
+    assert (pm.layout, pm.tiled) == (F.DENSE4, True)
+    assert np.array_equal(lin.dequantize().cpu().numpy() + np.float32(0), W + np.float32(0))
+    x = acts(3, N, torch.float16, seed=1)
+    y = lin(x.to(DEV)).float().cpu().numpy()
+    assert rel_fro(y, R.forward_ref(W, x.float().numpy())) < 2e-3               # fp16 output
+    sd = lin.state_dict()
+    back = CobaltLinear.from_state(sd["blob"], sd["cbk_meta"])
+    assert torch.equal(back.dequantize(), lin.dequantize())
