@@ -184,8 +184,8 @@ static Transient transient_dense4(const DMat& m) {
 }
 static DMat dense4_view(const DMat& m, uint8_t* ws, const Transient& t) {
   DMat d = m;
-  d.data = ws + t.data; d.row_off = nullptr;
-  d.scale = (const uint16_t*)(ws + t.scale); d.zero = ws + t.zero;
+  d.row_off = nullptr;
+  if (ws) { d.data = ws + t.data; d.scale = (const uint16_t*)(ws + t.scale); d.zero = ws + t.zero; }   // else: sizes only
   d.layout = CBK_DENSE4; d.bits = 4; d.group = 128; d.keep = 0; d.G = m.N / 128;
   d.flags = (m.flags & ~CBK_FLAG_TILED16) | CBK_FLAG_TILED16 | CBK_FLAG_ZERO_LE_128;   // 4-bit zero points are at most 15
   d.tiled = 1;
