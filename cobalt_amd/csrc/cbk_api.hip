@@ -187,7 +187,7 @@ static DMat dense4_view(const DMat& m, uint8_t* ws, const Transient& t) {
   d.row_off = nullptr;
   if (ws) { d.data = ws + t.data; d.scale = (const uint16_t*)(ws + t.scale); d.zero = ws + t.zero; }   // else: sizes only
   d.layout = CBK_DENSE4; d.bits = 4; d.group = 128; d.keep = 0; d.G = m.N / 128;
-  d.flags = (m.flags & ~CBK_FLAG_TILED16) | CBK_FLAG_TILED16 | CBK_FLAG_ZERO_LE_128;   // 4-bit zero points are at most 15
+  d.flags = m.flags | CBK_FLAG_TILED16;                             // CBK_FLAG_ZERO_LE_128 as the caller stated it
   d.tiled = 1;
   d.stride = (uint32_t)(m.N / 2); d.code_off = 0;
   return d;
