@@ -48,7 +48,7 @@ class _BlobWriter:
 
     def put(self, t: torch.Tensor) -> dict:
         self._pad()
-        raw = t.contiguous().reshape(-1).view(torch.uint8).cpu().numpy().tobytes()
+        raw = t.reshape(-1).clone(memory_format=torch.contiguous_format).view(torch.uint8).cpu().numpy().tobytes()
         off = self.pos
         self.f.write(raw)
         self.pos += len(raw)

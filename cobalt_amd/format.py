@@ -365,7 +365,9 @@ def _assemble(arrays: Dict[str, torch.Tensor], device) -> Tuple[torch.Tensor, Di
         pos += a.numel() * a.element_size()
     blob = torch.zeros(_align(pos, ARR_ALIGN), dtype=torch.uint8, device=device)
     for name, a in arrays.items():
-        b = a.contiguous().reshape(-1).view(torch.uint8)
+        # a copy with contiguous strides: a tensor whose only non-unit stride sits on a size-1
+        # dimension counts as contiguous, and its flat view would keep that stride
+        b = a.reshape(-1).clone(memory_format=torch.contiguous_format).view(torch.uint8)
         blob[offs[name]: offs[name] + b.numel()] = b.to(device)
     return blob, offs
 
@@ -467,7 +469,7 @@ def from_arrays(data, scale, zero, col_scale, K, N, layout, bits=None, group=Non
     if col_scale is not None:
         cs = torch.as_tensor(col_scale).reshape(-1, N)
         cs_rows = cs.shape[0]
-        arrays["col_scale"] = cs.contiguous().reshape(-1).view(torch.uint8)
+        arrays["col_scale"] = cs.reshape(-1).clone(memory_format=torch.contiguous_format).view(torch.uint8)
     blob, offs = _assemble(arrays, dev)
     flags = FLAG_ZERO_LE_128 if int(torch.as_tensor(zero).reshape(-1).view(torch.uint8).max()) <= 128 else 0
     return PackedMatrix(blob, offs, K, N, layout, bits, group, kpb, cs_rows, tuple(cs_splits),

@@ -231,3 +231,23 @@ def test_module_with_a_survivor_stream_matrix_can_be_repacked_at_load():
     sd = lin.state_dict()
     back = CobaltLinear.from_state(sd["blob"], sd["cbk_meta"])
     assert torch.equal(back.dequantize(), lin.dequantize())
+
+
+def test_pack_and_unpack_at_the_smallest_and_ragged_shapes():
+    """One row of one 128-column group; 17 rows (a tile and one row) of 128 and 384 columns: the
+    packing kernel's half unit, the tile padding and the unpacker, both byte orders."""
+    for case in ((F.BLK1632_4, 4, 128, 16), (F.BLKC, 3, 64, 10), (F.DENSE4, 4, 128, 0), (F.BLK1632_6, 6, 128, 16)):
+        layout, bits, group, keep = case
+        for K, N in ((1, 128), (17, 128), (17, 384)):
+            raw = make_raw(case, K, N, seed=K + N)
+            pk = oracle_pack(case, raw)
+            args = tuple(_t(raw[k]) for k in ("mask", "q", "scale", "zero", "col_scale")) + (layout, bits, group, keep or None)
+            for tiled in (False, True):
+                pm = ops.pack_raw(*args, tiled=tiled)
+                want = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV, tiled=tiled)
+                assert torch.equal(pm.blob, want.blob), (case_id(case), K, N, tiled)
+                mask, q = ops.unpack(pm)
+                back = ops.pack_raw(None if keep == 0 else mask, q, pm.to_rowmajor().array("scale").view(K, -1),
+                                    pm.to_rowmajor().array("zero").view(K, -1), _t(raw["col_scale"]), layout, bits, group,
+                                    keep or None, fix_zero=False, tiled=tiled)
+                assert torch.equal(back.blob, pm.blob), (case_id(case), K, N, tiled)
