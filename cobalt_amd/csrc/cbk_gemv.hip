@@ -174,22 +174,25 @@ __device__ inline void stage_convert(const XLoad& r, bool has_cs, int xdt, int N
   mx = fmaxf(mx, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, mx), 0x141, 0xF, 0xF, true)));
   const float d = mx > 0.f ? mx / 8323072.f : 1.f;
   const float inv = 1.f / d;
+  // X + 0x808080 has the bytes d0 + 128, d1 + 128, d2 + 128 of the balanced base-256 digits
+  // (X = d0 + 256 d1 + 65536 d2, -128 <= d < 128), so the digits of four columns are byte
+  // permutes of the four biased integers and one xor per digit plane
   uint32_t dw[NDIG][4];
-#pragma unroll
-  for (int k = 0; k < NDIG; ++k)
-#pragma unroll
-    for (int q = 0; q < 4; ++q) dw[k][q] = 0u;
+  uint32_t xb[16];
 #pragma unroll
   for (int bi = 0; bi < 16; ++bi) {
     const float v = ORDER == 0 ? xv[bi] : ORDER == 1 ? xv[frag_col(4, true, bi)] : xv[frag_col(2, true, bi)];
-    int X = (int)rintf(v * inv);                       // |X| <= 127 * 65536
-    const int d0 = (int)(int8_t)(X & 0xFF);
-    X = (X - d0) >> 8;
-    const int d1 = (int)(int8_t)(X & 0xFF);
-    const int d2 = (X - d1) >> 8;
-    dw[0][bi >> 2] |= ((uint32_t)d2 & 0xFFu) << (8 * (bi & 3));
-    dw[1][bi >> 2] |= ((uint32_t)d1 & 0xFFu) << (8 * (bi & 3));
-    dw[2][bi >> 2] |= ((uint32_t)d0 & 0xFFu) << (8 * (bi & 3));
+    xb[bi] = (uint32_t)((int)rintf(v * inv) + 0x808080);          // |X| <= 127 * 65536
+  }
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const uint32_t a = perm(xb[4 * q + 1], xb[4 * q], 0x05010400u);       // d0 d0 d1 d1 of columns 0, 1
+    const uint32_t b = perm(xb[4 * q + 3], xb[4 * q + 2], 0x05010400u);   // and of columns 2, 3
+    const uint32_t c01 = perm(xb[4 * q + 1], xb[4 * q], 0x0C0C0602u);     // d2 d2 0 0
+    const uint32_t c23 = perm(xb[4 * q + 3], xb[4 * q + 2], 0x06020C0Cu); // 0 0 d2 d2
+    dw[0][q] = (c01 | c23) ^ 0x80808080u;
+    dw[1][q] = perm(b, a, 0x07060302u) ^ 0x80808080u;
+    dw[2][q] = perm(b, a, 0x05040100u) ^ 0x80808080u;
   }
 #pragma unroll
   for (int k = 0; k < NDIG; ++k)
@@ -302,8 +305,21 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
   uint8_t* zreg = smem + LUT_BYTES;
   int* cnt = (int*)(zreg + ZERO_BYTES);                // [CNT_SLOTS] arrival counters
   int8_t* xq = (int8_t*)cnt + CNT_BYTES;
+  // The argument block is read in two dependent steps (header, then the record of the first
+  // matrix), each a round trip to memory for the first wavefronts that ask.  Touch its first
+  // cache lines now, with scalar loads whose results nobody uses, so that both steps find them
+  // in the scalar cache; the registers stay reserved until the loads have returned.
+  uint32_t ka[5];
+  static_assert(sizeof(GvBatch) >= 0x104, "the five touched lines lie inside the argument block");
+  {
+    const auto kp = __builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("s_load_dword %0, %5, 0x0\n\ts_load_dword %1, %5, 0x40\n\ts_load_dword %2, %5, 0x80\n\t"
+                 "s_load_dword %3, %5, 0xc0\n\ts_load_dword %4, %5, 0x100"
+                 : "=&s"(ka[0]), "=&s"(ka[1]), "=&s"(ka[2]), "=&s"(ka[3]), "=&s"(ka[4]) : "s"(kp));
+  }
   // Selector table, zero row and counters do not depend on the arguments: they are written
-  // while the argument block is on its way, and published by a barrier nobody waits long at.
+  // while the argument block is on its way, and published by the barrier that follows the
+  // staging of the first matrix's activations (nothing reads them before).
   {
     using C0 = Cfg<BITS, KEEP, GRP, MP>;
     if (tid < 256) {
@@ -315,7 +331,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     } else if (tid < 256 + ZERO_BYTES / 4 + CNT_SLOTS) {
       cnt[tid - 256 - ZERO_BYTES / 4] = 0;
     }
-    __syncthreads();
+    asm volatile("s_waitcnt lgkmcnt(0)" ::"s"(ka[0]), "s"(ka[1]), "s"(ka[2]), "s"(ka[3]), "s"(ka[4]));
   }
   const GvHead h = b.h;
   float* delta = (float*)(xq + h.xq_cap);
@@ -499,6 +515,8 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 #pragma unroll
         for (int p = 0; p < MP; ++p) ysum[p] = 0.f;
       }
+      // (unconditional: past the last position the loads repeat it; under a wave-uniform branch
+      // the compiler no longer spreads them over the decode, and every launch was 2-6 % slower)
       issue(t_lo + p1.tl, p1.S, tgt);
       if constexpr (QB) {
         const int a_m = wr >> 2;                                    // activation row of this lane's A row
