@@ -51,7 +51,8 @@ constexpr int LUT_BYTES = 256 * LUT_LANES * 8;
 constexpr int ZERO_BYTES = 256;
 constexpr int CNT_SLOTS = 64;                 // most reduction slots (arrival counters)
 constexpr int CNT_BYTES = CNT_SLOTS * 4;       // at a fixed place: zeroed before the arguments are read
-constexpr int X_LDS_BUDGET = 112 * 1024;      // activation digits: M * 3 * N bytes (of 160 KB LDS)
+constexpr int X_LDS_BUDGET = 112 * 1024;      // activation digits of one column slab: M * 3 * columns bytes (of 160 KB LDS)
+constexpr int DELTA_LDS_BUDGET = 6 * 1024;    // one float per 128-column chunk and activation row
 constexpr int NDIG = 3;                       // int8 digits per activation
 constexpr int GV_MAX_M = 8;                     // 5..8 only in the block-per-quarter arrangement
 constexpr int GV_MAX_BATCH = 8;               // matrices per launch
@@ -76,6 +77,8 @@ struct GvMat {
   int nS;                  // macro-steps per tile = ceil(N / 512)
   int cost0;               // sum of ntiles * nS over the matrices before this one
   int spi, sk;             // macro-steps per work item, work items per tile
+  int sp;                  // parts per column slab: the activation digits of sp * spi * 512 columns are staged at a
+                           // time (sp == sk: the whole row at once)
   // branch-free addressing of either byte order.  Row r of tile t starts at
   // data + t * tile_a + r * lane_mul and its 16-byte units are 1 << ush bytes apart; the scale /
   // zero entry of (row, group g) has index t * 16 * G + r * sz_mul + (g << csh).
@@ -128,26 +131,29 @@ __host__ __device__ constexpr bool block_split_capable(int bits, int keep, int g
 // eight threads of a chunk agree on its maximum with three lane exchanges.
 struct XLoad { uint4 x[2], c[2]; };
 
-// global loads of staging item `it` (activation row it / (N/16), columns 16 * (it % (N/16)) ...)
-__device__ inline void stage_load(const uint16_t* x, int64_t ldx, const uint16_t* cs, int n16, int it, bool one_row,
-                                  int par, XLoad& r) {
+// global loads of staging item `it` of the column slab that starts at column col0 and is n16 * 16
+// columns wide (activation row it / n16, columns col0 + 16 * (it % n16) ...)
+__device__ inline void stage_load(const uint16_t* x, int64_t ldx, const uint16_t* cs, int N, int col0, int n16, int it,
+                                  bool one_row, int par, XLoad& r) {
   const int row = one_row ? 0 : it / n16, c16 = it - row * n16;
   const int xrow = par ? row >> 1 : row;
-  const uint16_t* xp = x + (size_t)xrow * ldx + c16 * 16;
+  const uint16_t* xp = x + (size_t)xrow * ldx + col0 + c16 * 16;
   r.x[0] = ((const uint4*)xp)[0]; r.x[1] = ((const uint4*)xp)[1];
   r.c[0] = make_uint4(0, 0, 0, 0); r.c[1] = make_uint4(0, 0, 0, 0);
   if (cs) {
-    const uint16_t* cp = cs + (par ? (size_t)(row & 1) * n16 * 16 : (size_t)0) + c16 * 16;
+    const uint16_t* cp = cs + (par ? (size_t)(row & 1) * N : (size_t)0) + col0 + c16 * 16;
     r.c[0] = ((const uint4*)cp)[0]; r.c[1] = ((const uint4*)cp)[1];
   }
 }
 
 // conversion of one loaded item into digits and delta in LDS; the eight consecutive lanes of a
 // chunk are always active together (the item count is a multiple of 8)
+// (digits at row stride Ns = 16 * n16 bytes, deltas at the chunk's index in the whole row: ch0 is
+// the slab's first chunk)
 template <int ORDER>
-__device__ inline void stage_convert(const XLoad& r, bool has_cs, int xdt, int N, int n16, int it, bool one_row,
+__device__ inline void stage_convert(const XLoad& r, bool has_cs, int xdt, int N, int ch0, int n16, int it, bool one_row,
                                      int8_t* xq, float* delta) {
-  const int NCH = N >> 7;
+  const int NCH = N >> 7, Ns = n16 * 16;
   const int row = one_row ? 0 : it / n16, c16 = it - row * n16;
   const uint32_t* xw = (const uint32_t*)r.x;
   const uint32_t* cw = (const uint32_t*)r.c;
@@ -196,9 +202,9 @@ __device__ inline void stage_convert(const XLoad& r, bool has_cs, int xdt, int N
   }
 #pragma unroll
   for (int k = 0; k < NDIG; ++k)
-    *(uint4*)(xq + ((size_t)row * NDIG + k) * N + c16 * 16) = make_uint4(dw[k][0], dw[k][1], dw[k][2], dw[k][3]);
-  if ((c16 & 7) == 0) delta[row * (NCH + 4) + (c16 >> 3)] = d;
-  if (c16 < 4) delta[row * (NCH + 4) + NCH + c16] = 0.f;          // chunks past N
+    *(uint4*)(xq + ((size_t)row * NDIG + k) * Ns + c16 * 16) = make_uint4(dw[k][0], dw[k][1], dw[k][2], dw[k][3]);
+  if ((c16 & 7) == 0) delta[row * (NCH + 4) + ch0 + (c16 >> 3)] = d;
+  if (ch0 == 0 && c16 < 4) delta[row * (NCH + 4) + NCH + c16] = 0.f;   // chunks past N
 }
 
 // y(l) + y(l ^ 16), then that + the same of lane l ^ 32: the sum over the four lane quarters, in
@@ -357,21 +363,32 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 
   // The first record is requested together with the header: most workgroups start with it, and
   // for them the second round trip through the argument block before any load goes out is gone.
+  // One trip of the loop below = one matrix, or, for a matrix whose rows are longer than the
+  // staging area (more than one activation row only), one column slab of one group of its tiles.
+  // A single loop level on purpose: nested loops made the compiler keep several dozen more
+  // scalars alive across the decode loop, spilled into vector registers.
+  constexpr bool SLABS = MP > 1;
   GvMat gm = b.mat[0];
-  for (int mi = mi0; mi < h.n; ++mi) {
+  int g_lo = -1, pa = 0;                                          // tile group and first part of the next trip
+  for (int mi = mi0; mi < h.n;) {
     if (mi != 0) gm = b.mat[mi];                                  // one read of the whole record
     if (gm.cost0 >= c1) break;                                    // uniform over the workgroup
     const DMat& m = gm.m;
     const int nS = gm.nS;
-    int t_lo = (c0 - gm.cost0 + nS - 1) / nS, t_hi = (c1 - gm.cost0 + nS - 1) / nS;
-    t_lo = t_lo < 0 ? 0 : t_lo;
-    t_hi = t_hi > gm.ntiles ? gm.ntiles : t_hi;
-    if (t_lo >= t_hi) continue;                                   // uniform over the workgroup
+    int T_lo = (c0 - gm.cost0 + nS - 1) / nS, T_hi = (c1 - gm.cost0 + nS - 1) / nS;
+    T_lo = T_lo < 0 ? 0 : T_lo;
+    T_hi = T_hi > gm.ntiles ? gm.ntiles : T_hi;
+    if (T_lo >= T_hi) { ++mi; continue; }                         // uniform over the workgroup
     const int N = m.N, NCH = N >> 7;
     // items: tile tl (local), part j of SK; part j covers macro-steps [j*spi, min(nS,(j+1)*spi))
-    const int SK = gm.sk, spi = gm.spi;
+    const int SK = gm.sk, spi = gm.spi, SP = SLABS ? gm.sp : SK;
+    // A row whose digits do not fit in LDS is staged and multiplied slab by slab (SP parts of
+    // every tile at a time).  A tile's partial sums then wait in their reduction slot across the
+    // slabs, so the tiles are taken nslot at a time and the slots are never reused inside a group.
+    const bool slabbed = SLABS && SP < SK;
     const int gt = h.nslot >> 1;                                  // tiles per barrier group, a power of two
-    const int gsh = 31 - __builtin_clz((unsigned)gt);               // its logarithm: no division per item
+    const int gsh = slabbed ? 30 : 31 - __builtin_clz((unsigned)gt);   // its logarithm: no division per item
+    const int tgs = slabbed ? h.nslot : T_hi - T_lo;              // tiles per pass over the slabs
 
     // matrix constants, read from the kernel arguments once
     const uint8_t* const m_data = m.data;
@@ -379,7 +396,14 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     const uint8_t* const m_zero = m.zero;
     const int m_K = m.K, m_G = m.G, ush = gm.ush, csh = gm.csh;
     const uint32_t tile_a = gm.tile_a, lane_mul = gm.lane_mul, sz_mul = gm.sz_mul, code_u0 = m.code_off >> 4;
-    const int last_tile = t_hi - 1, last_S = nS - 1;
+    const int last_S = nS - 1;
+    const int t_lo = SLABS && g_lo >= 0 ? g_lo : T_lo;
+    const int t_hi = SLABS && t_lo + tgs < T_hi ? t_lo + tgs : T_hi;
+    const int last_tile = t_hi - 1;
+    const int pn = SLABS && SK - pa >= SP ? SP : SK - pa;         // parts of this slab
+    const int col0 = SLABS ? pa * spi * 512 : 0;                  // its columns: [col0, col0 + Ns)
+    const int Ns = SLABS && N - col0 >= pn * spi * 512 ? pn * spi * 512 : N - col0;
+    const int ch0 = col0 >> 7;
 
     // ---- issue the loads of one (tile, macro-step) position; out-of-range positions are clamped
     // Everything that depends only on (tile, S) is scalar work; a lane adds a 32-bit offset.
@@ -467,25 +491,25 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     // of loads in flight, slower on large launches)
     struct Pos { int tl, part, S; };
     const int ntl = t_hi - t_lo;
-    const int dq_t = GV_WAVES / SK, dq_p = GV_WAVES % SK;
+    const int dq_t = GV_WAVES / pn, dq_p = GV_WAVES % pn;
     auto advance = [&](Pos& p) -> bool {                           // false past the last position
       const int s_end = (p.part * spi + spi < nS) ? p.part * spi + spi : nS;
       if (p.S + 1 < s_end) { ++p.S; return true; }
       p.tl += dq_t; p.part += dq_p;
-      if (p.part >= SK) { p.part -= SK; ++p.tl; }
+      if (p.part >= pa + pn) { p.part -= pn; ++p.tl; }
       p.S = p.part * spi;
       return p.tl < ntl;
     };
-    Pos p0{wave / SK, wave % SK, (wave % SK) * spi};
+    Pos p0{wave / pn, pa + wave % pn, (pa + wave % pn) * spi};
     bool v0 = p0.tl < ntl;
     Pos p1 = p0; bool v1 = v0 && advance(p1);
     // The activation loads go out before the first weight loads: the weight prefetch of a whole
     // launch is tens of megabytes, and a request queued behind it would keep every wavefront
     // from decoding until that burst has drained.
-    const int n16 = N >> 4, xitems = h.M * n16;                   // a multiple of 8
+    const int n16 = Ns >> 4, xitems = h.M * n16;                  // a multiple of 8
     int xit = tid;
     XLoad xl;
-    if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, MP == 1, gm.par, xl);
+    if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, N, col0, n16, xit, MP == 1, gm.par, xl);
     // Two load buffers swap roles (being decoded, being loaded) by name: copying a buffer would
     // wait for the loads that are still filling it.  One step of loads in flight per wavefront
     // is the measured optimum (sixteen wavefronts per CU already cover the latency; a second
@@ -497,9 +521,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     if (!first) __syncthreads();                                  // previous matrix fully consumed
     first = false;
     while (xit < xitems) {
-      stage_convert<(!C::DENSE ? 0 : (BITS == 2 ? 2 : 1))>(xl, m.cs != nullptr, h.xdt, N, n16, xit, MP == 1, xq, delta);
+      stage_convert<(!C::DENSE ? 0 : (BITS == 2 ? 2 : 1))>(xl, m.cs != nullptr, h.xdt, N, ch0, n16, xit, MP == 1, xq, delta);
       xit += GV_THREADS;
-      if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, n16, xit, MP == 1, gm.par, xl);
+      if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, N, col0, n16, xit, MP == 1, gm.par, xl);
     }
     __syncthreads();
 
@@ -531,7 +555,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 #pragma unroll
         for (int g = 0; g < NG; ++g) {
           a_on[g] = a_dig < NDIG && a_m + 4 * g < h.M;
-          a_base[g] = xq_off + (uint32_t)(((a_m + 4 * g) * NDIG + a_dig) * N + kq * 32);
+          a_base[g] = xq_off + (uint32_t)(((a_m + 4 * g) * NDIG + a_dig) * Ns + kq * 32);
           dm[g] = kq + 4 * g < h.M ? kq + 4 * g : 0;
         }
 #pragma unroll
@@ -539,7 +563,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
           const int chunk = 4 * S + c;
           uint32_t aaddr[NG];
 #pragma unroll
-          for (int g = 0; g < NG; ++g) aaddr[g] = (a_on[g] && chunk < NCH) ? a_base[g] + (uint32_t)chunk * 128u : z_off;
+          for (int g = 0; g < NG; ++g) aaddr[g] = (a_on[g] && chunk < NCH) ? a_base[g] + (uint32_t)(chunk - ch0) * 128u : z_off;
           uint32_t rkc[4];
           uint2 selc[4];
           fetch_selectors<C>(cur.mk[c], lut, l16, rkc, selc);
@@ -580,7 +604,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 #pragma unroll
         for (int p = 0; p < MP; ++p) {
           const bool on = valid && a_slice == kq && a_dig < NDIG && p < h.M;
-          aaddr[p] = on ? xq_off + (uint32_t)((p * NDIG + a_dig) * N + chunk * 128) : z_off;
+          aaddr[p] = on ? xq_off + (uint32_t)((p * NDIG + a_dig) * Ns + (chunk - ch0) * 128) : z_off;
         }
         // ---- bring the chunk's first code bit to bit 0 of cw[0]
         uint32_t cw[C::ND];
@@ -719,8 +743,19 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       do_step(LB, LA);
     }
     // every wave passes the same number of group barriers
-    const int ngroups = ((t_hi - t_lo) + gt - 1) >> gsh;
+    const int ngroups = slabbed ? 1 : ((t_hi - t_lo) + gt - 1) >> gsh;
     for (; bars < ngroups - 1; ++bars) __syncthreads();
+    // next trip: the next slab of these tiles, the next group of tiles, the next matrix
+    if (SLABS) {
+      pa += SP;
+      if (pa >= SK) {
+        pa = 0;
+        g_lo = t_hi;
+        if (t_hi >= T_hi) { g_lo = -1; ++mi; }
+      }
+    } else {
+      ++mi;
+    }
   }
 }
 
@@ -743,7 +778,10 @@ bool gemv_fast_takes(const DMat& m, int M) {
   // 32-bit offsets inside the kernel: every array of the matrix below 4 GB
   if ((uint64_t)((m.K + 15) / 16 * 16) * m.stride + 1024 >= (1ull << 32)) return false;
   if ((uint64_t)((m.K + 15) / 16 * 16) * m.G * 2 >= (1ull << 32)) return false;
-  return (size_t)M * NDIG * m.N <= (size_t)X_LDS_BUDGET;
+  // the digits are staged in column slabs where a whole row does not fit; the per-chunk deltas
+  // of all rows stay in LDS for the whole matrix
+  if (M == 1) return (size_t)NDIG * m.N <= (size_t)X_LDS_BUDGET;   // (the one-row kernels stage whole rows only)
+  return (size_t)M * (m.N / 128 + 4) * 4 <= (size_t)DELTA_LDS_BUDGET;
 }
 
 bool gemv_same_config(const DMat& a, const DMat& b) {
@@ -837,12 +875,10 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
     cost += g.ntiles * g.nS;
     gb.h.cost_end[i] = cost;
     tiles += g.ntiles;
-    xq_cap = xq_cap > M * NDIG * m.N ? xq_cap : M * NDIG * m.N;
     delta_cap = delta_cap > M * (m.N / 128 + 4) ? delta_cap : M * (m.N / 128 + 4);
   }
   (void)workspace; (void)ws_bytes;
   for (int i = n; i < GV_MAX_BATCH; ++i) gb.h.cost_end[i] = cost;
-  gb.h.xq_cap = xq_cap; gb.h.delta_cap = delta_cap;
   int blocks = tiles < 256 ? tiles : 256;                       // one persistent workgroup per CU
   // macro-steps per work item: about one and a half items per wavefront over the whole launch
   // (the end of an item costs about as many instructions as a step; measured best between one
@@ -862,7 +898,18 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
     g.spi = (g.nS + g.sk - 1) / g.sk;                  // equal parts
     g.sk = (g.nS + g.spi - 1) / g.spi;
     sk_cap = sk_cap > g.sk ? sk_cap : g.sk;
+    // column slabs: as many whole parts as the digit budget holds (a part is at most 8 steps =
+    // 4096 columns, 12 KB per activation row, so one part of eight rows always fits)
+    const int N = g.m.N;
+    g.sp = g.sk;
+    if ((size_t)M * NDIG * N > (size_t)X_LDS_BUDGET) {
+      g.sp = X_LDS_BUDGET / (M * NDIG * g.spi * 512);
+      if (g.sp < 1 || M == 1) return CBK_ERR_UNSUPPORTED;         // (the one-row kernels stage whole rows only)
+    }
+    const int slab_cols = g.sp >= g.sk ? N : g.sp * g.spi * 512;
+    xq_cap = xq_cap > M * NDIG * slab_cols ? xq_cap : M * NDIG * slab_cols;
   }
+  gb.h.xq_cap = xq_cap; gb.h.delta_cap = delta_cap;
   // reduction slots: as many as fit 24 KB, a power of two between 2 and 64
   const int slot_floats = sk_cap * M * 16;
   int nslot = 64;
@@ -871,6 +918,7 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
   gb.h.cq = cost / blocks; gb.h.cr = cost % blocks;
   const size_t lds = (size_t)LUT_BYTES + ZERO_BYTES + CNT_BYTES + xq_cap + (size_t)delta_cap * 4 +
                      (size_t)gb.h.red_floats * 4;
+  if (lds > 160 * 1024) return CBK_ERR_UNSUPPORTED;
   const int bits = gb.mat[0].m.bits;
   if (bits == 6) return launch_mp<6, 16, 128>(gb, lds, blocks, st);   // BLK1632_6: one configuration
   return bits == 2 ? launch_keep<2>(gb, lds, blocks, st) : bits == 3 ? launch_keep<3>(gb, lds, blocks, st)

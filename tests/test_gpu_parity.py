@@ -255,6 +255,24 @@ def test_gemv_five_to_eight_rows_equal_single_rows(case):
             assert torch.equal(ops.gemv(pm, x, bias=bias, out_dtype=torch.float32), y)
 
 
+@pytest.mark.parametrize("case", [(F.BLK1632_4, 4, 128, 16), (F.DENSE4, 4, 128, 0), (F.BLKC, 3, 128, 10)], ids=case_id)
+def test_gemv_rows_longer_than_the_staging_area(case):
+    """Rows whose activation digits do not fit in LDS are staged and multiplied in column slabs, the
+    weights still streamed once: one row of 65536 columns, eight rows of 14336 and 21504 columns, and
+    a matrix with several 16-row tiles per workgroup (more tiles than reduction slots).  Checked
+    against float64 on the dequantised weights and, bit for bit, against the single-row results."""
+    for (K, N, Ms) in ((16, 65536, (1, 2)), (48, 21504, (8, 3)), (8208, 14336, (8,))):
+        pm = F.synth_packed(K, N, case[0], case[1], case[2], case[3], seed=K + N, device=DEV).to_tiled()
+        W = ops.dequant(pm, torch.float32).double()
+        for M in Ms:
+            x = acts(M, N, torch.bfloat16, seed=3 * M).to(DEV)
+            y = ops.gemv(pm, x, out_dtype=torch.float32)
+            ref = x.double() @ W.t()
+            assert float((y.double() - ref).abs().max() / ref.abs().max()) < 2e-5, (K, N, M)
+            for i in range(M):
+                assert torch.equal(ops.gemv(pm, x[i:i + 1], out_dtype=torch.float32)[0], y[i]), (K, N, M, i)
+
+
 @pytest.mark.parametrize("case", [(F.BLK1632_4, 4, 128, 16), (F.BLKC, 3, 64, 10), (F.DENSE4, 4, 128, 0)], ids=case_id)
 def test_linear_ragged_and_extreme_shapes(case):
     """One row, one chunk, row counts off the 16-row and 256-row tiles, column counts off the
