@@ -507,9 +507,18 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     // launch is tens of megabytes, and a request queued behind it would keep every wavefront
     // from decoding until that burst has drained.
     const int n16 = Ns >> 4, xitems = h.M * n16;                  // a multiple of 8
+    // The first two items of a thread (all there are, but for the longest rows) are loaded here
+    // and converted outside the loop further down: inside it the compiler's wait for an item's
+    // loads has to allow for the trip in which they were issued after the weight loads, and so
+    // waits for the weight loads as well; the conversion would start only once the first weights
+    // have arrived instead of running while they are on their way.
+    // (The second item only where its sixteen registers do not push the kernel into scratch.)
+    constexpr bool PRE2 = MP == 1 || (MP == 4 && QB);
     int xit = tid;
-    XLoad xl;
+    XLoad xl, xl2;
     if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, N, col0, n16, xit, MP == 1, gm.par, xl);
+    if (PRE2 && xit + GV_THREADS < xitems)
+      stage_load(gm.x, gm.ldx, m.cs, N, col0, n16, xit + GV_THREADS, MP == 1, gm.par, xl2);
     // Two load buffers swap roles (being decoded, being loaded) by name: copying a buffer would
     // wait for the loads that are still filling it.  One step of loads in flight per wavefront
     // is the measured optimum (sixteen wavefronts per CU already cover the latency; a second
@@ -520,10 +529,13 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     // ---- stage: selector table and counters (once), activation digits and deltas of this matrix
     if (!first) __syncthreads();                                  // previous matrix fully consumed
     first = false;
-    while (xit < xitems) {
-      stage_convert<(!C::DENSE ? 0 : (BITS == 2 ? 2 : 1))>(xl, m.cs != nullptr, h.xdt, N, ch0, n16, xit, MP == 1, xq, delta);
-      xit += GV_THREADS;
-      if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, N, col0, n16, xit, MP == 1, gm.par, xl);
+    constexpr int XORD = !C::DENSE ? 0 : (BITS == 2 ? 2 : 1);
+    if (xit < xitems) stage_convert<XORD>(xl, m.cs != nullptr, h.xdt, N, ch0, n16, xit, MP == 1, xq, delta);
+    if (PRE2 && xit + GV_THREADS < xitems)
+      stage_convert<XORD>(xl2, m.cs != nullptr, h.xdt, N, ch0, n16, xit + GV_THREADS, MP == 1, xq, delta);
+    for (xit += (PRE2 ? 2 : 1) * GV_THREADS; xit < xitems; xit += GV_THREADS) {
+      stage_load(gm.x, gm.ldx, m.cs, N, col0, n16, xit, MP == 1, gm.par, xl);
+      stage_convert<XORD>(xl, m.cs != nullptr, h.xdt, N, ch0, n16, xit, MP == 1, xq, delta);
     }
     __syncthreads();
 
