@@ -892,6 +892,16 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
   (void)workspace; (void)ws_bytes;
   for (int i = n; i < GV_MAX_BATCH; ++i) gb.h.cost_end[i] = cost;
   int blocks = tiles < 256 ? tiles : 256;                       // one persistent workgroup per CU
+  // A workgroup takes whole tiles.  Between one and two tiles per workgroup the launch lasts two
+  // tiles however they are dealt, and dealing two to each of fewer workgroups (384 tiles: 192 x 2
+  // instead of 128 x 2 + 128 x 1) was measured faster as long as at least three quarters of the
+  // CUs still get one (Mistral q,k,v: -1.9 us); with fewer workgroups than that, or more tiles
+  // each, having every CU at work counts for more.  Only where every tile costs the same.
+  {
+    bool same = true;
+    for (int i = 1; i < n; ++i) same = same && gb.mat[i].nS == gb.mat[0].nS;
+    if (same && tiles > 256 && tiles <= 512 && (tiles + 1) / 2 >= 192) blocks = (tiles + 1) / 2;
+  }
   // macro-steps per work item: about one and a half items per wavefront over the whole launch
   // (the end of an item costs about as many instructions as a step; measured best between one
   // and two); a tile is split into at most 16 parts, and into a power of two of them where the
