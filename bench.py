@@ -67,7 +67,7 @@ MIN_WARM_MS = 50.0
 # the same counters read for a device-to-device copy of known size), keyed by
 # (workload, launch grouping, M).  Stored figures from the runs summarised under profiles/, not
 # counters read during a bench run.
-MEASURED_TRAFFIC = {("mistral7b", "phase", 1): 22311131, ("gemma27b", "phase", 1): 43089816}
+MEASURED_TRAFFIC = {("mistral7b", "phase", 1): 22366413, ("gemma27b", "phase", 1): 43134566}
 
 
 def algorithmic_bytes(pm, M, e_x=2, e_y=2):
@@ -342,6 +342,7 @@ def prefill_gemm(torch, F, ops, dev, shapes, names, layout, bits, group, keep, M
             torch.cuda.synchronize()
             ms = e0.elapsed_time(e1) / reps
             err = prefill_parity(torch, ops, pm, x) if parity else None
+            dense_ms = library_dense_gemm_ms(torch, dev, M, K, N, dt, x) if parity else None
             if err is not None:
                 worst = max(worst, err)
                 assert err < 1e-3, f"prefill {name} {K}x{N} M={M}: rel. Frobenius error {err} against the dequantised weights"
@@ -349,6 +350,8 @@ def prefill_gemm(torch, F, ops, dev, shapes, names, layout, bits, group, keep, M
             row = {"matrix": f"{name} {K}x{N}", "ms": round(ms, 4), "tflops": round(2.0 * M * K * N / ms / 1e9, 1)}
             if err is not None:
                 row["rel_fro_vs_dequant_f64"] = float(f"{err:.3g}")
+            if dense_ms is not None:
+                row["library_dense_gemm_tflops"] = round(2.0 * M * K * N / dense_ms / 1e9, 1)
             rows.append(row)
             bpw = pm.bpw()
             del pm, x, y, ws
@@ -366,6 +369,25 @@ def prefill_gemm(torch, F, ops, dev, shapes, names, layout, bits, group, keep, M
                          "how": "192 sampled weight rows x all tokens of every timed matrix, float32 output against "
                                 "x.double() @ dequant(W).double().T"}
     return out
+
+
+def library_dense_gemm_ms(torch, dev, M, K, N, dt, x, reps=10, warm=5):
+    """The vendor library's dense GEMM (torch.matmul) on an unpacked matrix of the same shape and
+    activation type: what the GPU does with 16-bit weights that need no decoding (five times the
+    weight bytes).  A figure to read the packed kernel's against, not part of the path."""
+    w = torch.randn(K, N, device=dev, generator=torch.Generator(device=dev).manual_seed(K)).mul_(0.02).to(dt)
+    for _ in range(warm):
+        y = x @ w.t()
+    torch.cuda.synchronize()
+    st = torch.cuda.current_stream()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(st)
+    for _ in range(reps):
+        y = x @ w.t()
+    e1.record(st)
+    torch.cuda.synchronize()
+    del w, y
+    return e0.elapsed_time(e1) / reps
 
 
 # ------------------------------------------------------------------ ceilings and CPU baseline
