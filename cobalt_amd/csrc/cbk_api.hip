@@ -16,11 +16,11 @@ bool gemv_same_config(const DMat&, const DMat&);
 size_t gemv_fast_workspace(const DMat&, int M);
 constexpr int kMaxBatch = 8;
 int launch_act_mul(const void* t, int tdt, int64_t ldt, void* y, int ydt, int64_t ldy, int M, int K2, int act,
-                   const void* bias, hipStream_t st);
+                   const void* bias, hipStream_t st, bool halves = false);
 int launch_gemm(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*,
                 hipStream_t);
 int launch_gemm_big(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*, void*, size_t,
-                    hipStream_t);
+                    hipStream_t, bool halves = false);
 size_t gemm_big_workspace(const DMat&, int M);
 int launch_pack(const DMat&, const void* mask, const void* q, const void* scale, const void* zero, int zero_f16,
                 int fix_zero, int* status, hipStream_t);
@@ -505,6 +505,16 @@ int cbk_linear_act(const cbk_desc* in, const void* x, int x_dtype, int M, int64_
   if (!workspace || ((uintptr_t)workspace & 255) || workspace_bytes < mid + cbk_workspace_bytes(in, M))
     return CBK_ERR_WORKSPACE;
   const int tdt = act_mid_dtype(M, y_dtype);
+  if (M > 8 && m.cs_rows == 2 && gemm_big_takes(m, M)) {
+    // the tile kernel leaves t as two halves (gate outputs, then up outputs): a workgroup holds
+    // one parity of the rows, and interleaved it could only store single elements
+    rc = check_io(x, x_dtype, M, ldx, workspace, tdt, m.K, m.N, m.K);
+    if (rc) return rc;
+    rc = launch_gemm_big(m, x, x_dtype, M, ldx, workspace, tdt, m.K, nullptr, (uint8_t*)workspace + mid,
+                         workspace_bytes - mid, (hipStream_t)stream, true);
+    if (rc) return rc;
+    return launch_act_mul(workspace, tdt, m.K, y, y_dtype, ldy, M, m.K / 2, act, bias, (hipStream_t)stream, true);
+  }
   rc = cbk_linear(in, x, x_dtype, M, ldx, workspace, tdt, m.K, nullptr, (uint8_t*)workspace + mid,
                   workspace_bytes - mid, stream);                  // the activation kernel adds the bias
   if (rc) return rc;

@@ -58,6 +58,8 @@ struct GbArgs {
   int64_t ldy;
   const void* bias;
   int tiles_t, tiles_r;
+  int halves;              // gate/up matrix (par): 1 = write the gate outputs to columns [0, K/2) and the up outputs to
+                           // [K/2, K) of y instead of interleaving them (whole 16-byte stores; for cbk_linear_act)
   int ti;                  // 32-token blocks per wavefront: 4 (256-token tiles) or 1 (64-token tiles)
   // par = 1: gate/up matrix, two col_scale vectors by row parity.  A workgroup then takes 256
   // rows of one parity out of 512 (rows r0 + 2 i + p), and X' of that parity's vector, which
@@ -490,6 +492,19 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(GbArgs a) {
     b.ldy = a.part_ld;
     b.bias = nullptr;
     gb_epilogue<CBK_F32, 1, TI>(b, acc, smem, lane, wave, tok0, row0, rs);
+    return;
+  }
+  if (PAR == 1 && a.halves) {
+    // this workgroup's rows are one parity of the matrix: consecutive columns of that half of y
+    GbArgs b = a;
+    const int K2 = a.m.K >> 1;
+    b.y = (uint8_t*)a.y + (size_t)pp * K2 * (a.ydt == CBK_F32 ? 4 : 2);
+    b.m.K = K2;
+    b.bias = nullptr;
+    const int hrow0 = (r0 >> 1) + 128 * wr;
+    if (a.ydt == CBK_F32) gb_epilogue<CBK_F32, 1, TI>(b, acc, smem, lane, wave, tok0, hrow0, rs);
+    else if (a.ydt == CBK_F16) gb_epilogue<CBK_F16, 1, TI>(b, acc, smem, lane, wave, tok0, hrow0, rs);
+    else gb_epilogue<CBK_BF16T, 1, TI>(b, acc, smem, lane, wave, tok0, hrow0, rs);
     return;
   }
   if (a.ydt == CBK_F32) gb_epilogue<CBK_F32, kstep, TI>(a, acc, smem, lane, wave, tok0, row0, rs);

@@ -180,8 +180,10 @@ size_t gemm_big_workspace(const DMat& m, int M) {
   return b;
 }
 
+// halves: a gate/up matrix's outputs as two halves of y (GbArgs::halves) instead of interleaved
 int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
-                    const void* bias, void* ws, size_t ws_bytes, hipStream_t st) {
+                    const void* bias, void* ws, size_t ws_bytes, hipStream_t st, bool halves) {
+  if (halves && (m.cs_rows != 2 || (m.K & 1) || bias)) return CBK_ERR_UNSUPPORTED;
   if (family_of(m.layout) == FAM_SPARSE) return CBK_ERR_UNSUPPORTED;
   // q|k|v ranges off the row-tile grid: the caller passes them one by one
   if (m.cs_rows == 3 && (m.cs_split0 % GB_R || (m.cs_split0 + m.cs_split1) % GB_R)) return CBK_ERR_UNSUPPORTED;
@@ -205,6 +207,7 @@ int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, v
   GbArgs a;
   a.m = m; a.xp = (const uint16_t*)ws; a.M = M; a.Npad = Npad; a.y = y; a.ydt = ydt; a.ldy = ldy; a.bias = bias;
   a.par = par; a.xps = (size_t)Mpad * Npad;
+  a.halves = halves ? 1 : 0;
   a.row_scale = row_scale; a.rss = Mpad;
   a.vs0 = m.cs_rows == 3 ? m.cs_split0 : 0x7fffffff;
   a.vs1 = m.cs_rows == 3 ? m.cs_split0 + m.cs_split1 : 0x7fffffff;
