@@ -271,6 +271,21 @@ def test_gemv_rows_longer_than_the_staging_area(case):
             assert float((y.double() - ref).abs().max() / ref.abs().max()) < 2e-5, (K, N, M)
             for i in range(M):
                 assert torch.equal(ops.gemv(pm, x[i:i + 1], out_dtype=torch.float32)[0], y[i]), (K, N, M, i)
+    # a gate/up matrix stages two scaled copies of every activation row: four rows of 5376 columns
+    # are eight staged rows, more than the staging area holds at once
+    K, N = 64, 5376
+    pm = F.synth_packed(K, N, case[0], case[1], case[2], case[3], seed=5, device=DEV)
+    cs = (torch.rand(2, N, generator=torch.Generator().manual_seed(9)) + 0.5).half().to(DEV)
+    pm = F.from_arrays(pm.array("data"), pm.array("scale"), pm.array("zero"), cs, K, N, case[0], case[1], case[2],
+                       case[3] or None, device=DEV).to_tiled()
+    W = ops.dequant(pm, torch.float32).double()
+    for M in (4, 7):
+        x = acts(M, N, torch.bfloat16, seed=M).to(DEV)
+        y = ops.gemv(pm, x, out_dtype=torch.float32)
+        ref = x.double() @ W.t()
+        assert float((y.double() - ref).abs().max() / ref.abs().max()) < 2e-5, (K, N, M)
+        for i in range(M):
+            assert torch.equal(ops.gemv(pm, x[i:i + 1], out_dtype=torch.float32)[0], y[i]), (K, N, M, i)
 
 
 @pytest.mark.parametrize("case", [(F.BLK1632_4, 4, 128, 16), (F.BLKC, 3, 64, 10), (F.DENSE4, 4, 128, 0)], ids=case_id)
