@@ -169,8 +169,12 @@ int cbk_unpack(const cbk_desc* d, void* q, void* mask_bits, void* stream);
 
 /* Decode path, 1 <= M <= 16: y[m, k] = sum_j x[m, j] * W_hat[k, j] (+ bias[k]).
  * x is [M, ldx] fp16 or bf16, y is [M, ldy] in y_dtype (f32 / f16 / bf16), bias is NULL or
- * K values of y_dtype.  Replaces the harness entry `gemv` (test_gemv.cu:187-199) and
- * cbk::gemv_rows (cobalt_gemv.cuh:1196-1213); unlike those it applies col_scale itself. */
+ * K values of y_dtype.  Up to eight activation rows share one pass over the weights on the
+ * matrix-core kernel, whatever the row length (two to eight rows of a long row are staged in
+ * column slabs); more rows, or configurations that kernel takes four rows of at a time, are
+ * passes over the weights.  Row m of the result does not depend on M.  Replaces the harness
+ * entry `gemv` (test_gemv.cu:187-199) and cbk::gemv_rows (cobalt_gemv.cuh:1196-1213); unlike
+ * those it applies col_scale itself. */
 int cbk_gemv(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
              void* y, int y_dtype, int64_t ldy, const void* bias,
              void* workspace, size_t workspace_bytes, void* stream);
