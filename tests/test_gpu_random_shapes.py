@@ -81,3 +81,18 @@ def test_linear_act_random_shapes(case):
             err = rel_fro(_np(y), ref.astype(np.float32))
             # above 128 rows the intermediate is rounded to the output type before the activation
             assert err < (4e-3 if M > 128 else TOL), f"{case_id(case)} {K}x{N} M={M} tiled={tiled} {act}: {err}"
+
+
+def test_gemv_between_one_and_two_tiles_per_workgroup():
+    """257..512 row tiles: where at least 192 workgroups still get work, two tiles go to each of
+    half as many workgroups; below that (and above 512 tiles) the tiles are dealt over 256.  Same
+    results either way: against float64 on the dequantised weights, and batched against single calls."""
+    for K in (4112, 5376, 6144, 8192, 8208):
+        N = 384
+        pm = F.synth_packed(K, N, F.BLK1632_4, 4, 128, 16, seed=K, device=DEV).to_tiled()
+        W = ops.dequant(pm, torch.float32).double()
+        x = acts(2, N, torch.float16, seed=K % 89).to(DEV)
+        y = ops.gemv(pm, x, out_dtype=torch.float32)
+        ref = x.double() @ W.t()
+        assert float((y.double() - ref).abs().max() / ref.abs().max()) < 2e-5, K
+        assert torch.equal(ops.gemv(pm, x[1:2], out_dtype=torch.float32)[0], y[1])
