@@ -458,7 +458,7 @@ int cbk_gemm_static(const cbk_desc* in, const void* x, int x_dtype, int M, int64
 
 int cbk_linear(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ldx, void* y, int y_dtype,
                int64_t ldy, const void* bias, void* workspace, size_t workspace_bytes, void* stream) {
-  // up to 8 rows (two passes of the decode kernel) the weights are streamed faster than the
+  // up to 8 rows (one or two passes of the decode kernel) the weights are streamed faster than the
   // prefill kernel's 64-token tile decodes them (14336 x 4096: 28 us against 31 us; 54 us at 16 rows)
   if (M <= 8) return cbk_gemv(in, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, workspace, workspace_bytes, stream);
   cbk_desc d;
