@@ -7,7 +7,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libcbk_hip.so")
 SOURCES = ["cbk_api.hip", "cbk_dequant.hip", "cbk_gemv_generic.hip", "cbk_gemv.hip", "cbk_gemm.hip", "cbk_gemm_big.hip",
-           "cbk_gemm_big_b2.hip", "cbk_gemm_big_b3.hip", "cbk_gemm_big_b4.hip", "cbk_gemm_big_b6.hip", "cbk_act.hip", "cbk_pack.hip"]
+           "cbk_gemm_big_b2.hip", "cbk_gemm_big_b3.hip", "cbk_gemm_big_b4.hip", "cbk_gemm_big_b6.hip"] + [
+           f"cbk_gemm_big_b{b}_t{t}.hip" for b in (2, 3, 4) for t in (1, 2, 4)] + ["cbk_act.hip", "cbk_pack.hip"]
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-shared", "-std=c++17",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-command-line-argument"]

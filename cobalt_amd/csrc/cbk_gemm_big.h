@@ -168,7 +168,8 @@ __device__ inline void gb_epilogue(const GbArgs& a, v16f (&acc)[TI][4], uint8_t*
 // 3: one col_scale vector, column range split over several workgroups (GbArgs::nsplit).
 // Three instantiations rather than run-time switches: the schedule of the main loop is tuned
 // to the instruction and measurably shifts with every value that is added to it.
-// TI: 32-token blocks per wavefront.  4: the 256-token tile described above.  1: a 64-token tile
+// TI: 32-token blocks per wavefront.  4: the 256-token tile described above.  2: a 128-token tile
+// (each wavefront 64 tokens x 128 rows) for calls of 65 to 128 activation rows.  1: a 64-token tile
 // (each wavefront 32 tokens x 128 rows) for calls of at most 64 activation rows, whose time is
 // the weight decode: a quarter of the matrix instructions per stage, the same decode.
 template <int BITS, int KEEP, int GRP, int PAR, int TI = 4>
@@ -535,15 +536,17 @@ static int launch_big_ti(const GbArgs& a, int blocks, hipStream_t st) {
 
 template <int BITS, int KEEP, int GRP>
 static int launch_big_cfg(const GbArgs& a, int blocks, hipStream_t st) {
-  return a.ti == 1 ? launch_big_ti<BITS, KEEP, GRP, 1>(a, blocks, st) : launch_big_ti<BITS, KEEP, GRP, 4>(a, blocks, st);
+  return a.ti == 1 ? launch_big_ti<BITS, KEEP, GRP, 1>(a, blocks, st)
+       : a.ti == 2 ? launch_big_ti<BITS, KEEP, GRP, 2>(a, blocks, st) : launch_big_ti<BITS, KEEP, GRP, 4>(a, blocks, st);
 }
 
-// the (keep, group) instantiations of one code width
-template <int BITS>
+// the (keep, group) instantiations of one code width and one token tile (a translation unit each:
+// the 32 kernels of such a set are what one compiler process takes a minute and a half for)
+template <int BITS, int TI>
 static int launch_big_bits(const GbArgs& a, int keep, int group, int blocks, hipStream_t st) {
 #define CBK_GB_CASE(KEEP)                                                                            \
-  case KEEP: return group == 64 ? launch_big_cfg<BITS, KEEP, 64>(a, blocks, st)                      \
-                                : launch_big_cfg<BITS, KEEP, 128>(a, blocks, st);
+  case KEEP: return group == 64 ? launch_big_ti<BITS, KEEP, 64, TI>(a, blocks, st)                   \
+                                : launch_big_ti<BITS, KEEP, 128, TI>(a, blocks, st);
   switch (keep) {
     CBK_GB_CASE(0) CBK_GB_CASE(10) CBK_GB_CASE(16) CBK_GB_CASE(23)
     default: return CBK_ERR_UNSUPPORTED;

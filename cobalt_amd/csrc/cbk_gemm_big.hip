@@ -134,7 +134,7 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float* par
 // the price of the float32 partial tiles (written and read once).  Times in microseconds from
 // measurements of this kernel: 1.7 per stage and 10 per workgroup, 4 TB/s for the partials.
 // 32-token blocks per wavefront: calls of at most 64 activation rows take the 64-token tile
-static inline int gb_ti(int M) { return M <= 64 ? 1 : 4; }
+static inline int gb_ti(int M) { return M <= 64 ? 1 : M <= 128 ? 2 : 4; }
 
 // the matrices the byte-permute instantiations take (the others go through the generic reader,
 // whose launches are never split)
@@ -152,7 +152,7 @@ static int gb_nsplit(const DMat& m, int M) {
   const int T = 64 * gb_ti(M);
   const int tiles = ((M + T - 1) / T) * ((m.K + GB_R - 1) / GB_R);
   const int nst = gb_npad(m.N) / GB_K;
-  const double t_stage = T == 64 ? 1.1 : 1.7, t_wg = T == 64 ? 8.0 : 10.0;   // 64-token stage: bound by the weight loads' latency
+  const double t_stage = T == 64 ? 1.1 : T == 128 ? 1.3 : 1.7, t_wg = T == 64 ? 8.0 : 10.0;   // 64-token stage: bound by the weight loads' latency
   int best = 1;
   double t1 = 0, best_t = 0;
   for (int s = 1; s <= 16; ++s) {

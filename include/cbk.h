@@ -192,7 +192,7 @@ int cbk_gemv_batch(int n, const cbk_desc* descs, const void* const* xs, const in
                    int x_dtype, int M, void* const* ys, const int64_t* ldys, int y_dtype,
                    const void* const* biases, void* workspace, size_t workspace_bytes, void* stream);
 
-/* Prefill path, any M >= 1 (256-token tiles; a 64-token tile up to 64 rows).  Same contract as
+/* Prefill path, any M >= 1 (256-token tiles; a 128-token tile up to 128 rows, a 64-token tile up to 64).  Same contract as
  * cbk_gemv; activations are carried as fp16 inside, a token whose values leave fp16's range
  * scaled by a power of two on the way in and back on the way out.  The survivor-stream layouts
  * (SPARSE4, SPARSE4X, SPARSE4E) are re-packed for the call, above 16 rows, into the dense 4-bit
