@@ -129,13 +129,6 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float* par
   }
 }
 
-// How many workgroups share one output tile.  A launch of fewer tiles than a multiple of the
-// 256 CUs leaves CUs idle for a whole tile time; cutting the column range gives them work at
-// the price of the float32 partial tiles (written and read once).  Times in microseconds from
-// measurements of this kernel: 1.7 per stage and 10 per workgroup, 4 TB/s for the partials.
-// 32-token blocks per wavefront: calls of at most 64 activation rows take the 64-token tile
-static inline int gb_ti(int M) { return M <= 64 ? 1 : M <= 128 ? 2 : 4; }
-
 // the matrices the byte-permute instantiations take (the others go through the generic reader,
 // whose launches are never split)
 static bool gb_fast(const DMat& m) {
@@ -147,35 +140,56 @@ static bool gb_fast(const DMat& m) {
   return fam == FAM_DENSE;
 }
 
-static int gb_nsplit(const DMat& m, int M) {
-  if (m.cs_rows > 1 || !gb_fast(m)) return 1;
-  const int T = 64 * gb_ti(M);
+// Token tile and split of the column range of a call.
+//  * A launch of fewer tiles than a multiple of the 256 CUs leaves CUs idle for a whole tile
+//    time; cutting the column range over several workgroups per output tile gives them work at
+//    the price of the float32 partial tiles (written and read once).
+//  * Calls of at most 64 / 128 activation rows take the 64- / 128-token tile.  Larger calls
+//    take the 256-token tile unless the model below gives the 128-token tile the shorter time,
+//    which it does for small matrices (4096 x 4096 at 256 to 2048 rows: 16 to 128 tiles of 256
+//    tokens): twice the tiles, each 0.8 of the time.
+// Times in microseconds from measurements of this kernel: per 64-column stage 1.1 / 1.35 / 1.7
+// for the three tiles (the 64-token stage is bound by the weight loads' latency), 8 - 10 per
+// workgroup outside the stage loop, 4 TB/s for the partial tiles.  Over 24 measured calls
+// (eight shapes, 256 / 512 / 2048 rows) the choice is within 2 % of the faster tile; always
+// taking the 256-token tile loses 6 % on average and up to 34 %.
+struct GbPlan { int ti, nsplit; double t; };
+static GbPlan gb_plan_ti(const DMat& m, int M, int ti) {
+  const int T = 64 * ti;
   const int tiles = ((M + T - 1) / T) * ((m.K + GB_R - 1) / GB_R);
   const int nst = gb_npad(m.N) / GB_K;
-  const double t_stage = T == 64 ? 1.1 : T == 128 ? 1.3 : 1.7, t_wg = T == 64 ? 8.0 : 10.0;   // 64-token stage: bound by the weight loads' latency
-  int best = 1;
-  double t1 = 0, best_t = 0;
-  for (int s = 1; s <= 16; ++s) {
+  const double t_stage = ti == 1 ? 1.1 : ti == 2 ? 1.35 : 1.7, t_wg = ti == 1 ? 8.0 : 10.0;
+  GbPlan best{ti, 1, 0.0};
+  double t1 = 0;
+  const bool may_split = m.cs_rows <= 1 && gb_fast(m);
+  for (int s = 1; s <= (may_split ? 16 : 1); ++s) {
     const int per = ((nst + s - 1) / s + 3) / 4 * 4;                // stages per part, a multiple of 4
     if (s > 1 && (s - 1) * per >= nst) continue;                    // a part would be empty
     const double rounds = (double)((tiles * s + 255) / 256);
     double t = rounds * (per * t_stage + t_wg);
     if (s > 1) t += 2.0 * s * (double)M * m.K * 4 / 4.0e6 + 5.0;
-    if (s == 1) t1 = best_t = t;
-    else if (t < best_t) { best = s; best_t = t; }
+    if (s == 1) { t1 = t; best.t = t; }
+    else if (t < best.t) { best.nsplit = s; best.t = t; }
   }
-  if (best_t > 0.93 * t1) best = 1;                                 // not worth a second kernel
+  if (best.t > 0.93 * t1) { best.nsplit = 1; best.t = t1; }         // not worth a second kernel
   return best;
+}
+static GbPlan gb_plan(const DMat& m, int M) {
+  if (M <= 64) return gb_plan_ti(m, M, 1);
+  if (M <= 128) return gb_plan_ti(m, M, 2);
+  const GbPlan p4 = gb_plan_ti(m, M, 4), p2 = gb_plan_ti(m, M, 2);
+  return p2.t < p4.t ? p2 : p4;
 }
 
 static inline size_t gb_kpad(int K) { return (size_t)(K + 7) / 8 * 8; }
 
 size_t gemm_big_workspace(const DMat& m, int M) {
-  const size_t T = 64 * gb_ti(M), mpad = (size_t)(M + T - 1) / T * T;
+  const GbPlan plan = gb_plan(m, M);
+  const size_t T = 64 * plan.ti, mpad = (size_t)(M + T - 1) / T * T;
   const size_t nv = m.cs_rows > 1 ? m.cs_rows : 1;
   size_t b = (nv * mpad * gb_npad(m.N) * 2 + 255) & ~(size_t)255;     // X', one per col_scale vector
   b += (nv * mpad * 4 + 255) & ~(size_t)255;                          // and its row scales
-  const int ns = gb_nsplit(m, M);
+  const int ns = plan.nsplit;
   if (ns > 1) b += ((size_t)ns * M * gb_kpad(m.K) * 4 + 255) & ~(size_t)255;
   return b;
 }
@@ -190,7 +204,8 @@ int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, v
   if (ydt != CBK_F32 && ydt != CBK_F16 && ydt != CBK_BF16T) return CBK_ERR_DTYPE;
   if (!ws || ws_bytes < gemm_big_workspace(m, M)) return CBK_ERR_WORKSPACE;
   if ((uintptr_t)ws & 255) return CBK_ERR_ALIGN;
-  const int T = 64 * gb_ti(M);
+  const GbPlan plan = gb_plan(m, M);
+  const int T = 64 * plan.ti;
   const int Mpad = (M + T - 1) / T * T;
   const int Npad = gb_npad(m.N);
   const int par = m.cs_rows == 2 ? 1 : 0;
@@ -212,12 +227,12 @@ int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, v
   a.vs0 = m.cs_rows == 3 ? m.cs_split0 : 0x7fffffff;
   a.vs1 = m.cs_rows == 3 ? m.cs_split0 + m.cs_split1 : 0x7fffffff;
   const int nst_all = Npad / GB_K;
-  a.nsplit = gb_nsplit(m, M);
+  a.nsplit = plan.nsplit;
   a.nst_part = ((nst_all + a.nsplit - 1) / a.nsplit + 3) / 4 * 4;
   a.part_ld = (int64_t)gb_kpad(m.K);
   a.part_stride = (size_t)M * gb_kpad(m.K);
   a.part = (float*)((uint8_t*)ws + xbytes + sbytes);
-  a.ti = gb_ti(M);
+  a.ti = plan.ti;
   a.tiles_t = (M + T - 1) / T;
   a.tiles_r = par ? 2 * ((m.K + 2 * GB_R - 1) / (2 * GB_R)) : (m.K + GB_R - 1) / GB_R;
   const int nb = a.tiles_t * a.tiles_r * a.nsplit;
@@ -234,7 +249,7 @@ int launch_gemm_big(const DMat& m, const void* x, int xdt, int M, int64_t ldx, v
     rc = launch_gemm_big_b6(a, blocks, st);
   }
   if (rc == CBK_ERR_UNSUPPORTED) {
-    if (a.nsplit > 1) return CBK_ERR_UNSUPPORTED;                   // (gb_nsplit only splits what the cases above take)
+    if (a.nsplit > 1) return CBK_ERR_UNSUPPORTED;                   // (only what the cases above take is ever split)
     rc = launch_big_cfg<0, 0, 128>(a, blocks, st);                  // generic reader
   }
   if (rc == CBK_OK && a.nsplit > 1) {
