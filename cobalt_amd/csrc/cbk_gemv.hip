@@ -26,7 +26,10 @@
 // blocks of one chunk instead of on four chunks (see block_split_capable below), so that
 // every MFMA serves four activation rows (M = 5..8: two MFMAs per decoded fragment, one weight
 // pass); sums are formed in the same order as for M = 1, so a row's result does not depend on M.
-// The activation digits and the byte-permute selector table live in LDS for the whole launch.
+// The activation digits and the byte-permute selector table live in LDS for the whole launch;
+// where the digits of all rows of a matrix do not fit (two to eight activation rows of a long
+// row) they are staged one column slab at a time, whole split-K parts per slab, while the partial
+// sums of the tiles wait in their LDS slots: the weights are still read once.
 //
 // Expansion of the bitmap.  For one mask byte (8 columns, r survivors before it in its
 // 32-column block) the survivor codes r .. r+7 are shifted out of the block's code bits,
