@@ -11,7 +11,7 @@ SOURCES = ["cbk_api.hip", "cbk_dequant.hip", "cbk_gemv_generic.hip", "cbk_gemv.h
            f"cbk_gemm_big_b{b}_t{t}.hip" for b in (2, 3, 4) for t in (1, 2, 4)] + ["cbk_act.hip", "cbk_pack.hip"]
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-shared", "-std=c++17",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-         "-Wno-unused-command-line-argument"]
+         "-Wno-unused-command-line-argument", "-Wno-inline-asm"]
 
 
 def build_lib(verbose=True, extra=()):

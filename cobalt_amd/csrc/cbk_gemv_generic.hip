@@ -20,20 +20,23 @@ __device__ inline float wave_sum(float v) {
 
 constexpr int SP4_MAX_G = 512;     // groups per row whose offsets the SPARSE4 path keeps in LDS (N <= 65536)
 
-template <int XDT, int M>
+// PATH picks the reader at compile time (one kernel per reader keeps each one's register count,
+// and with it the number of resident wavefronts, its own): 0 DENSE8, 1 the other fixed-stride
+// layouts, 2 survivor streams with group offsets at hand, 3 SPARSE4 rows with more groups than
+// the offset table holds.
+template <int XDT, int M, int PATH>
 __global__ __launch_bounds__(256) void gemv_generic_kernel(DMat m, const void* x, int64_t ldx, void* y,
                                                            int ydt, int64_t ldy, const void* bias) {
-  __shared__ uint32_t sp4_goff[4 * SP4_MAX_G];
+  __shared__ uint32_t sp4_goff[PATH == 2 ? 4 * SP4_MAX_G : 4];
   const int lane = threadIdx.x & 63;
   const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
   const int nwaves = (gridDim.x * blockDim.x) >> 6;
-  const int fam = family_of(m.layout);
   for (int k = wave; k < m.K; k += nwaves) {
     float acc[M];
 #pragma unroll
     for (int i = 0; i < M; ++i) acc[i] = 0.f;
     const uint16_t* cs = m.cs ? m.cs + (size_t)cs_row_of(m, k) * m.N : nullptr;
-    if (m.layout == CBK_DENSE8) {
+    if constexpr (PATH == 0) {
       // one byte per column: a lane takes a 32-column block as two 16-byte units of codes and
       // whole vectors of activations and column scales
       const RowView row = row_view(m, k);
@@ -72,7 +75,7 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(DMat m, const void* x
 #pragma unroll
         for (int i = 0; i < M; ++i) acc[i] = fmaf(s, part[i], acc[i]);
       }
-    } else if (fam != FAM_SPARSE) {
+    } else if constexpr (PATH == 1) {
       const RowView row = row_view(m, k);
       for (int t = lane; t < m.N / BLOCK; t += 64) {
         int q[32];
@@ -95,7 +98,7 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(DMat m, const void* x
 #pragma unroll
         for (int i = 0; i < M; ++i) acc[i] = fmaf(s, part[i], acc[i]);
       }
-    } else if (m.layout != CBK_SPARSE4 || m.G <= SP4_MAX_G) {
+    } else if constexpr (PATH == 2) {
       // The byte offset of every group's codes is in the row's header (SPARSE4X / SPARSE4E) or
       // is summed up here from the bitmap (SPARSE4: a prefix sum of the groups' byte counts over
       // the wavefront, kept in LDS), so a lane can take one 32-column block: its survivors'
@@ -243,8 +246,8 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(DMat m, const void* x
   }
 }
 
-template <int XDT>
-static int launch_m(const DMat& m, const void* x, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
+template <int XDT, int PATH>
+static int launch_p(const DMat& m, const void* x, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
                     const void* bias, hipStream_t st) {
   const int blocks = (m.K + 3) / 4 < 4096 ? (m.K + 3) / 4 : 4096;
   const dim3 grid(blocks), blk(256);
@@ -254,13 +257,22 @@ static int launch_m(const DMat& m, const void* x, int M, int64_t ldx, void* y, i
     const void* xs = (const uint8_t*)x + (size_t)m0 * ldx * 2;
     void* ys = (uint8_t*)y + (size_t)m0 * ldy * (ydt == CBK_F32 ? 4 : 2);
     switch (mc) {
-      case 1: hipLaunchKernelGGL((gemv_generic_kernel<XDT, 1>), grid, blk, 0, st, m, xs, ldx, ys, ydt, ldy, bias); break;
-      case 2: hipLaunchKernelGGL((gemv_generic_kernel<XDT, 2>), grid, blk, 0, st, m, xs, ldx, ys, ydt, ldy, bias); break;
-      case 3: hipLaunchKernelGGL((gemv_generic_kernel<XDT, 3>), grid, blk, 0, st, m, xs, ldx, ys, ydt, ldy, bias); break;
-      default: hipLaunchKernelGGL((gemv_generic_kernel<XDT, 4>), grid, blk, 0, st, m, xs, ldx, ys, ydt, ldy, bias); break;
+      case 1: hipLaunchKernelGGL((gemv_generic_kernel<XDT, 1, PATH>), grid, blk, 0, st, m, xs, ldx, ys, ydt, ldy, bias); break;
+      case 2: hipLaunchKernelGGL((gemv_generic_kernel<XDT, 2, PATH>), grid, blk, 0, st, m, xs, ldx, ys, ydt, ldy, bias); break;
+      case 3: hipLaunchKernelGGL((gemv_generic_kernel<XDT, 3, PATH>), grid, blk, 0, st, m, xs, ldx, ys, ydt, ldy, bias); break;
+      default: hipLaunchKernelGGL((gemv_generic_kernel<XDT, 4, PATH>), grid, blk, 0, st, m, xs, ldx, ys, ydt, ldy, bias); break;
     }
   }
   return hipGetLastError() == hipSuccess ? CBK_OK : CBK_ERR_HIP;
+}
+
+template <int XDT>
+static int launch_m(const DMat& m, const void* x, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
+                    const void* bias, hipStream_t st) {
+  if (m.layout == CBK_DENSE8) return launch_p<XDT, 0>(m, x, M, ldx, y, ydt, ldy, bias, st);
+  if (family_of(m.layout) != FAM_SPARSE) return launch_p<XDT, 1>(m, x, M, ldx, y, ydt, ldy, bias, st);
+  if (m.layout != CBK_SPARSE4 || m.G <= SP4_MAX_G) return launch_p<XDT, 2>(m, x, M, ldx, y, ydt, ldy, bias, st);
+  return launch_p<XDT, 3>(m, x, M, ldx, y, ydt, ldy, bias, st);
 }
 
 int launch_gemv_generic(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt,
