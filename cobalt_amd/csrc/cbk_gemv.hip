@@ -774,6 +774,252 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
   }
 }
 
+// ------------------------------------------------------------------ survivor-stream rows
+// SPARSE4 / SPARSE4X / SPARSE4E at one to four activation rows.  Rows of different lengths do not
+// tile, so there is no matrix-core kernel for them; but the float row kernel spends about fourteen
+// vector instructions per column (pruned ones included) and is bound by that.  This kernel keeps
+// the arithmetic of the kernel above (activation digits in LDS, byte-permute expansion of the
+// bitmap into signed bytes q - zero, exact int32 sums per digit, one float FMA per 32-column block
+// with scale * delta) and forms the sums with v_dot4_i32_i8: about four instructions per column.
+// One wavefront per weight row, one lane per 32-column block, a workgroup of four wavefronts
+// stages the digits once and then walks rows.
+// Reference semantics: cbk::gemv_sparse4 (src/cobaltkernel/csrc/cobalt_gemv.cuh:216-301).
+constexpr int ST_WAVES = 16;
+constexpr int ST_THREADS = ST_WAVES * 64;
+constexpr int ST_LUT_LANES = 4;
+constexpr int ST_LUT_BYTES = 256 * ST_LUT_LANES * 8;
+constexpr int ST_X_BUDGET = 96 * 1024;        // digits of all activation rows of a pass
+
+// What a lane fetches for one (row, 32-column block) item, in two dependent steps: the group's mask
+// words and code offset, then (at an address made from those) the block's codes and the group's
+// scale and zero point.
+struct StMask { uint4 gmk; uint32_t goffv; };
+struct StCodes { uint32_t e[6]; uint32_t mw, sh, sraw, z; };
+
+template <int M>
+__global__ __launch_bounds__(ST_THREADS) void gemv_stream_kernel(DMat m, const uint16_t* x, int64_t ldx, int xdt,
+                                                                 void* y, int ydt, int64_t ldy, const void* bias) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  uint2* lut = (uint2*)smem;
+  const int N = m.N, NCH = N >> 7, NB = N >> 5;
+  int8_t* xq = (int8_t*)(smem + ST_LUT_BYTES);
+  float* delta = (float*)(xq + (size_t)M * NDIG * N);
+  uint32_t* goffs = (uint32_t*)(delta + M * (NCH + 4));          // [ST_WAVES][G], SPARSE4 only
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  if (tid < 256) {
+    const uint2 e = make_selectors((uint32_t)tid, 0);
+#pragma unroll
+    for (int j = 0; j < ST_LUT_LANES; ++j) lut[tid * ST_LUT_LANES + j] = e;
+  }
+  const int n16 = N >> 4, xitems = M * n16;                      // a multiple of 8
+  for (int it = tid; it < xitems; it += ST_THREADS) {
+    XLoad xl;
+    stage_load(x, ldx, m.cs, N, 0, n16, it, M == 1, 0, xl);
+    stage_convert<0>(xl, m.cs != nullptr, xdt, N, 0, n16, it, M == 1, xq, delta);
+  }
+  __syncthreads();
+  const bool has_goff = m.layout != CBK_SPARSE4;
+  const int hdr = ((N >> 3) + (has_goff ? ((m.G * 2 + 15) & ~15) : 0) + 15) & ~15;
+  uint32_t* lgoff = goffs + wave * m.G;
+  const uint32_t l4 = lane & (ST_LUT_LANES - 1);
+  // this wavefront's rows k0, k0 + ks, ...; its items are (row, pass over the row's blocks), in order
+  const int k0 = (int)blockIdx.x * ST_WAVES + wave, ks = (int)gridDim.x * ST_WAVES;
+  if (k0 >= m.K) return;                                          // (after the only barrier)
+  const int nrows = (m.K - k0 + ks - 1) / ks;
+  const int nt = (NB + 63) >> 6, nitems = nrows * nt;
+  const uint8_t* const m_data = m.data;
+  const uint32_t* const m_row_off = m.row_off;
+
+  // Items run through a three-deep pipeline: while item q is multiplied, the codes of item q + 1
+  // and the mask words of item q + 2 are on their way.  Positions past the end repeat the last item.
+  struct Pos { int k, it; uint32_t ro; };
+  auto next_pos = [&](Pos& p) {
+    if (p.it + 1 < nt) { ++p.it; return; }
+    if (p.k + ks < m.K) { p.k += ks; p.it = 0; p.ro = m_row_off[p.k]; }
+  };
+  auto block_of = [&](const Pos& p) { const int t = lane + 64 * p.it; return t < NB ? t : NB - 1; };
+  auto issue_mask = [&](const Pos& p, StMask& a) {
+    const int g = block_of(p) >> 2;
+    const uint8_t* row = m_data + p.ro;
+    a.gmk = ((const uint4*)row)[g];                               // the four mask words of the group
+    a.goffv = has_goff ? (uint32_t)((const uint16_t*)(row + (N >> 3)))[g] : 0u;
+  };
+  auto issue_codes = [&](const Pos& p, const StMask& a, StCodes& c) {
+    const int t = block_of(p), g = t >> 2, j = t & 3;
+    const uint8_t* row = m_data + p.ro;
+    if (!has_goff && p.it == 0) {
+      // SPARSE4: the byte offset of every group's codes is a prefix sum of the groups' byte counts
+      const uint32_t* bm = (const uint32_t*)row;
+      uint32_t carry = 0;
+      for (int g0 = 0; g0 < m.G; g0 += 64) {
+        const int gg = g0 + lane;
+        uint32_t nb = 0;                                          // bytes of group gg: an even number of nibbles
+        if (gg < m.G) {
+          const uint4 v = ((const uint4*)bm)[gg];
+          nb = (uint32_t)(__popc(v.x) + __popc(v.y) + __popc(v.z) + __popc(v.w) + 1) >> 1;
+        }
+        uint32_t incl = nb;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+          const uint32_t v = (uint32_t)__shfl_up((int)incl, o, 64);
+          incl += lane >= o ? v : 0u;
+        }
+        if (gg < m.G) lgoff[gg] = carry + incl - nb;
+        carry += (uint32_t)__shfl((int)incl, 63, 64);
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+    c.mw = j == 0 ? a.gmk.x : j == 1 ? a.gmk.y : j == 2 ? a.gmk.z : a.gmk.w;
+    const uint32_t pre = (j > 0 ? __popc(a.gmk.x) : 0) + (j > 1 ? __popc(a.gmk.y) : 0) + (j > 2 ? __popc(a.gmk.z) : 0);
+    const uint8_t* cp = row + hdr + (has_goff ? a.goffv : lgoff[g]) + (pre >> 1);
+    const uintptr_t ca = (uintptr_t)cp & ~(uintptr_t)3;
+    c.sh = (uint32_t)(((uintptr_t)cp & 3) * 8 + (pre & 1) * 4);   // < 32
+#pragma unroll
+    for (int i = 0; i < 6; ++i) c.e[i] = ((const uint32_t*)ca)[i];               // 17 bytes + skew; rows end in a readable tail
+    c.sraw = m.scale[(size_t)p.k * m.G + g];
+    c.z = m.zero[(size_t)p.k * m.G + g];
+  };
+
+  float ysum[M];
+#pragma unroll
+  for (int i = 0; i < M; ++i) ysum[i] = 0.f;
+  auto compute = [&](const Pos& p, const StCodes& c) {
+    const int traw = lane + 64 * p.it;
+    const bool valid = traw < NB;
+    const int t = valid ? traw : NB - 1, g = t >> 2;
+    uint32_t w[5];
+#pragma unroll
+    for (int i = 0; i < 5; ++i) w[i] = __builtin_amdgcn_alignbit(c.e[i + 1], c.e[i], c.sh);
+    const uint32_t mw = c.mw;
+    const uint32_t nz = 0x80808080u - c.z * 0x01010101u;
+    int acc[M][NDIG];
+#pragma unroll
+    for (int i = 0; i < M; ++i)
+#pragma unroll
+      for (int d = 0; d < NDIG; ++d) acc[i][d] = 0;
+    // The lanes take the four mask bytes of their blocks in different orders (byte jb ^ rot in
+    // turn jb): a lane's digits are 32 bytes from its neighbour's, and with every lane on the same
+    // byte of its block the 8-byte reads of 32 lanes would fall on eight of the 64 LDS banks.
+    const uint32_t rot = ((uint32_t)lane >> 3) & 3u;
+#pragma unroll
+    for (int jb = 0; jb < 4; ++jb) {
+      const uint32_t jl = (uint32_t)jb ^ rot;
+      const uint32_t mb = (mw >> (8u * jl)) & 0xFFu;
+      const uint32_t r = (uint32_t)__popc(mw & ~(0xFFFFFFFFu << (8u * jl)));                 // survivors before this byte
+      // 32 bits of the stream from nibble r on: dword r / 8 and the next one, picked by selects
+      const uint32_t idx = r >> 3, bs = (r & 7u) * 4u;
+      uint32_t lo = w[0], hi = w[1];
+#pragma unroll
+      for (int i = 1; i < 4; ++i) { lo = idx == (uint32_t)i ? w[i] : lo; hi = idx == (uint32_t)i ? w[i + 1] : hi; }
+      lo = idx >= 4u ? w[4] : lo; hi = idx >= 4u ? 0u : hi;
+      const uint32_t win = __builtin_amdgcn_alignbit(hi, lo, bs);
+      const uint32_t p0 = bias_pool(win & 0x0F0F0F0Fu, nz), p1 = bias_pool((win >> 4) & 0x0F0F0F0Fu, nz);
+      const uint2 sel = lut[mb * ST_LUT_LANES + l4];
+      const int b0 = (int)perm(p1, p0, sel.x), b1 = (int)perm(p1, p0, sel.y);   // q - zero of columns 0-3, 4-7; pruned: 0
+      const int c0 = t * 32 + 8 * (int)jl;
+#pragma unroll
+      for (int i = 0; i < M; ++i)
+#pragma unroll
+        for (int d = 0; d < NDIG; ++d) {
+          const uint2 a = *(const uint2*)(xq + (size_t)(i * NDIG + d) * N + c0);
+          acc[i][d] = __builtin_amdgcn_sdot4(b0, (int)a.x, acc[i][d], false);
+          acc[i][d] = __builtin_amdgcn_sdot4(b1, (int)a.y, acc[i][d], false);
+        }
+    }
+    const float s = valid ? h2f((uint16_t)c.sraw) : 0.f;
+#pragma unroll
+    for (int i = 0; i < M; ++i) {
+      const float f = fmaf((float)(acc[i][0] * 256 + acc[i][1]), 256.f, (float)acc[i][2]);
+      ysum[i] = fmaf(f, s * delta[i * (NCH + 4) + g], ysum[i]);
+    }
+    if (p.it + 1 == nt) {                                         // the row is complete
+      const int k = p.k;
+#pragma unroll
+      for (int i = 0; i < M; ++i) {
+        float v = ysum[i];
+        ysum[i] = 0.f;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+        if (lane == 0) {
+          if (bias) v += (ydt == CBK_F32) ? ((const float*)bias)[k]
+                       : (ydt == CBK_F16) ? h2f(((const uint16_t*)bias)[k]) : bf2f(((const uint16_t*)bias)[k]);
+          if (ydt == CBK_F32) ((float*)y)[(size_t)i * ldy + k] = v;
+          else if (ydt == CBK_F16) ((uint16_t*)y)[(size_t)i * ldy + k] = f2h(v);
+          else ((uint16_t*)y)[(size_t)i * ldy + k] = f2bf(v);
+        }
+      }
+    }
+  };
+
+  Pos pc{k0, 0, m_row_off[k0]};                                   // item being multiplied
+  Pos pb = pc;                                                    // item whose codes are being fetched
+  StMask am;
+  StCodes ca, cb;                                                 // swap roles by name (a copy would wait for the loads)
+  issue_mask(pc, am);
+  issue_codes(pc, am, ca);
+  next_pos(pb);
+  Pos pa = pb;                                                    // item whose mask words are being fetched
+  issue_mask(pb, am);
+  for (int q = 0; q < nitems; q += 2) {
+    issue_codes(pb, am, cb);
+    next_pos(pa);
+    issue_mask(pa, am);
+    compute(pc, ca);
+    pc = pb; pb = pa;
+    if (q + 1 >= nitems) break;
+    issue_codes(pb, am, ca);
+    next_pos(pa);
+    issue_mask(pa, am);
+    compute(pc, cb);
+    pc = pb; pb = pa;
+  }
+}
+
+template <int M>
+static int launch_stream_m(const DMat& m, const void* x, int64_t ldx, int xdt, void* y, int ydt, int64_t ldy,
+                           const void* bias, hipStream_t st) {
+  auto kern = gemv_stream_kernel<M>;
+  static std::atomic<int> configured{0};
+  if (!configured.load(std::memory_order_acquire)) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
+      return CBK_ERR_HIP;
+    configured.store(1, std::memory_order_release);
+  }
+  const size_t lds = (size_t)ST_LUT_BYTES + (size_t)M * NDIG * m.N + (size_t)M * (m.N / 128 + 4) * 4 +
+                     (m.layout == CBK_SPARSE4 ? (size_t)ST_WAVES * m.G * 4 : 0);
+  if (lds > 160 * 1024) return CBK_ERR_UNSUPPORTED;
+  int blocks = (m.K + ST_WAVES - 1) / ST_WAVES;
+  blocks = blocks < 256 ? blocks : 256;                           // one persistent workgroup per CU
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(ST_THREADS), lds, st, m, (const uint16_t*)x, ldx, xdt, y, ydt, ldy, bias);
+  return hipGetLastError() == hipSuccess ? CBK_OK : CBK_ERR_HIP;
+}
+
+// CBK_ERR_UNSUPPORTED: not a case of this kernel (the caller falls back on the float row kernel).
+int launch_gemv_stream(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
+                       const void* bias, hipStream_t st) {
+  if (family_of(m.layout) != FAM_SPARSE || m.bits != 4 || m.group != 128 || m.cs_rows > 1) return CBK_ERR_UNSUPPORTED;
+  if (!(m.flags & CBK_FLAG_ZERO_LE_128)) return CBK_ERR_UNSUPPORTED;
+  if (xdt != CBK_F16 && xdt != CBK_BF16T) return CBK_ERR_DTYPE;
+  if ((size_t)NDIG * m.N > (size_t)ST_X_BUDGET) return CBK_ERR_UNSUPPORTED;
+  int mc = (int)((size_t)ST_X_BUDGET / ((size_t)NDIG * m.N));      // activation rows per pass
+  mc = mc > 4 ? 4 : mc;
+  for (int m0 = 0; m0 < M; m0 += mc) {
+    const int mp = M - m0 < mc ? M - m0 : mc;
+    const void* xs = (const uint8_t*)x + (size_t)m0 * ldx * 2;
+    void* ys = (uint8_t*)y + (size_t)m0 * ldy * (ydt == CBK_F32 ? 4 : 2);
+    int rc;
+    switch (mp) {
+      case 1: rc = launch_stream_m<1>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
+      case 2: rc = launch_stream_m<2>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
+      case 3: rc = launch_stream_m<3>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
+      default: rc = launch_stream_m<4>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
+    }
+    if (rc) return rc;
+  }
+  return CBK_OK;
+}
+
 // ------------------------------------------------------------------ host side
 static inline size_t up256(size_t v) { return (v + 255) & ~(size_t)255; }
 
