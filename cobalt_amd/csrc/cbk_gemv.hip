@@ -794,7 +794,7 @@ constexpr int ST_X_BUDGET = 96 * 1024;        // digits of all activation rows o
 // words and code offset, then (at an address made from those) the block's codes and the group's
 // scale and zero point.
 struct StMask { uint4 gmk; uint32_t goffv; };
-struct StCodes { uint32_t e[6]; uint32_t mw, sh, sraw, z; };
+struct StCodes { uint32_t e[5]; uint32_t mw, sh, sraw, z; };
 
 template <int M>
 __global__ __launch_bounds__(ST_THREADS) void gemv_stream_kernel(DMat m, const uint16_t* x, int64_t ldx, int xdt,
@@ -807,26 +807,15 @@ __global__ __launch_bounds__(ST_THREADS) void gemv_stream_kernel(DMat m, const u
   uint32_t* goffs = (uint32_t*)(delta + M * (NCH + 4));          // [ST_WAVES][G], SPARSE4 only
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  if (tid < 256) {
-    const uint2 e = make_selectors((uint32_t)tid, 0);
-#pragma unroll
-    for (int j = 0; j < ST_LUT_LANES; ++j) lut[tid * ST_LUT_LANES + j] = e;
-  }
-  const int n16 = N >> 4, xitems = M * n16;                      // a multiple of 8
-  for (int it = tid; it < xitems; it += ST_THREADS) {
-    XLoad xl;
-    stage_load(x, ldx, m.cs, N, 0, n16, it, M == 1, 0, xl);
-    stage_convert<0>(xl, m.cs != nullptr, xdt, N, 0, n16, it, M == 1, xq, delta);
-  }
-  __syncthreads();
   const bool has_goff = m.layout != CBK_SPARSE4;
   const int hdr = ((N >> 3) + (has_goff ? ((m.G * 2 + 15) & ~15) : 0) + 15) & ~15;
   uint32_t* lgoff = goffs + wave * m.G;
   const uint32_t l4 = lane & (ST_LUT_LANES - 1);
   // this wavefront's rows k0, k0 + ks, ...; its items are (row, pass over the row's blocks), in order
-  const int k0 = (int)blockIdx.x * ST_WAVES + wave, ks = (int)gridDim.x * ST_WAVES;
-  if (k0 >= m.K) return;                                          // (after the only barrier)
-  const int nrows = (m.K - k0 + ks - 1) / ks;
+  // (a wavefront without rows goes through the first loads on the last row and leaves after the barrier)
+  const int kw = (int)blockIdx.x * ST_WAVES + wave, ks = (int)gridDim.x * ST_WAVES;
+  const int k0 = kw < m.K ? kw : m.K - 1;
+  const int nrows = kw < m.K ? (m.K - k0 + ks - 1) / ks : 0;
   const int nt = (NB + 63) >> 6, nitems = nrows * nt;
   const uint8_t* const m_data = m.data;
   const uint32_t* const m_row_off = m.row_off;
@@ -876,7 +865,7 @@ __global__ __launch_bounds__(ST_THREADS) void gemv_stream_kernel(DMat m, const u
     const uintptr_t ca = (uintptr_t)cp & ~(uintptr_t)3;
     c.sh = (uint32_t)(((uintptr_t)cp & 3) * 8 + (pre & 1) * 4);   // < 32
 #pragma unroll
-    for (int i = 0; i < 6; ++i) c.e[i] = ((const uint32_t*)ca)[i];               // 17 bytes + skew; rows end in a readable tail
+    for (int i = 0; i < 5; ++i) c.e[i] = ((const uint32_t*)ca)[i];               // 16 bytes + skew; rows end in a readable tail
     c.sraw = m.scale[(size_t)p.k * m.G + g];
     c.z = m.zero[(size_t)p.k * m.G + g];
   };
@@ -888,9 +877,9 @@ __global__ __launch_bounds__(ST_THREADS) void gemv_stream_kernel(DMat m, const u
     const int traw = lane + 64 * p.it;
     const bool valid = traw < NB;
     const int t = valid ? traw : NB - 1, g = t >> 2;
-    uint32_t w[5];
+    uint32_t w[4];                                                // the block's codes (at most 32 nibbles) from bit 0 on
 #pragma unroll
-    for (int i = 0; i < 5; ++i) w[i] = __builtin_amdgcn_alignbit(c.e[i + 1], c.e[i], c.sh);
+    for (int i = 0; i < 4; ++i) w[i] = __builtin_amdgcn_alignbit(c.e[i + 1], c.e[i], c.sh);
     const uint32_t mw = c.mw;
     const uint32_t nz = 0x80808080u - c.z * 0x01010101u;
     int acc[M][NDIG];
@@ -907,13 +896,12 @@ __global__ __launch_bounds__(ST_THREADS) void gemv_stream_kernel(DMat m, const u
       const uint32_t jl = (uint32_t)jb ^ rot;
       const uint32_t mb = (mw >> (8u * jl)) & 0xFFu;
       const uint32_t r = (uint32_t)__popc(mw & ~(0xFFFFFFFFu << (8u * jl)));                 // survivors before this byte
-      // 32 bits of the stream from nibble r on: dword r / 8 and the next one, picked by selects
-      const uint32_t idx = r >> 3, bs = (r & 7u) * 4u;
-      uint32_t lo = w[0], hi = w[1];
-#pragma unroll
-      for (int i = 1; i < 4; ++i) { lo = idx == (uint32_t)i ? w[i] : lo; hi = idx == (uint32_t)i ? w[i + 1] : hi; }
-      lo = idx >= 4u ? w[4] : lo; hi = idx >= 4u ? 0u : hi;
-      const uint32_t win = __builtin_amdgcn_alignbit(hi, lo, bs);
+      // 32 bits of the stream from nibble r on (r <= 24, and a shift of 0 at r = 24): dwords r / 8 and
+      // r / 8 + 1, picked with two levels of bitwise selects under the sign-extended bits 4 and 3 of r
+      const uint32_t m64 = (uint32_t)__builtin_amdgcn_sbfe((int)r, 4, 1), m32 = (uint32_t)__builtin_amdgcn_sbfe((int)r, 3, 1);
+      const uint32_t x0 = mask_select(m64, w[0], w[2]), x1 = mask_select(m64, w[1], w[3]), x2 = w[2] & ~m64;
+      const uint32_t lo = mask_select(m32, x0, x1), hi = mask_select(m32, x1, x2);
+      const uint32_t win = __builtin_amdgcn_alignbit(hi, lo, (r & 7u) * 4u);
       const uint32_t p0 = bias_pool(win & 0x0F0F0F0Fu, nz), p1 = bias_pool((win >> 4) & 0x0F0F0F0Fu, nz);
       const uint2 sel = lut[mb * ST_LUT_LANES + l4];
       const int b0 = (int)perm(p1, p0, sel.x), b1 = (int)perm(p1, p0, sel.y);   // q - zero of columns 0-3, 4-7; pruned: 0
@@ -961,6 +949,21 @@ __global__ __launch_bounds__(ST_THREADS) void gemv_stream_kernel(DMat m, const u
   next_pos(pb);
   Pos pa = pb;                                                    // item whose mask words are being fetched
   issue_mask(pb, am);
+  // Selector table and activation digits, while the first rows' bytes are on their way (three
+  // dependent loads: row offset, mask words, codes).
+  if (tid < 256) {
+    const uint2 e = make_selectors((uint32_t)tid, 0);
+#pragma unroll
+    for (int j = 0; j < ST_LUT_LANES; ++j) lut[tid * ST_LUT_LANES + j] = e;
+  }
+  const int n16 = N >> 4, xitems = M * n16;                      // a multiple of 8
+  for (int it = tid; it < xitems; it += ST_THREADS) {
+    XLoad xl;
+    stage_load(x, ldx, m.cs, N, 0, n16, it, M == 1, 0, xl);
+    stage_convert<0>(xl, m.cs != nullptr, xdt, N, 0, n16, it, M == 1, xq, delta);
+  }
+  __syncthreads();
+  if (kw >= m.K) return;
   for (int q = 0; q < nitems; q += 2) {
     issue_codes(pb, am, cb);
     next_pos(pa);

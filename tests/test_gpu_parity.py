@@ -115,6 +115,32 @@ def test_gemv_sparse_streams_on_long_rows(case):
         assert rel_fro(_np(y), R.forward_ref(W, _np(x))) < 1e-5, (case_id(case), M)
 
 
+@pytest.mark.parametrize("case", SPARSE_CASES, ids=case_id)
+def test_gemv_sparse_streams_integer_dot_kernel(case):
+    """The decode kernel of the survivor streams (activation digits in LDS, byte-permute expansion,
+    integer dot products): rows shorter than the 64 blocks of a wavefront, more rows than one pass of
+    the resident wavefronts, the longest row whose digits fit (one activation row per pass) and one
+    beyond it (float row kernel); one to nine activation rows, both activation types, a bias;
+    a row's result does not depend on how many rows the call has."""
+    for (K, N) in ((5, 128), (37, 384), (300, 4096), (4200, 256), (16, 21504), (9, 32768), (6, 32896)):
+        raw = make_raw(case, K, N, seed=K + N + case[0])
+        pk = oracle_pack(case, raw)
+        pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV)
+        W = R.dequant(pk, K, N, case[0], col_scale=raw["col_scale"], **kw_of(case))
+        bias = acts(1, K, torch.float32, seed=K)[0]
+        for M, dtype in ((1, torch.float16), (2, torch.bfloat16), (3, torch.float16), (4, torch.bfloat16), (5, torch.float16),
+                         (9, torch.float16)):
+            x = acts(M, N, dtype, seed=M + N)
+            ref = R.forward_ref(W, _np(x))
+            y = ops.gemv(pm, x.to(DEV), out_dtype=torch.float32)
+            assert rel_fro(_np(y), ref) < 1e-5, (case_id(case), K, N, M)
+            yb = ops.gemv(pm, x.to(DEV), bias=bias.to(DEV), out_dtype=torch.float32)
+            assert rel_fro(_np(yb), ref + _np(bias)[None, :]) < 1e-5, (case_id(case), K, N, M)
+            if N <= 32768:
+                y1 = ops.gemv(pm, x[M - 1:M].to(DEV), out_dtype=torch.float32)
+                assert torch.equal(y1[0], y[M - 1]), (case_id(case), K, N, M)
+
+
 ALL_MFMA_CASES = [(F.BLKC, b, g, k) for b in (2, 3, 4) for g in (64, 128) for k in (10, 16, 23)] + \
                  [(F.DENSEB, b, g, 0) for b in (2, 3, 4) for g in (64, 128)]
 
