@@ -1023,6 +1023,194 @@ int launch_gemv_stream(const DMat& m, const void* x, int xdt, int M, int64_t ldx
   return CBK_OK;
 }
 
+// ------------------------------------------------------------------ 8-bit dense rows
+// DENSE8 (group 128) at one to four activation rows per pass, on the same activation digits:
+// the codes are the bytes themselves, q - 128 is a signed byte (one xor), and
+//   sum_j (q_j - z) X_j = sum_j (q_j - 128) X_j - (z - 128) sum_j X_j
+// with the integer activations X of the group; their sum per 128-column chunk is formed once per
+// launch from the digits.  One wavefront per weight row, one lane per 32-column block (32 code
+// bytes), v_dot4_i32_i8 per four columns and digit, the next block's loads in flight while this
+// one is multiplied.  Any uint8 zero point.
+// Reference semantics: cbk::detail::gemv_dense8 (src/cobaltkernel/csrc/cobalt_gemv.cuh:1127-1171).
+struct D8Loads { uint4 c0, c1; uint32_t sraw, z; };
+
+template <int M>
+__global__ __launch_bounds__(ST_THREADS) void gemv_dense8_kernel(DMat m, const uint16_t* x, int64_t ldx, int xdt,
+                                                                 void* y, int ydt, int64_t ldy, const void* bias) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int N = m.N, NCH = N >> 7, NB = N >> 5;
+  int8_t* xq = (int8_t*)smem;
+  float* delta = (float*)(xq + (size_t)M * NDIG * N);
+  float* fsum = delta + M * (NCH + 4);                            // [M][NCH] sum of the chunk's integer activations
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // this wavefront's rows kw, kw + ks, ...; its items are (row, pass over the row's blocks), in order
+  // (a wavefront without rows goes through the first loads on the last row and leaves after the barriers)
+  const int kw = (int)blockIdx.x * ST_WAVES + wave, ks = (int)gridDim.x * ST_WAVES;
+  const int k0 = kw < m.K ? kw : m.K - 1;
+  const int nrows = kw < m.K ? (m.K - k0 + ks - 1) / ks : 0;
+  const int nt = (NB + 63) >> 6, nitems = nrows * nt;
+  struct Pos { int k, it; };
+  auto next_pos = [&](Pos& p) {
+    if (p.it + 1 < nt) { ++p.it; return; }
+    if (p.k + ks < m.K) { p.k += ks; p.it = 0; }
+  };
+  auto issue = [&](const Pos& p, D8Loads& L) {
+    int t = lane + 64 * p.it;
+    t = t < NB ? t : NB - 1;
+    const RowView row = row_view(m, p.k);
+    L.c0 = *(const uint4*)row.unit(2 * t);
+    L.c1 = *(const uint4*)row.unit(2 * t + 1);
+    const size_t gi = meta_index(m, p.k, t >> 2);
+    L.sraw = m.scale[gi];
+    L.z = m.zero[gi];
+  };
+  float ysum[M];
+#pragma unroll
+  for (int i = 0; i < M; ++i) ysum[i] = 0.f;
+  auto compute = [&](const Pos& p, const D8Loads& L) {
+    const int traw = lane + 64 * p.it;
+    const bool valid = traw < NB;
+    const int t = valid ? traw : NB - 1, g = t >> 2;
+    const uint32_t cw[8] = {L.c0.x, L.c0.y, L.c0.z, L.c0.w, L.c1.x, L.c1.y, L.c1.z, L.c1.w};
+    int acc[M][NDIG];
+#pragma unroll
+    for (int i = 0; i < M; ++i)
+#pragma unroll
+      for (int d = 0; d < NDIG; ++d) acc[i][d] = 0;
+    // the lanes take the two 16-byte halves of their blocks in alternating order: the digits of
+    // neighbouring lanes are 32 bytes apart, and sixteen 16-byte reads at that stride would fall
+    // on half of the LDS banks
+    const int rot = (lane >> 3) & 1;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int hh = h ^ rot;
+      uint32_t b[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) b[u] = (hh ? cw[4 + u] : cw[u]) ^ 0x80808080u;      // q - 128 as signed bytes
+#pragma unroll
+      for (int i = 0; i < M; ++i)
+#pragma unroll
+        for (int d = 0; d < NDIG; ++d) {
+          const uint4 a = *(const uint4*)(xq + (size_t)(i * NDIG + d) * N + t * 32 + 16 * hh);
+          acc[i][d] = __builtin_amdgcn_sdot4((int)b[0], (int)a.x, acc[i][d], false);
+          acc[i][d] = __builtin_amdgcn_sdot4((int)b[1], (int)a.y, acc[i][d], false);
+          acc[i][d] = __builtin_amdgcn_sdot4((int)b[2], (int)a.z, acc[i][d], false);
+          acc[i][d] = __builtin_amdgcn_sdot4((int)b[3], (int)a.w, acc[i][d], false);
+        }
+    }
+    const float s = valid ? h2f((uint16_t)L.sraw) : 0.f;
+    const float zc = (t & 3) == 0 ? (float)((int)L.z - 128) : 0.f;   // the group's zero-point term: once, in its first block
+#pragma unroll
+    for (int i = 0; i < M; ++i) {
+      const float f = fmaf((float)(acc[i][0] * 256 + acc[i][1]), 256.f, (float)acc[i][2]);
+      ysum[i] = fmaf(fmaf(-zc, fsum[i * NCH + g], f), s * delta[i * (NCH + 4) + g], ysum[i]);
+    }
+    if (p.it + 1 == nt) {                                         // the row is complete
+      const int k = p.k;
+#pragma unroll
+      for (int i = 0; i < M; ++i) {
+        float v = ysum[i];
+        ysum[i] = 0.f;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+        if (lane == 0) {
+          if (bias) v += (ydt == CBK_F32) ? ((const float*)bias)[k]
+                       : (ydt == CBK_F16) ? h2f(((const uint16_t*)bias)[k]) : bf2f(((const uint16_t*)bias)[k]);
+          if (ydt == CBK_F32) ((float*)y)[(size_t)i * ldy + k] = v;
+          else if (ydt == CBK_F16) ((uint16_t*)y)[(size_t)i * ldy + k] = f2h(v);
+          else ((uint16_t*)y)[(size_t)i * ldy + k] = f2bf(v);
+        }
+      }
+    }
+  };
+
+  Pos pc{k0, 0};                                                  // item being multiplied
+  D8Loads la, lb;                                                 // swap roles by name (a copy would wait for the loads)
+  issue(pc, la);
+  Pos pn = pc;                                                    // item whose bytes are being fetched
+  next_pos(pn);
+  // activation digits and the chunks' sums, while the first row's bytes are on their way
+  const int n16 = N >> 4, xitems = M * n16;                      // a multiple of 8
+  for (int it = tid; it < xitems; it += ST_THREADS) {
+    XLoad xl;
+    stage_load(x, ldx, m.cs, N, 0, n16, it, M == 1, 0, xl);
+    stage_convert<0>(xl, m.cs != nullptr, xdt, N, 0, n16, it, M == 1, xq, delta);
+  }
+  __syncthreads();
+  for (int c = tid; c < M * NCH; c += ST_THREADS) {
+    const int row = c / NCH, ch = c - row * NCH;
+    int sd[NDIG];
+#pragma unroll
+    for (int d = 0; d < NDIG; ++d) {
+      int sum = 0;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const uint4 a = *(const uint4*)(xq + (size_t)(row * NDIG + d) * N + ch * 128 + 16 * u);
+        sum = __builtin_amdgcn_sdot4(0x01010101, (int)a.x, sum, false);
+        sum = __builtin_amdgcn_sdot4(0x01010101, (int)a.y, sum, false);
+        sum = __builtin_amdgcn_sdot4(0x01010101, (int)a.z, sum, false);
+        sum = __builtin_amdgcn_sdot4(0x01010101, (int)a.w, sum, false);
+      }
+      sd[d] = sum;
+    }
+    fsum[c] = (float)((sd[0] * 256 + sd[1]) * 256 + sd[2]);       // |sum| < 2^31: 128 columns of at most 127 * 65536
+  }
+  __syncthreads();
+  if (kw >= m.K) return;
+  for (int q = 0; q < nitems; q += 2) {
+    issue(pn, lb);
+    compute(pc, la);
+    pc = pn; next_pos(pn);
+    if (q + 1 >= nitems) break;
+    issue(pn, la);
+    compute(pc, lb);
+    pc = pn; next_pos(pn);
+  }
+}
+
+template <int M>
+static int launch_dense8_m(const DMat& m, const void* x, int64_t ldx, int xdt, void* y, int ydt, int64_t ldy,
+                           const void* bias, hipStream_t st) {
+  auto kern = gemv_dense8_kernel<M>;
+  static std::atomic<int> configured{0};
+  if (!configured.load(std::memory_order_acquire)) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
+      return CBK_ERR_HIP;
+    configured.store(1, std::memory_order_release);
+  }
+  const size_t lds = (size_t)M * NDIG * m.N + (size_t)M * (m.N / 128 + 4) * 4 + (size_t)M * (m.N / 128) * 4;
+  if (lds > 160 * 1024) return CBK_ERR_UNSUPPORTED;
+  int blocks = (m.K + ST_WAVES - 1) / ST_WAVES;
+  blocks = blocks < 256 ? blocks : 256;                           // one persistent workgroup per CU
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(ST_THREADS), lds, st, m, (const uint16_t*)x, ldx, xdt, y, ydt, ldy, bias);
+  return hipGetLastError() == hipSuccess ? CBK_OK : CBK_ERR_HIP;
+}
+
+// CBK_ERR_UNSUPPORTED: not a case of this kernel (the caller falls back on the float row kernel).
+int launch_gemv_dense8(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
+                       const void* bias, hipStream_t st) {
+  if (m.layout != CBK_DENSE8 || m.bits != 8 || m.group != 128 || m.cs_rows > 1) return CBK_ERR_UNSUPPORTED;
+  if (xdt != CBK_F16 && xdt != CBK_BF16T) return CBK_ERR_DTYPE;
+  if ((size_t)NDIG * m.N > (size_t)ST_X_BUDGET) return CBK_ERR_UNSUPPORTED;
+  int mc = (int)((size_t)ST_X_BUDGET / ((size_t)NDIG * m.N));      // activation rows per pass
+  mc = mc > 4 ? 4 : mc;
+  for (int m0 = 0; m0 < M; m0 += mc) {
+    const int mp = M - m0 < mc ? M - m0 : mc;
+    const void* xs = (const uint8_t*)x + (size_t)m0 * ldx * 2;
+    void* ys = (uint8_t*)y + (size_t)m0 * ldy * (ydt == CBK_F32 ? 4 : 2);
+    int rc;
+    switch (mp) {
+      case 1: rc = launch_dense8_m<1>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
+      case 2: rc = launch_dense8_m<2>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
+      case 3: rc = launch_dense8_m<3>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
+      default: rc = launch_dense8_m<4>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
+    }
+    if (rc) return rc;
+  }
+  return CBK_OK;
+}
+
 // ------------------------------------------------------------------ host side
 static inline size_t up256(size_t v) { return (v + 255) & ~(size_t)255; }
 

@@ -84,8 +84,8 @@ enum cbk_status {
  *             matrix-core decode kernel needs q - zero to fit a signed byte; without the flag
  *             cbk_gemv runs the slower float row kernel, which takes any uint8 zero point.
  *             (The matrix-core kernels take layouts 1, 6, 7, 8, 9 with 2/3/4-bit codes, or 6-bit
- *             for layout 7; SPARSE4/4X/4E decode with an integer-dot row kernel of their own,
- *             8-bit codes go through the float row kernel and the generic tile reader.)
+ *             for layout 7; SPARSE4/4X/4E and DENSE8 decode with integer-dot row kernels of their
+ *             own, 8-bit prefill goes through the generic tile reader.)
  *             CBK_FLAG_TILED16: data / scale / zero are in 16-row tile-interleaved order, a
  *             permutation of the same bytes made once at load time so that the sixteen rows a
  *             wavefront decodes together are contiguous in HBM: with s = cbk_row_stride(),

@@ -115,10 +115,11 @@ def test_gemv_sparse_streams_on_long_rows(case):
         assert rel_fro(_np(y), R.forward_ref(W, _np(x))) < 1e-5, (case_id(case), M)
 
 
-@pytest.mark.parametrize("case", SPARSE_CASES, ids=case_id)
-def test_gemv_sparse_streams_integer_dot_kernel(case):
-    """The decode kernel of the survivor streams (activation digits in LDS, byte-permute expansion,
-    integer dot products): rows shorter than the 64 blocks of a wavefront, more rows than one pass of
+@pytest.mark.parametrize("case", SPARSE_CASES + [(F.DENSE8, 8, 128, 0)], ids=case_id)
+def test_gemv_integer_dot_row_kernels(case):
+    """The decode kernels of the survivor streams and of DENSE8 (activation digits in LDS, integer
+    dot products; the streams with the byte-permute expansion, the 8-bit codes as q - 128 and the
+    zero point, any uint8 value, through the groups' digit sums): rows shorter than the 64 blocks of a wavefront, more rows than one pass of
     the resident wavefronts, the longest row whose digits fit (one activation row per pass) and one
     beyond it (float row kernel); one to nine activation rows, both activation types, a bias;
     a row's result does not depend on how many rows the call has."""
