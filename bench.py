@@ -213,10 +213,11 @@ def decode_layer_sets(torch, F, L, dev, shapes, sets, M, dt, launch, steps, warm
     return res, xs, y_first
 
 
-def per_matrix(torch, F, L, dev, shapes, layout, bits, group, keep, M, dt, iters=24):
+def per_matrix(torch, F, L, dev, shapes, layout, bits, group, keep, M, dt, iters=24, tiled=True):
     """Each distinct matrix of the layer set on its own: one launch per matrix, distinct copies of
     at least 512 MB in rotation (the protocol of src/cobaltkernel/test_gemv.py:201-202, :521-522),
-    one HIP graph per rotation."""
+    one HIP graph per rotation.  tiled=False keeps the row-major order (the survivor-stream
+    layouts have no other)."""
     rows, seen = [], set()
     stream = torch.cuda.Stream(dev)
     xdt = F.dtype_code(dt)
@@ -225,9 +226,10 @@ def per_matrix(torch, F, L, dev, shapes, layout, bits, group, keep, M, dt, iters
         if (K, N) in seen:
             continue
         seen.add((K, N))
-        one = K * F.row_stride(layout, N, bits, group, keep) + K * (N // group) * 3
-        copies = max(2, -(-2 * INFINITY_CACHE // one))
-        pms = [F.synth_packed(K, N, layout, bits, group, keep, seed=7000 + c, device=dev).to_tiled() for c in range(copies)]
+        order = (lambda p: p.to_tiled()) if tiled else (lambda p: p)
+        pm0 = order(F.synth_packed(K, N, layout, bits, group, keep, seed=7000, device=dev))
+        copies = max(2, -(-2 * INFINITY_CACHE // pm0.stream_bytes()))
+        pms = [pm0] + [order(F.synth_packed(K, N, layout, bits, group, keep, seed=7000 + c, device=dev)) for c in range(1, copies)]
         x = torch.randn(M, N, device=dev, generator=torch.Generator(device=dev).manual_seed(N)).to(dt)
         y = torch.empty(M, K, dtype=dt, device=dev)
         args = []
@@ -649,6 +651,11 @@ def main():
     }
     if not a.no_secondary:
         out["per_matrix"] = per_matrix(torch, F, L, dev, shapes, layout, a.bits, a.group, a.keep, M, dt)
+        # the layouts that decode on the row kernels (integer dot products), on the workload's gate matrix
+        gate = [sh for sh in shapes if sh[0] == "gate"]
+        out["row_kernel_layouts"] = [
+            dict(layout=F.LAYOUT_NAME[lay], **per_matrix(torch, F, L, dev, gate, lay, b, 128, None, M, dt, tiled=False)[0])
+            for lay, b in ((F.SPARSE4X, 4), (F.DENSE8, 8))]
         other = "mistral7b" if a.workload == "gemma27b" else "gemma27b"
         oshapes, odt = SHAPES[other], torch_dtype(torch, WORKLOAD_DTYPE[other])
         osets, _ = make_sets(torch, F, dev, oshapes, layout, a.bits, a.group, a.keep, 2 * INFINITY_CACHE)

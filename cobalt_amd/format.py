@@ -520,6 +520,40 @@ def fuse_rows(parts, interleave: bool = False) -> PackedMatrix:
     return out
 
 
+def _synth_sparse(K, N, layout, bits, group, g, dev, cs_rows) -> PackedMatrix:
+    """synth_packed for the survivor-stream layouts: every column kept with probability 1/2, rows
+    laid out as src/cobaltkernel/pack_cobalt.py:201-250 does ([bitmap N/8][group byte offsets u16,
+    SPARSE4X / SPARSE4E][pad to 16][codes, every group padded to whole bytes], rows padded to 16)."""
+    G = N // group
+    has_goff = layout != SPARSE4
+    hdr = _align(N // 8 + (_align(G * 2, 16) if has_goff else 0), 16)
+    mask = torch.randint(0, 256, (K, N // 8), generator=g, device=dev, dtype=torch.int32).to(torch.uint8)
+    cnt = unpack_mask(mask, N).reshape(K, G, group).sum(-1).to(torch.int64)
+    gbytes = (cnt + 1) // 2
+    gcum = torch.cumsum(gbytes, 1) - gbytes
+    row_bytes = (hdr + gbytes.sum(1) + 15) // 16 * 16
+    row_off = torch.zeros(K + 1, dtype=torch.int64, device=dev)
+    row_off[1:] = torch.cumsum(row_bytes, 0)
+    total = int(row_off[K])
+    if total >= 1 << 32:
+        raise ValueError("the rows do not fit 32-bit offsets")
+    data = torch.randint(0, 256, (total + BLOB_TAIL,), generator=g, device=dev, dtype=torch.int32).to(torch.uint8)
+    head = torch.zeros(K, hdr, dtype=torch.uint8, device=dev)
+    head[:, : N // 8] = mask
+    if has_goff:
+        head[:, N // 8: N // 8 + 2 * G] = gcum.to(torch.int16).view(torch.uint8).reshape(K, 2 * G)
+    pos = row_off[:K, None] + torch.arange(hdr, device=dev)[None, :]
+    data[pos.reshape(-1)] = head.reshape(-1)
+    scale = (torch.rand(K, G, generator=g, device=dev) * 0.01 + 1e-3).half()
+    zero = torch.randint(0, 1 << bits, (K, G), generator=g, device=dev, dtype=torch.int32).to(torch.uint8)
+    arrays = {"data": data, "scale": scale, "zero": zero, "row_off": row_off.to(torch.int32).view(torch.uint8)}
+    if cs_rows:
+        arrays["col_scale"] = (torch.rand(cs_rows, N, generator=g, device=dev) * 1.5 + 0.5).half()
+    blob, offs = _assemble(arrays, dev)
+    return PackedMatrix(blob, offs, K, N, layout, bits, group, 0, cs_rows, (0, 0), total, int(cnt.sum()), 0,
+                        FLAG_ZERO_LE_128)
+
+
 def synth_packed(K: int, N: int, layout: int, bits=None, group=None, keep=None, seed: int = 0,
                  device="cpu", cs_rows: int = 1) -> PackedMatrix:
     """A VALID packed matrix with random content, made directly in packed form (the idea of
@@ -528,11 +562,11 @@ def synth_packed(K: int, N: int, layout: int, bits=None, group=None, keep=None, 
     For the dense family every column counts as a survivor.  Used for bandwidth runs, where the
     kernel's time depends on the mask statistics and not on the values."""
     bits, group, kpb = canon(layout, bits, group, keep)
-    if layout in _SPARSE:
-        raise NotImplementedError
     dev = torch.device(device)
     g = torch.Generator(device=dev).manual_seed(seed)
     G = N // group
+    if layout in _SPARSE:
+        return _synth_sparse(K, N, layout, bits, group, g, dev, cs_rows)
     stride = row_stride(layout, N, bits, group, kpb)
     data = torch.zeros(K * stride + BLOB_TAIL, dtype=torch.uint8, device=dev)
     rows = data[: K * stride].view(K, stride)

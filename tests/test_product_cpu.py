@@ -49,6 +49,25 @@ def test_synth_packed_is_valid(case):
     assert np.array_equal(pk2["data"], pk["data"])
 
 
+@pytest.mark.parametrize("layout", [F.SPARSE4, F.SPARSE4X, F.SPARSE4E], ids=lambda l: F.LAYOUT_NAME[l])
+def test_synth_packed_survivor_streams_are_valid(layout):
+    """The synthetic rows have the structure the oracle's reader checks (stored group offsets equal
+    the bitmap's prefix sums, rows padded to 16 bytes) and, random padding nibbles aside, are the
+    bytes the oracle's packer makes from the decoded codes."""
+    K, N = 9, 640
+    pm = F.synth_packed(K, N, layout, seed=5)
+    pm.validate(deep=True)
+    ro = pm.array("row_off").numpy().view(np.uint32)
+    pk = dict(data=pm.array("data").numpy(), scale=pm.array("scale").numpy().reshape(K, -1),
+              zero=pm.array("zero").numpy().reshape(K, -1), row_off=ro)
+    q, kp = R.unpack_codes(pk, K, N, layout)
+    assert int(kp.sum()) == pm.n_survivors and q.max() <= 15 and (q[~kp] == 0).all()
+    pk2 = R.pack_matrix(R.pack_bits(kp), q, pk["scale"], pk["zero"], layout, fix_zero=False)
+    assert np.array_equal(pk2["row_off"], ro) and pk2["data"].size == pk["data"].size
+    q2, kp2 = R.unpack_codes(pk2, K, N, layout)
+    assert np.array_equal(q2, q) and np.array_equal(kp2, kp)
+
+
 def test_stream_helpers_roundtrip():
     g = torch.Generator().manual_seed(0)
     for bits in (2, 3, 4, 6, 8):
