@@ -780,9 +780,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 // vector instructions per column (pruned ones included) and is bound by that.  This kernel keeps
 // the arithmetic of the kernel above (activation digits in LDS, byte-permute expansion of the
 // bitmap into signed bytes q - zero, exact int32 sums per digit, one float FMA per 32-column block
-// with scale * delta) and forms the sums with v_dot4_i32_i8: about four instructions per column.
-// One wavefront per weight row, one lane per 32-column block, a workgroup of four wavefronts
-// stages the digits once and then walks rows.
+// with scale * delta) and forms the sums with v_dot4_i32_i8: about seven instructions per column.
+// One wavefront per weight row, one lane per 32-column block; a persistent workgroup of sixteen
+// wavefronts per CU stages the digits once and then walks rows.
 // Reference semantics: cbk::gemv_sparse4 (src/cobaltkernel/csrc/cobalt_gemv.cuh:216-301).
 constexpr int ST_WAVES = 16;
 constexpr int ST_THREADS = ST_WAVES * 64;
