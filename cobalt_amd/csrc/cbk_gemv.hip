@@ -775,7 +775,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 }
 
 // ------------------------------------------------------------------ survivor-stream rows
-// SPARSE4 / SPARSE4X / SPARSE4E at one to four activation rows.  Rows of different lengths do not
+// SPARSE4 / SPARSE4X / SPARSE4E at one to eight activation rows per pass.  Rows of different lengths do not
 // tile, so there is no matrix-core kernel for them; but the float row kernel spends about fourteen
 // vector instructions per column (pruned ones included) and is bound by that.  This kernel keeps
 // the arithmetic of the kernel above (activation digits in LDS, byte-permute expansion of the
@@ -789,6 +789,7 @@ constexpr int ST_THREADS = ST_WAVES * 64;
 constexpr int ST_LUT_LANES = 4;
 constexpr int ST_LUT_BYTES = 256 * ST_LUT_LANES * 8;
 constexpr int ST_X_BUDGET = 96 * 1024;        // digits of all activation rows of a pass
+constexpr int ST_MAX_M = 8;                   // activation rows per pass
 
 // What a lane fetches for one (row, 32-column block) item, in two dependent steps: the group's mask
 // words and code offset, then (at an address made from those) the block's codes and the group's
@@ -1006,7 +1007,7 @@ int launch_gemv_stream(const DMat& m, const void* x, int xdt, int M, int64_t ldx
   if (xdt != CBK_F16 && xdt != CBK_BF16T) return CBK_ERR_DTYPE;
   if ((size_t)NDIG * m.N > (size_t)ST_X_BUDGET) return CBK_ERR_UNSUPPORTED;
   int mc = (int)((size_t)ST_X_BUDGET / ((size_t)NDIG * m.N));      // activation rows per pass
-  mc = mc > 4 ? 4 : mc;
+  mc = mc > ST_MAX_M ? ST_MAX_M : mc;
   for (int m0 = 0; m0 < M; m0 += mc) {
     const int mp = M - m0 < mc ? M - m0 : mc;
     const void* xs = (const uint8_t*)x + (size_t)m0 * ldx * 2;
@@ -1016,7 +1017,11 @@ int launch_gemv_stream(const DMat& m, const void* x, int xdt, int M, int64_t ldx
       case 1: rc = launch_stream_m<1>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
       case 2: rc = launch_stream_m<2>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
       case 3: rc = launch_stream_m<3>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
-      default: rc = launch_stream_m<4>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
+      case 4: rc = launch_stream_m<4>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
+      case 5: rc = launch_stream_m<5>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
+      case 6: rc = launch_stream_m<6>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
+      case 7: rc = launch_stream_m<7>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
+      default: rc = launch_stream_m<8>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
     }
     if (rc) return rc;
   }
@@ -1024,7 +1029,7 @@ int launch_gemv_stream(const DMat& m, const void* x, int xdt, int M, int64_t ldx
 }
 
 // ------------------------------------------------------------------ 8-bit dense rows
-// DENSE8 (group 128) at one to four activation rows per pass, on the same activation digits:
+// DENSE8 (group 128) at one to eight activation rows per pass, on the same activation digits:
 // the codes are the bytes themselves, q - 128 is a signed byte (one xor), and
 //   sum_j (q_j - z) X_j = sum_j (q_j - 128) X_j - (z - 128) sum_j X_j
 // with the integer activations X of the group; their sum per 128-column chunk is formed once per
@@ -1194,7 +1199,7 @@ int launch_gemv_dense8(const DMat& m, const void* x, int xdt, int M, int64_t ldx
   if (xdt != CBK_F16 && xdt != CBK_BF16T) return CBK_ERR_DTYPE;
   if ((size_t)NDIG * m.N > (size_t)ST_X_BUDGET) return CBK_ERR_UNSUPPORTED;
   int mc = (int)((size_t)ST_X_BUDGET / ((size_t)NDIG * m.N));      // activation rows per pass
-  mc = mc > 4 ? 4 : mc;
+  mc = mc > ST_MAX_M ? ST_MAX_M : mc;
   for (int m0 = 0; m0 < M; m0 += mc) {
     const int mp = M - m0 < mc ? M - m0 : mc;
     const void* xs = (const uint8_t*)x + (size_t)m0 * ldx * 2;
@@ -1204,7 +1209,11 @@ int launch_gemv_dense8(const DMat& m, const void* x, int xdt, int M, int64_t ldx
       case 1: rc = launch_dense8_m<1>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
       case 2: rc = launch_dense8_m<2>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
       case 3: rc = launch_dense8_m<3>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
-      default: rc = launch_dense8_m<4>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
+      case 4: rc = launch_dense8_m<4>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
+      case 5: rc = launch_dense8_m<5>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
+      case 6: rc = launch_dense8_m<6>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
+      case 7: rc = launch_dense8_m<7>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
+      default: rc = launch_dense8_m<8>(m, xs, ldx, xdt, ys, ydt, ldy, bias, st); break;
     }
     if (rc) return rc;
   }
