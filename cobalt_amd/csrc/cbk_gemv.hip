@@ -223,6 +223,17 @@ __device__ inline float quarter_sum(float y) {
   return c + d;
 }
 
+// Sum over the wavefront, in every lane, without a trip through LDS: quads, half rows and rows by
+// DPP lane moves (each step adds the mirror image that holds the other half's sum), then the four
+// rows with the swap instructions.
+__device__ inline float wave_sum_dpp(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));    // quad_perm [1,0,3,2]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));    // quad_perm [2,3,0,1]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));   // row_half_mirror
+  v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));   // row_mirror
+  return quarter_sum(v);
+}
+
 // ------------------------------------------------------------------ one 32-column block
 // mask bytes of a block and the number of survivors before each of them
 template <class C>
@@ -926,10 +937,9 @@ __global__ __launch_bounds__(ST_THREADS) void gemv_stream_kernel(DMat m, const u
       const int k = p.k;
 #pragma unroll
       for (int i = 0; i < M; ++i) {
-        float v = ysum[i];
+        const float v0 = ysum[i];
         ysum[i] = 0.f;
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+        float v = wave_sum_dpp(v0);
         if (lane == 0) {
           if (bias) v += (ydt == CBK_F32) ? ((const float*)bias)[k]
                        : (ydt == CBK_F16) ? h2f(((const uint16_t*)bias)[k]) : bf2f(((const uint16_t*)bias)[k]);
@@ -1115,10 +1125,9 @@ __global__ __launch_bounds__(ST_THREADS) void gemv_dense8_kernel(DMat m, const u
       const int k = p.k;
 #pragma unroll
       for (int i = 0; i < M; ++i) {
-        float v = ysum[i];
+        const float v0 = ysum[i];
         ysum[i] = 0.f;
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+        float v = wave_sum_dpp(v0);
         if (lane == 0) {
           if (bias) v += (ydt == CBK_F32) ? ((const float*)bias)[k]
                        : (ydt == CBK_F16) ? h2f(((const uint16_t*)bias)[k]) : bf2f(((const uint16_t*)bias)[k]);
