@@ -96,3 +96,21 @@ def test_gemv_between_one_and_two_tiles_per_workgroup():
         ref = x.double() @ W.t()
         assert float((y.double() - ref).abs().max() / ref.abs().max()) < 2e-5, K
         assert torch.equal(ops.gemv(pm, x[1:2], out_dtype=torch.float32)[0], y[1])
+
+
+@pytest.mark.parametrize("layout", [F.SPARSE4, F.SPARSE4X, F.SPARSE4E], ids=lambda l: F.LAYOUT_NAME[l])
+def test_synthetic_survivor_streams(layout):
+    """The synthetic variable-length matrices the benchmark times: the device dequantiser reads them
+    as the oracle does (bit for bit), and the decode kernel agrees with float64 on those weights."""
+    K, N = 200, 1152
+    pm = F.synth_packed(K, N, layout, seed=2, device=DEV)
+    W = ops.dequant(pm, torch.float32)
+    pk = dict(data=pm.array("data").cpu().numpy(), scale=pm.array("scale").cpu().numpy().reshape(K, -1),
+              zero=pm.array("zero").cpu().numpy().reshape(K, -1), row_off=pm.array("row_off").cpu().numpy().view(np.uint32))
+    cs = pm.array("col_scale").cpu().numpy().reshape(1, N)
+    assert np.array_equal(_np(W), R.dequant(pk, K, N, layout, col_scale=cs[0]))
+    for M in (1, 5):
+        x = acts(M, N, torch.float16, seed=M).to(DEV)
+        y = ops.gemv(pm, x, out_dtype=torch.float32)
+        ref = x.double() @ W.double().t()
+        assert float((y.double() - ref).abs().max() / ref.abs().max()) < 2e-5, M
