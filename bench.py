@@ -213,11 +213,12 @@ def decode_layer_sets(torch, F, L, dev, shapes, sets, M, dt, launch, steps, warm
     return res, xs, y_first
 
 
-def per_matrix(torch, F, L, dev, shapes, layout, bits, group, keep, M, dt, iters=24, tiled=True):
+def per_matrix(torch, F, L, dev, shapes, layout, bits, group, keep, M, dt, iters=24, tiled=True, use_graph=True):
     """Each distinct matrix of the layer set on its own: one launch per matrix, distinct copies of
     at least 512 MB in rotation (the protocol of src/cobaltkernel/test_gemv.py:201-202, :521-522),
-    one HIP graph per rotation.  tiled=False keeps the row-major order (the survivor-stream
-    layouts have no other)."""
+    one HIP graph per rotation, or launches from the host with use_graph=False (counter runs:
+    the profiler's counter collection is kept away from graph capture and replay).  tiled=False
+    keeps the row-major order (the survivor-stream layouts have no other)."""
     rows, seen = [], set()
     stream = torch.cuda.Stream(dev)
     xdt = F.dtype_code(dt)
@@ -248,23 +249,26 @@ def per_matrix(torch, F, L, dev, shapes, layout, bits, group, keep, M, dt, iters
         with torch.cuda.stream(stream):
             rotation()
             stream.synchronize()
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g, stream=stream):
-                rotation()
+            g = None
+            if use_graph:
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=stream):
+                    rotation()
+            once = g.replay if use_graph else rotation
             for _ in range(3):
-                g.replay()
+                once()
             stream.synchronize()
             reps = max(1, -(-iters // copies))
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(stream)
             for _ in range(reps):
-                g.replay()
+                once()
             e1.record(stream)
             stream.synchronize()
         us = e0.elapsed_time(e1) * 1e3 / (reps * copies)
         nbytes = algorithmic_bytes(pms[0], M)
         rows.append({"matrix": f"{name} {K}x{N}", "bytes": nbytes, "distinct_copies": copies, "launches_timed": reps * copies,
-                     "us": round(us, 2), "gbs": round(nbytes / us / 1e3, 1),
+                     "hip_graph": use_graph, "us": round(us, 2), "gbs": round(nbytes / us / 1e3, 1),
                      "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
         del pms, args, g, x, y, w
         torch.cuda.empty_cache()
@@ -392,6 +396,151 @@ def library_dense_gemm_ms(torch, dev, M, K, N, dt, x, reps=10, warm=5):
     return e0.elapsed_time(e1) / reps
 
 
+
+def decode_parity(torch, ops, pm, x, y):
+    """rel. Frobenius error of decode outputs y [M, K] (float32) against x.double() @ W.double().T with W
+    the library's bit-exact dequantisation of the same packed bytes (float64 on the GPU)."""
+    W = ops.dequant(pm, torch.float32).double()
+    ref = x.double() @ W.T
+    err = float((y.double() - ref).norm() / ref.norm())
+    del W, ref
+    return err
+
+
+def decode_rows_sweep(torch, F, L, dev, workload, layout, bits, group, keep, Ms, steps, warmup, use_graph=True,
+                      launch="phase", parity=False, ops=None):
+    """The decode step of one workload at several activation row counts on the same resident layer
+    sets (built once)."""
+    shapes = SHAPES[workload]
+    dt = torch_dtype(torch, WORKLOAD_DTYPE[workload])
+    sets, _ = make_sets(torch, F, dev, shapes, layout, bits, group, keep, 2 * INFINITY_CACHE)
+    out = {}
+    for M in Ms:
+        res, xs, y_first = decode_layer_sets(torch, F, L, dev, shapes, sets, M, dt, launch, steps, warmup, use_graph)
+        row = {"workload": f"{workload} decode layer set, 7 GEMVs, M={M}, {WORKLOAD_DTYPE[workload]} activations, "
+                           f"{F.LAYOUT_NAME[layout]} {bits}-bit keep {keep}/32 group {group}, {sets[0][0].bpw():.4f} bpw",
+               "M": M, "ms_per_step": round(res["ms_per_step"], 5), "gbs": round(res["gbs"], 1),
+               "frac_of_hbm_peak": round(res["gbs"] / HBM_PEAK_GBS, 4), "layer_set_bytes": res["step_bytes"],
+               "distinct_layer_sets": res["distinct_layer_sets"], "steps": steps, "hip_graph": use_graph}
+        if parity:
+            worst = max(decode_parity(torch, ops, pm, xs[N], y_first[name]) for pm, (name, _, N) in zip(sets[0], shapes))
+            assert worst < 1e-3, f"{workload} M={M}: decode outputs off the dequantised weights by {worst}"
+            row["parity"] = {"worst_rel_fro": float(f"{worst:.3g}"), "tolerance": 1e-3,
+                             "how": "every matrix of the first layer set, float32 output against x.double() @ "
+                                    "dequant(W).double().T (bit-exact dequantiser of the same bytes)"}
+        out[M] = row
+        del xs, y_first
+    del sets
+    torch.cuda.empty_cache()
+    return out
+
+
+def config0_single_layer(torch, F, ops, L, dev, cpu=True):
+    """The reference's own CPU-runnable case: W 4096x4096 ~ N(0, 0.02) with 1 % of the columns
+    scaled by 10, calibration activations 128x4096 ~ N(0, 1) for the Wanda score and the OBS
+    update, column-balanced mask at sparsity 0.5, 4-bit RTN in groups of 128, packed as BLK1632_4;
+    x is 1x4096 fp16.  Compressed and packed on the GPU by this package, decoded at M=1."""
+    import numpy as np
+    from cobalt_amd.linear import CobaltLinear
+    g = torch.Generator().manual_seed(0)
+    K = N = 4096
+    W = torch.randn(K, N, generator=g) * 0.02
+    W[:, torch.randperm(N, generator=g)[:41]] *= 10
+    X = torch.randn(128, N, generator=g)
+    x = torch.randn(1, N, generator=g).half()
+    lin = torch.nn.Linear(N, K, bias=False)
+    lin.weight.data.copy_(W)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    m = CobaltLinear.from_linear(lin.to(dev), X_cal=X.to(dev), sparsity=0.5, bits=4, group=128)
+    torch.cuda.synchronize()
+    t_compress = time.perf_counter() - t0
+    pm_rm = m.packed()
+    pm = pm_rm.to_tiled()
+    xd = x.to(dev)
+    y32 = ops.gemv(pm, xd, out_dtype=torch.float32)
+    err = decode_parity(torch, ops, pm, xd, y32)
+    assert err < 1e-3, f"config 0: decode off the dequantised weights by {err}"
+    dense = xd.float() @ W.to(dev).T
+    vs_dense = float((y32 - dense).norm() / dense.norm())
+    copies = [pm] + [pm.clone() for _ in range(-(-2 * INFINITY_CACHE // pm.stream_bytes()) - 1)]
+    st = torch.cuda.current_stream()
+    y = None
+    for c in copies:
+        y = ops.gemv(c, xd)
+    torch.cuda.synchronize()
+    g_ = torch.cuda.CUDAGraph()
+    stream = torch.cuda.Stream(dev)
+    stream.wait_stream(st)
+    with torch.cuda.stream(stream):
+        ys = torch.empty(1, K, dtype=torch.float16, device=dev)
+        P = ctypes.c_void_p
+        xdt = F.dtype_code(torch.float16)
+        args = [((F.CbkDesc * 1)(c.desc()), (P * 1)(xd.data_ptr()), (ctypes.c_int64 * 1)(N), (P * 1)(ys.data_ptr()),
+                 (ctypes.c_int64 * 1)(K)) for c in copies]
+
+        def rotation():
+            for d, xp, ldx, yp, ldy in args:
+                rc = L.cbk_gemv_batch(1, d, xp, ldx, xdt, 1, yp, ldy, xdt, None, None, 0, stream.cuda_stream)
+                if rc:
+                    raise RuntimeError(L.cbk_strerror(rc).decode())
+        rotation()
+        stream.synchronize()
+        with torch.cuda.graph(g_, stream=stream):
+            rotation()
+        for _ in range(3):
+            g_.replay()
+        stream.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(3):
+            g_.replay()
+        e1.record(stream)
+        stream.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / (3 * len(copies))
+    nbytes = algorithmic_bytes(pm, 1)
+    out = {"workload": "single linear layer 4096x4096, CoBALT-compressed on the GPU (column-balanced mask, sparsity 0.5, "
+                       "OBS, 4-bit RTN, group 128) -> BLK1632_4, x 1x4096 fp16",
+           "bpw": round(pm.bpw(), 4), "compress_and_pack_s": round(t_compress, 3), "decode_us": round(us, 2),
+           "distinct_copies": len(copies), "bytes": nbytes, "gbs": round(nbytes / us / 1e3, 1),
+           "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+           "rel_fro_vs_dequant_f64": float(f"{err:.3g}"), "rel_fro_vs_uncompressed_layer": float(f"{vs_dense:.3g}")}
+    if cpu:
+        from oracle import cbk_ref_c as C
+        from oracle import torch_ref as T
+        cpm = pm_rm.to("cpu")
+        stride = cpm.data_bytes // K
+        data = cpm.array("data")[: K * stride].reshape(K, stride)
+        scale, zero = cpm.array("scale").reshape(K, -1), cpm.array("zero").reshape(K, -1)
+        cs = cpm.array("col_scale").reshape(1, N)
+        pk = dict(data=cpm.array("data").numpy(), scale=scale.numpy(), zero=zero.numpy())
+        yo = C.forward(pk, K, N, cpm.layout, x.float().numpy(), col_scale=cs.numpy())
+        out["gpu_vs_oracle_rel_fro"] = float(np.linalg.norm(y32.cpu().numpy() - yo) / np.linalg.norm(yo))
+        assert out["gpu_vs_oracle_rel_fro"] < 1e-3
+        ta = []
+        for i in range(6):
+            t0 = time.perf_counter()
+            Wh = T.dequant(data, scale, zero, cs, K, N, cpm.layout, 4, 128, 16)
+            T.forward(Wh, x)
+            ta.append(time.perf_counter() - t0)
+        out["cpu_dequant_matmul_ms"] = round(sorted(ta[1:])[2] * 1e3, 2)
+        out["cpu_note"] = "torch float32 dequantise-then-matmul of the same packed bytes on the host cores, median of 5 after a warm-up"
+    del copies, g_
+    torch.cuda.empty_cache()
+    return out
+
+
+def config2_block(torch, F, ops, L, dev, steps, warmup, use_graph=True):
+    """Mistral-7B shapes at sparsity 0.7 (10 survivors per 32 columns), 3-bit codes, group 128:
+    decode at M=1 and the MLP prefill at M=2048, fp16 activations, each with its parity figure."""
+    dec = decode_rows_sweep(torch, F, L, dev, "mistral7b", F.BLKC, 3, 128, 10, [1], steps, warmup, use_graph, parity=True, ops=ops)[1]
+    pf = prefill_gemm(torch, F, ops, dev, SHAPES["mistral7b"], ["gate", "up", "down"], F.BLKC, 3, 128, 10, 2048, torch.float16,
+                      reps=10, warm=5)
+    pf["workload"] = "mistral7b MLP (gate, up, down), M=2048, f16 activations"
+    return {"workload": "mistral7b shapes, sparsity 0.6875 (10 of 32 kept), 3-bit codes across word boundaries, group 128, "
+                        "f16 activations", "decode_m1": dec, "prefill_m2048": pf}
+
+
 # ------------------------------------------------------------------ ceilings and CPU baseline
 def measured_ceilings(torch, dev):
     """What this GPU reaches on back-to-back dense f16 MFMAs and on a plain streaming read of
@@ -446,12 +595,16 @@ def cpu_model():
     return platform.processor() or "unknown"
 
 
-def cpu_baseline(torch, pms, shapes, xs, ys, M, budget_s=25.0):
+def cpu_baseline(torch, pms, shapes, xs, ys, M, budget_s=18.0, prefill_budget_s=14.0, prefill_m=256, prefill_to=2048):
     """The reference's CPU forward restated in torch (oracle/torch_ref.py): per distinct shape of
     the layer set, (i) dequantise-then-matmul per call (the module's low-memory path,
     benchmarks/benchmark_suite.py:1201-1209) and (ii) matmul with the dequantised weights cached
     (:1210-1217), float32, all the host cores this process may use; on the packed bytes the GPU
-    used.  The C oracle checks the GPU outputs of the same layer set first."""
+    used.  Decode leg at M rows: one warm-up, then the median of 5 runs (fewer only if the time
+    budget runs out, and the JSON says how many).  Prefill leg at `prefill_m` rows per distinct
+    shape, with the figure for `prefill_to` rows extrapolated (dequantisation once, matmul time
+    in proportion to the rows) and flagged as such.  The C oracle checks the GPU outputs of the
+    same layer set first."""
     import numpy as np
     from oracle import cbk_ref_c as C
     from oracle import torch_ref as T
@@ -461,7 +614,6 @@ def cpu_baseline(torch, pms, shapes, xs, ys, M, budget_s=25.0):
     torch.set_num_threads(cores)
     C.set_threads(min(16, cores))
     worst = 0.0
-    t_stop = time.time() + budget_s
     for pm, (name, K, N) in zip(pms, shapes):                       # parity of the GPU outputs (checker, untimed)
         pk = dict(data=pm.array("data").numpy(), scale=pm.array("scale").numpy().reshape(K, -1),
                   zero=pm.array("zero").numpy().reshape(K, -1))
@@ -470,39 +622,45 @@ def cpu_baseline(torch, pms, shapes, xs, ys, M, budget_s=25.0):
                       keep_per_block=pm.keep or None)
         got = ys[name].float().cpu().numpy()
         worst = max(worst, float(np.linalg.norm(got - y) / np.linalg.norm(y)))
-    rows, seen = [], set()
+    rows, prows, seen = [], [], set()
     tot_bytes = tot_a = tot_b = 0.0
     order = sorted(range(len(shapes)), key=lambda i: shapes[i][1] * shapes[i][2])       # small shapes first
+    distinct = []
     for i in order:
+        if (shapes[i][1], shapes[i][2]) not in seen:
+            seen.add((shapes[i][1], shapes[i][2]))
+            distinct.append(i)
+
+    def arrays(pm, K, N):
+        stride = pm.data_bytes // K
+        return (pm.array("data")[: K * stride].reshape(K, stride), pm.array("scale").reshape(K, -1), pm.array("zero").reshape(K, -1),
+                pm.array("col_scale").reshape(pm.cs_rows, N) if pm.cs_rows else None)
+
+    med = lambda v: sorted(v)[len(v) // 2]
+    t_stop = time.time() + budget_s
+    for i in distinct:
         name, K, N = shapes[i]
-        if (K, N) in seen:
-            continue
         if rows and time.time() > t_stop:
             break
-        seen.add((K, N))
         pm = pms[i]
-        stride = pm.data_bytes // K
-        data = pm.array("data")[: K * stride].reshape(K, stride)
-        scale = pm.array("scale").reshape(K, -1)
-        zero = pm.array("zero").reshape(K, -1)
-        cs = pm.array("col_scale").reshape(pm.cs_rows, N) if pm.cs_rows else None
+        data, scale, zero, cs = arrays(pm, K, N)
         x = xs[N].cpu()
         deq = lambda: T.dequant(data, scale, zero, cs, K, N, pm.layout, pm.bits, pm.group, pm.keep or 16)
         W = deq()
         T.forward(W, x)                                               # warm-up of both parts
         ta, tb = [], []
-        for _ in range(3):
+        for _ in range(5):
             t0 = time.perf_counter()
             W = deq()
             y = T.forward(W, x)
             ta.append(time.perf_counter() - t0)
-            if time.time() > t_stop:
+            if time.time() > t_stop and len(ta) >= 3:
                 break
         for _ in range(5):
             t0 = time.perf_counter()
             y = T.forward(W, x)
             tb.append(time.perf_counter() - t0)
-        a, b = sorted(ta)[len(ta) // 2], sorted(tb)[len(tb) // 2]
+        a, b = med(ta), med(tb)
         nbytes = algorithmic_bytes(pm, M)
         mult = sum(1 for _, k, n in shapes if (k, n) == (K, N))
         tot_bytes += nbytes * mult
@@ -511,20 +669,56 @@ def cpu_baseline(torch, pms, shapes, xs, ys, M, budget_s=25.0):
         rows.append({"matrix": f"{name} {K}x{N}", "dequant_matmul_ms": round(a * 1e3, 2), "matmul_cached_ms": round(b * 1e3, 3),
                      "runs": [len(ta), len(tb)]})
         del W, y
+    # prefill leg
+    t_stop = time.time() + prefill_budget_s
+    pf_flop = pf_s = 0.0
+    for i in distinct:
+        name, K, N = shapes[i]
+        if prows and time.time() > t_stop:
+            break
+        pm = pms[i]
+        data, scale, zero, cs = arrays(pm, K, N)
+        x = torch.randn(prefill_m, N, generator=torch.Generator().manual_seed(N)).to(xs[N].dtype)
+        W = T.dequant(data, scale, zero, cs, K, N, pm.layout, pm.bits, pm.group, pm.keep or 16)
+        T.forward(W, x)
+        td, tm = [], []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            W = T.dequant(data, scale, zero, cs, K, N, pm.layout, pm.bits, pm.group, pm.keep or 16)
+            t1 = time.perf_counter()
+            y = T.forward(W, x)
+            t2 = time.perf_counter()
+            td.append(t1 - t0)
+            tm.append(t2 - t1)
+            if time.time() > t_stop and len(td) >= 3:
+                break
+        d_, m_ = med(td), med(tm)
+        ext = d_ + m_ * prefill_to / prefill_m
+        mult = sum(1 for _, k, n in shapes if (k, n) == (K, N))
+        pf_flop += 2.0 * prefill_to * K * N * mult
+        pf_s += ext * mult
+        prows.append({"matrix": f"{name} {K}x{N}", "M": prefill_m, "dequant_ms": round(d_ * 1e3, 2), "matmul_ms": round(m_ * 1e3, 2),
+                      "runs": len(td), f"extrapolated_ms_at_M{prefill_to}": round(ext * 1e3, 1), "extrapolated": True})
+        del W, y
     done = "+".join(r["matrix"].split()[0] for r in rows)
     return dict(value=round(tot_bytes / tot_a / 1e9, 4), unit="GB/s", cores=cores, kind="port",
                 sample=f"torch {torch.__version__} float32 dequantise-then-matmul per call at M={M} over the distinct shapes "
-                       f"{done} of the first layer set (same packed bytes as the GPU run), median of up to 3 runs each after one "
-                       f"warm-up, {cores} threads on {cpu_model()} ({os.cpu_count()} logical CPUs visible); `value` is the "
+                       f"{done} of the first layer set (same packed bytes as the GPU run), median of 5 runs each (see `runs`) "
+                       f"after one warm-up, {cores} threads on {cpu_model()} ({os.cpu_count()} logical CPUs visible); `value` is the "
                        f"algorithmic bytes of those matrices per second of the per-call path; `matmul_cached_gbs` is the "
-                       f"same bytes over the matmul with cached float32 weights (median of 5)",
+                       f"same bytes over the matmul with cached float32 weights (median of 5); `prefill` is the same path "
+                       f"at M={prefill_m}, its M={prefill_to} figures extrapolated, not measured",
                 matmul_cached_gbs=round(tot_bytes / tot_b / 1e9, 3), per_matrix=rows,
                 ms_per_layer_set_dequant_matmul=round(tot_a * 1e3, 1), ms_per_layer_set_matmul_cached=round(tot_b * 1e3, 2),
+                prefill={"M_measured": prefill_m, "M_extrapolated_to": prefill_to, "per_matrix": prows,
+                         "extrapolated_tflops": round(pf_flop / pf_s / 1e12, 3) if pf_s else None,
+                         "shapes_done": "+".join(r["matrix"].split()[0] for r in prows),
+                         "note": "dequantise once + matmul time scaled by rows; an extrapolation, flagged per row"},
                 gpu_vs_oracle_rel_fro=worst, checker="C oracle (oracle/cbk_ref.c) on every matrix of the first layer set")
 
 
 # ------------------------------------------------------------------ the nine-cell grid
-def grid(torch, F, ops, L, dev, a):
+def grid(torch, F, ops, L, dev, a, prefill_reps=5, prefill_warm=3):
     """Gemma-3-27B shapes x 62 layers, sparsity 0.3 / 0.5 / 0.7 as 23 / 16 / 10 survivors per 32
     columns, 2 / 3 / 4-bit codes, group 64: decode step at M=1 and prefill at M=4096, bf16."""
     shapes = SHAPES["gemma27b"]
@@ -534,12 +728,12 @@ def grid(torch, F, ops, L, dev, a):
     for keep in (23, 16, 10):
         for bits in (2, 3, 4):
             sets, _ = make_sets(torch, F, dev, shapes, F.BLKC, bits, 64, keep, 2 * INFINITY_CACHE)
-            res, _, _ = decode_layer_sets(torch, F, L, dev, shapes, sets, 1, dt, "phase", a.steps, a.warmup)
+            res, _, _ = decode_layer_sets(torch, F, L, dev, shapes, sets, 1, dt, "phase", a.steps, a.warmup, not a.no_graph)
             bpw = sets[0][0].bpw()
             del sets
             torch.cuda.empty_cache()
             pf = prefill_gemm(torch, F, ops, dev, shapes, [n for n, _, _ in shapes], F.BLKC, bits, 64, keep, a.grid_prefill_m, dt,
-                              reps=5, warm=3, parity=False)
+                              reps=prefill_reps, warm=prefill_warm, parity=False)
             cell = {"sparsity": round(1 - keep / 32, 4), "keep_per_32": keep, "bits": bits, "group": 64, "bpw": round(bpw, 4),
                     "layer_set_bytes": res["step_bytes"],
                     "decode_ms_per_layer": round(res["ms_per_step"], 5), "decode_gbs": round(res["gbs"], 1),
@@ -586,6 +780,10 @@ def main():
                     help="also run a 1 GiB device-to-device copy (reference reading for the HBM traffic counters)")
     ap.add_argument("--grid", action="store_true", help="the nine-cell sweep of the 62-layer Gemma stack instead of the headline")
     ap.add_argument("--grid-prefill-m", type=int, default=4096)
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the legs of the other benchmark configurations (single layer, M=4/8, 3-bit Mistral, the grid)")
+    ap.add_argument("--only", default=None, choices=["per-matrix", "row-kernels"],
+                    help="run one secondary leg alone (profiling runs): the per-matrix rows or the row-kernel layouts")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -604,6 +802,16 @@ def main():
     dt = torch_dtype(torch, dname)
     shapes = SHAPES[a.workload]
     M = a.m
+    if a.only:                                                      # one leg alone, for profiler runs
+        gate = [sh for sh in shapes if sh[0] == "gate"]
+        if a.only == "per-matrix":
+            rows = per_matrix(torch, F, L, dev, shapes, layout, a.bits, a.group, a.keep, M, dt, use_graph=not a.no_graph)
+        else:
+            rows = [dict(layout=F.LAYOUT_NAME[lay], **per_matrix(torch, F, L, dev, gate, lay, b, 128, None, M, dt, tiled=False,
+                                                                 use_graph=not a.no_graph)[0])
+                    for lay, b in ((F.SPARSE4X, 4), (F.DENSE8, 8))]
+        print(json.dumps({"leg": a.only, "workload": a.workload, "M": M, "rows": rows}))
+        return
 
     sets, first_rowmajor = make_sets(torch, F, dev, shapes, layout, a.bits, a.group, a.keep, 2 * INFINITY_CACHE,
                                      keep_first_rowmajor=not a.no_cpu)
@@ -650,11 +858,12 @@ def main():
                      "launches_timed": a.steps * launches, "bytes_per_launch": int(bytes_per_launch)},
     }
     if not a.no_secondary:
-        out["per_matrix"] = per_matrix(torch, F, L, dev, shapes, layout, a.bits, a.group, a.keep, M, dt)
+        out["per_matrix"] = per_matrix(torch, F, L, dev, shapes, layout, a.bits, a.group, a.keep, M, dt, use_graph=not a.no_graph)
         # the layouts that decode on the row kernels (integer dot products), on the workload's gate matrix
         gate = [sh for sh in shapes if sh[0] == "gate"]
         out["row_kernel_layouts"] = [
-            dict(layout=F.LAYOUT_NAME[lay], **per_matrix(torch, F, L, dev, gate, lay, b, 128, None, M, dt, tiled=False)[0])
+            dict(layout=F.LAYOUT_NAME[lay], **per_matrix(torch, F, L, dev, gate, lay, b, 128, None, M, dt, tiled=False,
+                                                         use_graph=not a.no_graph)[0])
             for lay, b in ((F.SPARSE4X, 4), (F.DENSE8, 8))]
         other = "mistral7b" if a.workload == "gemma27b" else "gemma27b"
         oshapes, odt = SHAPES[other], torch_dtype(torch, WORKLOAD_DTYPE[other])
@@ -678,6 +887,17 @@ def main():
                            "tflops": mid["tflops"], "per_matrix": mid["per_matrix"]}
     if not a.no_lm_head:
         out["lm_head_gemv"] = lm_head_gemv(torch, F, ops, dev, a.workload, M, dt)
+    if not a.no_configs:
+        # the other configurations the benchmark names, each a block of its own
+        g = not a.no_graph
+        out["config0_single_layer"] = config0_single_layer(torch, F, ops, L, dev, cpu=not a.no_cpu)
+        rows = {wl: decode_rows_sweep(torch, F, L, dev, wl, layout, a.bits, a.group, a.keep, [4, 8], a.steps, a.warmup, g,
+                                      a.launch, parity=True, ops=ops) for wl in ("mistral7b", "gemma27b")}
+        out["config1_mistral7b_m4"], out["config1_mistral7b_m8"] = rows["mistral7b"][4], rows["mistral7b"][8]
+        out["config3_gemma27b_m4"], out["config3_gemma27b_m8"] = rows["gemma27b"][4], rows["gemma27b"][8]
+        out["config2_mistral7b_b3_keep10"] = config2_block(torch, F, ops, L, dev, a.steps, a.warmup, g)
+        cells = grid(torch, F, ops, L, dev, a, prefill_reps=3, prefill_warm=2)
+        out["config4_grid"] = {"workload": cells["config"]["workload"], "cells": cells["cells"]}
     ceil = measured_ceilings(torch, dev)
     if ceil:
         out["measured_ceilings"] = ceil

@@ -183,8 +183,7 @@ def matrix_from_entry(e: dict, blob: torch.Tensor) -> F.PackedMatrix:
     pm = F.PackedMatrix(blob, offs, K, N, layout, bits, group, keep, cs_rows, _cs_splits(e), data_bytes,
                         int(e.get("n_survivors", 0)), int(e.get("n_zero_fixed", 0)))
     pm.validate(deep=blob.device.type == "cpu")
-    if int(pm.array("zero").max()) <= 128:
-        pm.flags |= F.FLAG_ZERO_LE_128
+    pm.flags |= F.zero_flags(int(pm.array("zero").max()), bits)
     if e.get("fused_from"):
         pm.meta["fused_from"] = list(e["fused_from"])
     return pm

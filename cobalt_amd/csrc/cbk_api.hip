@@ -167,6 +167,13 @@ static int check_io(const void* x, int xdt, int M, int64_t ldx, const void* y, i
 // the duration of the call, as the dense 4-bit layout in tiled order (pruned columns hold the
 // zero point, so every weight dequantises to the same value) and runs the prefill kernel on that:
 // two small kernels (image -> codes and bitmap, codes -> rows) in front of the matrix product.
+// A pruned column of the dense image stores the zero point as its code, so this needs every zero
+// point to be a 4-bit code itself (CBK_FLAG_ZERO_ON_GRID: the host cannot look), and a fixed row
+// stride cannot carry row-fused column scales; such matrices, and calls without the workspace,
+// are served by the row kernel in slices of 16 activation rows.
+static inline bool sparse_repackable(const DMat& m) {
+  return m.cs_rows <= 1 && (m.flags & CBK_FLAG_ZERO_ON_GRID) != 0;
+}
 struct Transient {
   size_t q, mask, data, scale, zero, end;   // byte offsets in the workspace, 256-byte aligned
 };
@@ -236,7 +243,7 @@ size_t cbk_workspace_bytes(const cbk_desc* in, int M) {
   DMat m;
   if (to_dmat(in, &m, false)) return 0;
   if (family_of(m.layout) == FAM_SPARSE) {                          // cbk_gemm / cbk_linear above 16 rows: see Transient
-    if (M <= 16) return 0;
+    if (M <= 16 || !sparse_repackable(m)) return 0;                 // the row kernel needs none
     const Transient t = transient_dense4(m);
     return t.end + gemm_big_workspace(dense4_view(m, nullptr, t), M);
   }
@@ -380,10 +387,21 @@ int cbk_gemm(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ldx,
   if (family_of(m.layout) == FAM_SPARSE) {
     if (M <= 16)                                                    // not worth re-packing: the row kernel
       return cbk_gemv(in, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, workspace, workspace_bytes, stream);
-    if (m.cs_rows > 1) return CBK_ERR_UNSUPPORTED;                  // row fusion needs a fixed row stride
     const Transient t = transient_dense4(m);
-    if (!workspace || workspace_bytes < t.end) return CBK_ERR_WORKSPACE;
-    if ((uintptr_t)workspace & 255) return CBK_ERR_ALIGN;
+    const bool room = workspace && !((uintptr_t)workspace & 255) &&
+                      workspace_bytes >= t.end + gemm_big_workspace(dense4_view(m, nullptr, t), M);
+    if (!sparse_repackable(m) || !room) {
+      // zero points that are no 4-bit codes, row-fused column scales, or no room for the dense
+      // image: the row kernel, sixteen activation rows per pass, without a workspace
+      const size_t ysz = y_dtype == CBK_F32 ? 4 : 2;
+      for (int m0 = 0; m0 < M; m0 += 16) {
+        const int mc = M - m0 < 16 ? M - m0 : 16;
+        rc = cbk_gemv(in, (const uint8_t*)x + (size_t)m0 * ldx * 2, x_dtype, mc, ldx,
+                      (uint8_t*)y + (size_t)m0 * ldy * ysz, y_dtype, ldy, bias, nullptr, 0, stream);
+        if (rc) return rc;
+      }
+      return CBK_OK;
+    }
     uint8_t* ws = (uint8_t*)workspace;
     const DMat d = dense4_view(m, ws, t);
     rc = launch_unpack(m, ws + t.q, ws + t.mask, (hipStream_t)stream);
@@ -461,19 +479,8 @@ int cbk_linear(const cbk_desc* in, const void* x, int x_dtype, int M, int64_t ld
   // up to 8 rows (one or two passes of the decode kernel) the weights are streamed faster than the
   // prefill kernel's 64-token tile decodes them (14336 x 4096: 28 us against 31 us; 54 us at 16 rows)
   if (M <= 8) return cbk_gemv(in, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, workspace, workspace_bytes, stream);
-  cbk_desc d;
-  if (in && canon(in, &d) == CBK_OK && family_of(d.layout) == FAM_SPARSE && (M <= 16 || d.cs_rows > 1)) {
-    // the variable-length layouts have no MFMA path of their own: up to 16 rows the row GEMV (more
-    // rows go through cbk_gemm, which re-packs the matrix for the call)
-    for (int m0 = 0; m0 < M; m0 += 16) {
-      const int mc = M - m0 < 16 ? M - m0 : 16;
-      int rc = cbk_gemv(in, (const uint8_t*)x + (size_t)m0 * ldx * 2, x_dtype, mc, ldx,
-                        (uint8_t*)y + (size_t)m0 * ldy * (y_dtype == CBK_F32 ? 4 : 2), y_dtype, ldy, bias,
-                        workspace, workspace_bytes, stream);
-      if (rc) return rc;
-    }
-    return CBK_OK;
-  }
+  // (the variable-length layouts have no matrix-core path of their own: cbk_gemm sends them to the
+  // row kernel or re-packs them for the call)
   return cbk_gemm(in, x, x_dtype, M, ldx, y, y_dtype, ldy, bias, workspace, workspace_bytes, stream);
 }
 

@@ -81,11 +81,12 @@ __device__ inline uint16_t f2bf(float f) {            // round to nearest even
   return (uint16_t)(u >> 16);
 }
 __device__ inline uint16_t f2h(float f) { return __half_as_ushort(__float2half_rn(f)); }
-// The power of two s >= 1 with mx / s in [2^14, 2^15) for a finite mx >= 2^15, else 1.  The GEMM
+// The power of two s >= 1 with mx / s in [2^14, 2^15) for a finite mx >= 2^15, else 1 (the
+// exponent arithmetic holds for every finite float; an infinite or NaN maximum is left alone).  The GEMM
 // kernels feed the fp16 matrix pipe: a token whose activations reach beyond fp16's range is
 // divided by s before the cast and its outputs are multiplied by s, both exact.
 __device__ inline float token_scale(float mx) {
-  if (!(mx >= 32768.f) || mx > 3.0e38f) return 1.f;
+  if (!(mx >= 32768.f) || !(mx <= 3.4028234663852886e38f)) return 1.f;
   const uint32_t e = ((__float_as_uint(mx) >> 23) & 0xffu) - 14u;      // biased exponent of mx, less 14
   return __uint_as_float(e << 23);
 }

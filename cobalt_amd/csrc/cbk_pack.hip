@@ -34,7 +34,7 @@ struct BitSink {
   int n = 0;
   uint32_t o;
   __device__ inline void put(const PackArgs& a, int k, uint32_t code, int bits) {
-    acc |= (uint64_t)code << n;
+    acc |= (uint64_t)(code & ((1u << bits) - 1u)) << n;            // never into the neighbouring code
     n += bits;
     while (n >= 8) { *dst_byte(a, k, o++) = (uint8_t)acc; acc >>= 8; n -= 8; }
   }
@@ -90,7 +90,9 @@ __device__ inline GroupQ group_quant(const PackArgs& a, int k, int g, const uint
   return r;
 }
 
-// status[0] |= 1: a block without exactly `keep` survivors; status[1] += groups re-derived
+// status[0] |= 1: a block without exactly `keep` survivors; |= 2: a dense layout had to store a zero
+// point above 2^bits - 1 at a pruned column (its low bits are stored; the column no longer
+// dequantises to 0); status[1] += groups re-derived
 __global__ __launch_bounds__(256) void pack_rows_kernel(PackArgs a, int* status) {
   const int units = (a.N + 255) >> 8;
   const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -105,7 +107,7 @@ __global__ __launch_bounds__(256) void pack_rows_kernel(PackArgs a, int* status)
   BitSink sink;
   if (a.fam == FAM_DENSE) sink.o = (uint32_t)(c0 >> 3) * a.bits;
   else sink.o = (uint32_t)(a.N >> 3) + (uint32_t)(c0 >> 5) * a.keep * a.bits / 8;   // c0/32 is a multiple of 8
-  bool wrong = false;
+  bool wrong = false, off_grid = false;
   int fixed = 0, g_now = -1;
   GroupQ gq;
   for (int t = 0; t < nb; ++t) {
@@ -123,6 +125,7 @@ __global__ __launch_bounds__(256) void pack_rows_kernel(PackArgs a, int* status)
     *(uint4*)(c) = *(const uint4*)(qrow + 32 * t);
     *(uint4*)(c + 16) = *(const uint4*)(qrow + 32 * t + 16);
     if (a.fam == FAM_DENSE) {
+      if (m != 0xffffffffu && gq.z_out > (uint32_t)nl) off_grid = true;
 #pragma unroll
       for (int j = 0; j < 32; ++j) sink.put(a, k, ((m >> j) & 1u) ? gq.code(c[j], nl) : gq.z_out, a.bits);
       continue;
@@ -157,6 +160,7 @@ __global__ __launch_bounds__(256) void pack_rows_kernel(PackArgs a, int* status)
   sink.flush(a, k);
   if (status) {
     if (wrong) atomicOr(status, 1);
+    if (off_grid) atomicOr(status, 2);
     if (fixed) atomicAdd(status + 1, fixed);
   }
 }

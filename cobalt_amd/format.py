@@ -33,6 +33,12 @@ _SPARSE = (SPARSE4, SPARSE4X, SPARSE4E)
 F32, F16, BF16T = 0, 1, 2
 FLAG_ZERO_LE_128 = 1
 FLAG_TILED16 = 2
+FLAG_ZERO_ON_GRID = 4          # every stored zero point is itself a code (<= 2^bits - 1)
+
+
+def zero_flags(zero_max: int, bits: int) -> int:
+    """The two promises about the zero points a descriptor can carry (include/cbk.h)."""
+    return (FLAG_ZERO_LE_128 if zero_max <= 128 else 0) | (FLAG_ZERO_ON_GRID if zero_max <= (1 << bits) - 1 else 0)
 TILED_TAIL = 512
 
 
@@ -449,7 +455,7 @@ def pack_raw(mask_bits: Optional[torch.Tensor], q: torch.Tensor, scale: torch.Te
         cs_rows = cs.shape[0]
         arrays["col_scale"] = cs
     blob, offs = _assemble(arrays, dev)
-    flags = FLAG_ZERO_LE_128 if int(out_zero.max()) <= 128 else 0
+    flags = zero_flags(int(out_zero.max()), bits)
     return PackedMatrix(blob, offs, K, N, layout, bits, group, kpb, cs_rows, tuple(cs_splits),
                         K * stride, n_surv, n_fixed, flags)
 
@@ -471,7 +477,7 @@ def from_arrays(data, scale, zero, col_scale, K, N, layout, bits=None, group=Non
         cs_rows = cs.shape[0]
         arrays["col_scale"] = cs.reshape(-1).clone(memory_format=torch.contiguous_format).view(torch.uint8)
     blob, offs = _assemble(arrays, dev)
-    flags = FLAG_ZERO_LE_128 if int(torch.as_tensor(zero).reshape(-1).view(torch.uint8).max()) <= 128 else 0
+    flags = zero_flags(int(torch.as_tensor(zero).reshape(-1).view(torch.uint8).max()), bits)
     return PackedMatrix(blob, offs, K, N, layout, bits, group, kpb, cs_rows, tuple(cs_splits),
                         data.numel() - BLOB_TAIL, flags=flags)
 
@@ -551,7 +557,7 @@ def _synth_sparse(K, N, layout, bits, group, g, dev, cs_rows) -> PackedMatrix:
         arrays["col_scale"] = (torch.rand(cs_rows, N, generator=g, device=dev) * 1.5 + 0.5).half()
     blob, offs = _assemble(arrays, dev)
     return PackedMatrix(blob, offs, K, N, layout, bits, group, 0, cs_rows, (0, 0), total, int(cnt.sum()), 0,
-                        FLAG_ZERO_LE_128)
+                        FLAG_ZERO_LE_128 | FLAG_ZERO_ON_GRID)
 
 
 def synth_packed(K: int, N: int, layout: int, bits=None, group=None, keep=None, seed: int = 0,
@@ -592,4 +598,4 @@ def synth_packed(K: int, N: int, layout: int, bits=None, group=None, keep=None, 
         arrays["col_scale"] = (torch.rand(cs_rows, N, generator=g, device=dev) * 1.5 + 0.5).half()
     blob, offs = _assemble(arrays, dev)
     return PackedMatrix(blob, offs, K, N, layout, bits, group, kpb, cs_rows, (0, 0), K * stride, n_surv, 0,
-                        FLAG_ZERO_LE_128)
+                        FLAG_ZERO_LE_128 | FLAG_ZERO_ON_GRID)

@@ -225,11 +225,14 @@ def pack_raw(mask_bits, q, scale, zero, col_scale, layout, bits=None, group=None
                              _stream_ptr(dev))
     _lib.check(rc, "cbk_pack")
     wrong, pm.n_zero_fixed = (int(v) for v in status.tolist())
-    if wrong:
+    if wrong & 2:
+        raise ValueError(f"{F.LAYOUT_NAME[layout]} stores the zero point as the code of a pruned column, and a zero point "
+                         f"of this matrix is above {nl}: such a column would not dequantise to 0 (pack with fix_zero=True, "
+                         f"or keep a bitmap layout)")
+    if wrong & 1:
         raise ValueError(f"{F.LAYOUT_NAME[layout]} needs exactly {kpb} survivors in every aligned block of "
                          f"{F.BLOCK} columns; the mask has a block with another count")
-    if int(pm.array("zero").max()) <= 128:
-        pm.flags |= F.FLAG_ZERO_LE_128
+    pm.flags |= F.zero_flags(int(pm.array("zero").max()), bits)
     return pm.validate()
 
 

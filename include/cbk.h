@@ -45,6 +45,7 @@ enum cbk_layout {
 
 #define CBK_FLAG_ZERO_LE_128 1
 #define CBK_FLAG_TILED16 2
+#define CBK_FLAG_ZERO_ON_GRID 4
 
 enum cbk_dtype { CBK_F32 = 0, CBK_F16 = 1, CBK_BF16T = 2, CBK_U8 = 3 /* cbk_pack's zero points only */ };
 
@@ -92,7 +93,12 @@ enum cbk_status {
  *             byte o of row k is at data[(k/16)*16*s + ((o/16)*16 + k%16)*16 + o%16], the
  *             scale / zero entry of (row k, group g) at index ((k/16)*G + g)*16 + k%16; K is
  *             padded with zero rows to a multiple of 16 and data ends with 512 readable bytes.
- *             Fixed-stride layouts only.  Every entry point takes both orders. */
+ *             Fixed-stride layouts only.  Every entry point takes both orders.
+ *             CBK_FLAG_ZERO_ON_GRID: the caller guarantees that every stored zero point is
+ *             <= 2^bits - 1, i.e. is itself a code.  Only then can a survivor-stream matrix be
+ *             re-packed as dense codes (a pruned column of a dense layout stores the zero point
+ *             as its code): without the flag cbk_gemm / cbk_linear serve SPARSE4 / 4X / 4E
+ *             above 16 rows as 16-row slices on the row kernel, which takes any zero point. */
 typedef struct cbk_desc {
   const void* data;
   const void* row_off;
@@ -152,9 +158,10 @@ int cbk_dequant(const cbk_desc* d, int row0, int nrows, int with_col_scale,
  * point lies outside [0, 2^bits - 1] gets scale, zero point and codes re-derived from the hull of
  * its dequantised survivors and 0, as _fix_zero_range does (src/cobaltkernel/pack_cobalt.py:55-87),
  * in correctly rounded float32 steps in that function's order.  `status`, if given, is two device
- * ints the caller has set to 0: status[0] becomes 1 when a block does not hold exactly `keep`
- * survivors (the bytes written for such a block are then meaningless), status[1] counts the
- * groups re-derived.  The byte layouts are the ones `pack_matrix` (pack_cobalt.py:98-250) writes
+ * ints the caller has set to 0: bit 0 of status[0] is set when a block does not hold exactly
+ * `keep` survivors (the bytes written for such a block are then meaningless), bit 1 when a dense
+ * layout had to store, at a pruned column, a zero point above 2^bits - 1 (only its low bits are
+ * stored: that column no longer dequantises to 0); status[1] counts the groups re-derived.  The byte layouts are the ones `pack_matrix` (pack_cobalt.py:98-250) writes
  * with torch operations. */
 int cbk_pack(const cbk_desc* dst, const void* mask_bits, const void* q, const void* scale,
              const void* zero, int zero_dtype, int fix_zero, int* status, void* stream);
@@ -196,8 +203,10 @@ int cbk_gemv_batch(int n, const cbk_desc* descs, const void* const* xs, const in
  * cbk_gemv; activations are carried as fp16 inside, a token whose values leave fp16's range
  * scaled by a power of two on the way in and back on the way out.  The survivor-stream layouts
  * (SPARSE4, SPARSE4X, SPARSE4E) are re-packed for the call, above 16 rows, into the dense 4-bit
- * layout inside the workspace (cbk_workspace_bytes counts it) and go to the row kernel below
- * that.  Replaces the harness entry `gemm` (test_gemm.cu:151-165) and cbk::gemm_tile
+ * layout inside the workspace (cbk_workspace_bytes counts it) when the descriptor carries
+ * CBK_FLAG_ZERO_ON_GRID, has at most one col_scale vector and the workspace is large enough;
+ * otherwise, and up to 16 rows, they go to the row kernel in slices of 16 activation rows,
+ * which needs no workspace.  Replaces the harness entry `gemm` (test_gemm.cu:151-165) and cbk::gemm_tile
  * (cobalt_gemm.cuh:243-609). */
 int cbk_gemm(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
              void* y, int y_dtype, int64_t ldy, const void* bias,
@@ -213,7 +222,10 @@ int cbk_gemm(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
  * rows of 5376 columns; prompts beyond that go through cbk_gemm).  All calls on one GPU share
  * that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race;
  * calls on one stream are safe.  Nothing in the array needs to start at zero and nothing is
- * carried from one call to the next. */
+ * carried from one call to the next.  The first call on a GPU looks up the array's address
+ * there, and the first call of each kernel configuration sets a kernel attribute: neither can
+ * be recorded, so make one call per GPU and configuration (same layout, code width, row count
+ * class) outside stream capture before capturing calls of it into a graph. */
 #define CBK_STATIC_SCRATCH_BYTES (16u << 20)
 int cbk_gemm_static(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
                     void* y, int y_dtype, int64_t ldy, const void* bias, void* stream);

@@ -1,6 +1,7 @@
 """The producer side on the GPU: the library's packing kernel (RAW arrays -> CBK1 rows, row-major
 or tiled) bit for bit against the oracle's packer, the torch packer and the reference's own bytes;
 the compressor run on the GPU against the reference's vectors."""
+import ctypes
 import os
 import time
 
@@ -8,7 +9,7 @@ import numpy as np
 import pytest
 import torch
 
-from cobalt_amd import compress as C, format as F, ops
+from cobalt_amd import _lib, compress as C, format as F, ops
 from cobalt_amd.linear import CobaltLinear
 from oracle import cbk_ref as R
 from helpers import FIXED_CASES, case_id, make_raw, oracle_pack
@@ -211,6 +212,37 @@ def test_survivor_streams_repacked_as_dense_rows(case):
             assert rel_fro(y, ref) < 1e-3, (case_id(case), M, p.layout)
     y = ops.gemm(pm, acts(5, N, torch.float16, seed=5).to(DEV), out_dtype=torch.float32)       # few rows: the row kernel
     assert rel_fro(y.cpu().numpy(), R.forward_ref(W, acts(5, N, torch.float16, seed=5).float().numpy())) < 1e-3
+
+
+def test_survivor_stream_with_zero_points_off_the_code_grid():
+    """A survivor-stream image may carry zero points that are no 4-bit codes (packed without the
+    repair).  A dense layout cannot hold such a matrix (a pruned column stores the zero point as
+    its code), so above 16 rows the call must not re-pack it: it runs as 16-row slices on the row
+    kernel and meets the oracle at every row count; re-packing it on request is refused; and the
+    packing kernel never lets a wide zero point spill into the neighbouring code."""
+    case = (F.SPARSE4X, 4, 128, 0)
+    K, N = 200, 1024
+    raw = R.synth_raw_matrix(K, N, 0.5, 4, seed=33)
+    raw["zero"] = raw["zero"].copy()
+    raw["zero"][::3, ::2] = 20                                   # off the grid, below 128
+    pk = oracle_pack(case, raw, fix_zero=False)
+    assert int(pk["zero"].max()) == 20
+    W = R.dequant(pk, K, N, F.SPARSE4X, col_scale=raw["col_scale"])
+    pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV)
+    assert pm.flags & F.FLAG_ZERO_LE_128 and not pm.flags & F.FLAG_ZERO_ON_GRID
+    assert _lib.lib().cbk_workspace_bytes(ctypes.byref(pm.desc()), 64) == 0
+    assert np.array_equal(ops.dequant(pm, torch.float32).cpu().numpy() + np.float32(0), W + np.float32(0))
+    for M in (1, 16, 17, 40):
+        x = acts(M, N, torch.bfloat16, seed=M)
+        y = ops.linear(pm, x.to(DEV), out_dtype=torch.float32).cpu().numpy()
+        assert rel_fro(y, R.forward_ref(W, x.float().numpy())) < 1e-3, M
+    with pytest.raises(ValueError, match="zero point"):
+        ops.transcode(pm, F.DENSE4)
+    # the same matrix with a workspace that would hold the dense image: still the row kernel
+    x = acts(17, N, torch.float16, seed=2)
+    ws = torch.empty(8 << 20, dtype=torch.uint8, device=DEV)
+    y = ops.gemm(pm, x.to(DEV), out_dtype=torch.float32, workspace=ws).cpu().numpy()
+    assert rel_fro(y, R.forward_ref(W, x.float().numpy())) < 1e-3
 
 
 def test_module_with_a_survivor_stream_matrix_can_be_repacked_at_load():

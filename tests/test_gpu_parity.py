@@ -591,7 +591,9 @@ def test_gemm_activations_beyond_fp16_range():
     the prefill kernels feed the fp16 matrix pipe, so such a token is scaled by a power of two on
     the way in and back on the way out.  Tokens 1, 70 and 299 carry values up to 1e36 / 1e9 / 7e4;
     every token, large or not, meets the float64 product to the usual tolerance, and the small
-    tokens give the same bits as in a call without the large ones."""
+    tokens give the same bits as in a call without the large ones.  Token 200 of the bf16 case holds
+    one value of 1.6e38, half of the largest finite bf16, so that its product with a column scale of
+    up to 2 is still a finite float32 at the very top of the range."""
     case = (F.BLK1632_4, 4, 128, 16)
     K, N, M = 512, 1024, 300
     for cs_rows, splits in ((1, (0, 0)), (2, (0, 0)), (3, (256, 128)), (3, (40, 24))):
@@ -603,13 +605,15 @@ def test_gemm_activations_beyond_fp16_range():
             for tok, top in zip((1, 70, 299), big):
                 xb[tok] = (x[tok].float() * (top / float(x[tok].float().abs().max()))).to(dtype)
                 xb[tok, 5] = top
+            if dtype == torch.bfloat16:
+                xb[200, 5] = 1.6e38
             y = ops.gemm(pm, xb.to(DEV), out_dtype=torch.float32)
             assert bool(torch.isfinite(y).all())
             ref = R.forward_ref(W, _np(xb))
-            for tok in (0, 1, 70, 150, 299):
+            for tok in (0, 1, 70, 150, 200, 299):
                 err = rel_fro(_np(y[tok:tok + 1]), ref[tok:tok + 1])
                 assert err < TOL, f"cs_rows={cs_rows} splits={splits} {dtype} token {tok}: {err}"
-            keep = [t for t in range(M) if t not in (1, 70, 299)]
+            keep = [t for t in range(M) if t not in (1, 70, 200, 299)]
             assert torch.equal(y[keep], small[keep])
             y64 = ops.gemm(pm, xb[:40].to(DEV), out_dtype=torch.float32)          # the 64-token instantiation
             small64 = ops.gemm(pm, x[:40].to(DEV), out_dtype=torch.float32)

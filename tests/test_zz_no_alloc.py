@@ -1,7 +1,9 @@
 """cbk_gemm_static (the entry point that takes no workspace and allocates nothing) against cbk_gemm
 on the same inputs, through the C ABI: the same kernels run in the same order, so the outputs are
-bit-identical.  Two calls in a row, the second on a smaller input, then the refusal of a call that
-needs more scratch than the library's array holds."""
+bit-identical.  Two calls in a row, the second on a smaller input; a call recorded into a HIP graph
+and replayed (after one eager call of the same configuration: the first call on a GPU looks up the
+array's address, which cannot be recorded), with the allocator's counters unchanged across it; then
+the refusal of a call that needs more scratch than the library's array holds."""
 import ctypes
 
 import pytest
@@ -38,6 +40,42 @@ def test_static_scratch_matches_cbk_gemm_twice():
     rc, got = _static(big, x, torch.bfloat16)
     assert rc == 0
     assert torch.equal(got, ops.gemm(big, x))
+
+
+def test_static_scratch_call_inside_a_graph_allocates_nothing():
+    g = torch.Generator(device=DEV).manual_seed(5)
+    pm = F.synth_packed(768, 5376, F.BLK1632_4, seed=13, device=DEV).to_tiled()
+    M = 300
+    x = torch.randn(M, pm.N, device=DEV, generator=g).to(torch.bfloat16)
+    want = ops.gemm(pm, x, out_dtype=torch.float32)
+    y = torch.full((M, pm.K), float("nan"), dtype=torch.float32, device=DEV)
+    d = pm.desc()
+    L = _lib.lib()
+
+    def call(stream):
+        return L.cbk_gemm_static(ctypes.byref(d), x.data_ptr(), F.dtype_code(x.dtype), M, x.stride(0), y.data_ptr(),
+                                 F.F32, pm.K, None, stream)
+
+    st = torch.cuda.Stream()
+    st.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(st):
+        assert call(st.cuda_stream) == 0                       # eager: address lookup, kernel attributes
+        st.synchronize()
+        assert torch.equal(y, want)
+        before = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved())
+        assert call(st.cuda_stream) == 0
+        st.synchronize()
+        assert (torch.cuda.memory_allocated(), torch.cuda.memory_reserved()) == before
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=st):
+            assert call(st.cuda_stream) == 0
+        for _ in range(3):                                     # every replay against the eager result
+            y.fill_(float("nan"))
+            st.synchronize()
+            graph.replay()
+            st.synchronize()
+            assert torch.equal(y, want)
+    torch.cuda.current_stream().wait_stream(st)
 
 
 def test_static_scratch_refuses_what_does_not_fit():
