@@ -270,6 +270,7 @@ def per_matrix(torch, F, L, dev, shapes, layout, bits, group, keep, M, dt, iters
         rows.append({"matrix": f"{name} {K}x{N}", "bytes": nbytes, "distinct_copies": copies, "launches_timed": reps * copies,
                      "hip_graph": use_graph, "us": round(us, 2), "gbs": round(nbytes / us / 1e3, 1),
                      "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
+        print(f"per_matrix {name} {K}x{N}: {us:.2f} us", file=sys.stderr, flush=True)
         del pms, args, g, x, y, w
         torch.cuda.empty_cache()
     return rows
@@ -585,6 +586,16 @@ def measured_ceilings(torch, dev):
                    "grid-stride 16-byte reads of 1 GiB, eight in flight per lane, best of three grid sizes"}
 
 
+def copy_calibration(torch, dev):
+    """A 1 GiB device-to-device copy: the known reading the HBM traffic counters are scaled by."""
+    src = torch.empty(2**30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+
+
 def cpu_model():
     try:
         for line in open("/proc/cpuinfo"):
@@ -810,6 +821,8 @@ def main():
             rows = [dict(layout=F.LAYOUT_NAME[lay], **per_matrix(torch, F, L, dev, gate, lay, b, 128, None, M, dt, tiled=False,
                                                                  use_graph=not a.no_graph)[0])
                     for lay, b in ((F.SPARSE4X, 4), (F.DENSE8, 8))]
+        if a.copy_calibration:
+            copy_calibration(torch, dev)
         print(json.dumps({"leg": a.only, "workload": a.workload, "M": M, "rows": rows}))
         return
 
@@ -818,12 +831,7 @@ def main():
     bpw = sets[0][0].bpw()
     res, xs, y_first = decode_layer_sets(torch, F, L, dev, shapes, sets, M, dt, a.launch, a.steps, a.warmup, not a.no_graph)
     if a.copy_calibration:
-        src = torch.empty(2**30, dtype=torch.uint8, device=dev)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+        copy_calibration(torch, dev)
     del sets
     torch.cuda.empty_cache()
 

@@ -181,8 +181,14 @@ __device__ inline void stage_convert(const XLoad& r, bool has_cs, int xdt, int N
   mx = fmaxf(mx, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, mx), 0xB1, 0xF, 0xF, true)));
   mx = fmaxf(mx, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, mx), 0x4E, 0xF, 0xF, true)));
   mx = fmaxf(mx, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, mx), 0x141, 0xF, 0xF, true)));
-  const float d = mx > 0.f ? mx / 8323072.f : 1.f;
-  const float inv = 1.f / d;
+  // delta = max|x'| / 8323072 (= 127 * 65536: 24 signed bits) by a multiplication, its reciprocal by the
+  // hardware approximation and one Newton step; two divisions were a tenth of this function.
+  // (24 bits, not 23 with a cheaper rounding: activations of 1e4 at the pruned columns of a chunk,
+  // the reference's own probe, leave the ordinary ones 10 bits less, and the result must still
+  // meet the layer tolerance.)
+  const float d = mx > 1e-30f ? mx * (1.f / 8323072.f) : 1.f;
+  float inv = __builtin_amdgcn_rcpf(d);
+  inv = inv * fmaf(-d, inv, 2.f);
   // X + 0x808080 has the bytes d0 + 128, d1 + 128, d2 + 128 of the balanced base-256 digits
   // (X = d0 + 256 d1 + 65536 d2, -128 <= d < 128), so the digits of four columns are byte
   // permutes of the four biased integers and one xor per digit plane
@@ -191,7 +197,7 @@ __device__ inline void stage_convert(const XLoad& r, bool has_cs, int xdt, int N
 #pragma unroll
   for (int bi = 0; bi < 16; ++bi) {
     const float v = ORDER == 0 ? xv[bi] : ORDER == 1 ? xv[frag_col(4, true, bi)] : xv[frag_col(2, true, bi)];
-    xb[bi] = (uint32_t)((int)rintf(v * inv) + 0x808080);          // |X| <= 127 * 65536
+    xb[bi] = (uint32_t)((int)rintf(v * inv) + 0x808080);          // |X| <= 127 * 65536 (+ 2 from the rounding of inv)
   }
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
@@ -1378,22 +1384,35 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
     g.spi = (g.nS + g.sk - 1) / g.sk;                  // equal parts
     g.sk = (g.nS + g.spi - 1) / g.spi;
     sk_cap = sk_cap > g.sk ? sk_cap : g.sk;
-    // column slabs: as many whole parts as the digit budget holds (a part is at most 8 steps =
-    // 4096 columns, 12 KB per activation row, so one part of eight rows always fits)
+  }
+  // LDS: selector table, zero row and counters, the deltas, the reduction slots, and the activation
+  // digits, which get what the others leave: at least four reduction slots are kept back (up to 24 KB
+  // of them where there is room), so that eight rows of 5376 columns (126 KB of digits) are still
+  // staged whole.  Rows whose digits do not fit are staged in column slabs: as many whole parts as the
+  // budget holds (a part is at most 8 steps = 4096 columns, 12 KB per activation row, so one part of
+  // eight rows always fits).
+  const size_t slot_bytes = (size_t)sk_cap * M * 16 * 4;
+  const size_t fixed = (size_t)LUT_BYTES + ZERO_BYTES + CNT_BYTES + (size_t)delta_cap * 4;
+  const size_t red_floor = 4 * slot_bytes < 24 * 1024 ? 4 * slot_bytes : 24 * 1024;
+  const size_t x_budget = M == 1 ? (size_t)X_LDS_BUDGET : 160 * 1024 - fixed - red_floor;
+  for (int i = 0; i < n; ++i) {
+    GvMat& g = gb.mat[i];
     const int N = g.m.N;
     g.sp = g.sk;
-    if ((size_t)M * NDIG * N > (size_t)X_LDS_BUDGET) {
-      g.sp = X_LDS_BUDGET / (M * NDIG * g.spi * 512);
+    if ((size_t)M * NDIG * N > x_budget) {
+      g.sp = (int)(x_budget / ((size_t)M * NDIG * g.spi * 512));
       if (g.sp < 1 || M == 1) return CBK_ERR_UNSUPPORTED;         // (the one-row kernels stage whole rows only)
     }
     const int slab_cols = g.sp >= g.sk ? N : g.sp * g.spi * 512;
     xq_cap = xq_cap > M * NDIG * slab_cols ? xq_cap : M * NDIG * slab_cols;
   }
   gb.h.xq_cap = xq_cap; gb.h.delta_cap = delta_cap;
-  // reduction slots: as many as fit 24 KB, a power of two between 2 and 64
+  // reduction slots: as many as fit what is left, at most 24 KB: a power of two between 2 and 64
   const int slot_floats = sk_cap * M * 16;
+  size_t red_room = 160 * 1024 - fixed - (size_t)xq_cap;
+  red_room = red_room < 24 * 1024 ? red_room : 24 * 1024;
   int nslot = 64;
-  while (nslot > 2 && (size_t)nslot * slot_floats * 4 > 24 * 1024) nslot >>= 1;
+  while (nslot > 2 && (size_t)nslot * slot_bytes > red_room) nslot >>= 1;
   gb.h.sk_cap = sk_cap; gb.h.nslot = nslot; gb.h.red_floats = nslot * slot_floats;
   gb.h.cq = cost / blocks; gb.h.cr = cost % blocks;
   const size_t lds = (size_t)LUT_BYTES + ZERO_BYTES + CNT_BYTES + xq_cap + (size_t)delta_cap * 4 +

@@ -166,6 +166,10 @@ def test_gemv_every_kernel_configuration(case, tiled):
 
 
 def test_gemv_batch_matches_single_calls():
+    """A batched launch against one call per matrix.  How a row is cut into parts depends on the
+    launch as a whole (its tiles against the 256 workgroups), so the two agree to float32 rounding
+    of the partial sums, not to the bit; each of them is run-to-run identical, and inside one
+    grouping a row's result does not depend on M (the tests further down)."""
     case = (F.BLK1632_4, 4, 128, 16)
     shapes = [(4096, 4096), (1024, 4096), (1024, 4096), (512, 14336)]
     pms = [F.synth_packed(K, N, *case[:3], case[3], seed=i, device=DEV).to_tiled() for i, (K, N) in enumerate(shapes)]
@@ -173,13 +177,16 @@ def test_gemv_batch_matches_single_calls():
         xs = [acts(M, N, torch.float16, seed=N + i).to(DEV) for i, (K, N) in enumerate(shapes)]
         bs = [torch.randn(K, device=DEV).half() for K, N in shapes]
         ys = ops.gemv_batch(pms, xs, biases=bs, out_dtype=torch.float32)
-        for pm, x, b, y in zip(pms, xs, bs, ys):
-            assert torch.equal(y, ops.gemv(pm, x, bias=b, out_dtype=torch.float32))
+        again = ops.gemv_batch(pms, xs, biases=bs, out_dtype=torch.float32)
+        for pm, x, b, y, y2 in zip(pms, xs, bs, ys, again):
+            single = ops.gemv(pm, x, bias=b, out_dtype=torch.float32)
+            assert float((y - single).abs().max() / single.abs().max()) < 1e-6
+            assert torch.equal(y, y2)
     # a mixed batch (different code widths) degrades to single calls and still agrees
     pm3 = F.synth_packed(256, 4096, F.BLKC, 3, 128, 10, seed=5, device=DEV)
     xs = [acts(2, 4096, torch.bfloat16, seed=1).to(DEV)] * 2
     ys = ops.gemv_batch([pms[0], pm3], xs, out_dtype=torch.float32)
-    assert torch.equal(ys[0], ops.gemv(pms[0], xs[0], out_dtype=torch.float32))
+    assert torch.equal(ys[0], ops.gemv(pms[0], xs[0], out_dtype=torch.float32))     # (the same launches either way)
     assert torch.equal(ys[1], ops.gemv(pm3, xs[1], out_dtype=torch.float32))
 
 
@@ -453,6 +460,49 @@ def test_linear_act_gated_epilogue(case, act):
            else torch.nn.functional.silu(t[:, 0::2])) * t[:, 1::2]
     one = ops.linear_act(pm, x, act, out_dtype=torch.float32)
     assert rel_fro(_np(one), _np(two)) < 1e-6
+
+
+@pytest.mark.parametrize("act", ["gelu_tanh", "silu"])
+def test_linear_act_for_nine_to_128_rows(act):
+    """Between 9 and 128 activation rows (the 64- and 128-token tiles of the matrix kernel, a float32
+    intermediate and one rounding of the result).  Row counts on and off the tile sizes, more than
+    one row tile with a ragged last one (K = 2 * 331), with and without bias, every output type,
+    both byte orders, and a y with a leading dimension beyond K / 2; against the oracle's float64
+    gate/up product."""
+    for case in (FUSED_CASES[0], (F.BLKC, 3, 64, 10), (F.DENSE4, 4, 128, 0)):
+        K, N = 662, 1152
+        for tiled in (False, True):
+            pm, W = _fused(case, K, N, 2, (0, 0), seed=K + 9, tiled=tiled)
+            bias = acts(1, K, torch.float32, seed=13)[0]
+            for M, dtype, odt, with_bias in ((9, torch.float16, torch.float32, True), (40, torch.bfloat16, torch.bfloat16, False),
+                                             (64, torch.float16, torch.float16, True), (65, torch.bfloat16, torch.float32, False),
+                                             (128, torch.float16, torch.float32, True)):
+                x = acts(M, N, dtype, seed=M + 2)
+                b = bias.to(odt) if with_bias else None
+                t = R.forward_ref(W, _np(x))
+                if with_bias:
+                    t = t + _np(b)[None, :]
+                ref = _gated_ref(t, act)
+                y = ops.linear_act(pm, x.to(DEV), act, bias=None if b is None else b.to(DEV), out_dtype=odt)
+                assert y.shape == (M, K // 2) and y.dtype == odt
+                err = rel_fro(_np(y), ref)
+                tol = 4e-3 if odt == torch.bfloat16 else TOL
+                assert err < tol, f"{case_id(case)} {act} tiled={tiled} M={M} {dtype}->{odt}: {err}"
+                assert torch.equal(ops.linear_act(pm, x.to(DEV), act, bias=None if b is None else b.to(DEV), out_dtype=odt), y)
+    # through the C ABI into a y with a leading dimension larger than K / 2: the columns beyond stay untouched
+    pm, W = _fused(FUSED_CASES[0], 256, 512, 2, (0, 0), seed=3, tiled=True)
+    M, ldy = 20, 136
+    x = acts(M, 512, torch.float16, seed=5).to(DEV)
+    y = torch.full((M, ldy), -7.0, dtype=torch.float32, device=DEV)
+    L, d = _lib.lib(), pm.desc()
+    need = L.cbk_linear_act_workspace_bytes(ctypes.byref(d), M, F.F32)
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+    rc = L.cbk_linear_act(ctypes.byref(d), x.data_ptr(), F.F16, M, 512, y.data_ptr(), F.F32, ldy, None,
+                          _lib.ACT_CODE[act], ws.data_ptr(), need, None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    ref = _gated_ref(R.forward_ref(W, _np(x)), act)
+    assert rel_fro(_np(y[:, :128]), ref) < TOL and bool((y[:, 128:] == -7.0).all())
 
 
 def test_linear_act_rejects_bad_calls():
