@@ -28,15 +28,27 @@ phases of the step.
 in TFLOP/s against the 2.5 PFLOP/s dense bf16/f16 MFMA peak, and checks sampled output rows of
 the timed configuration against a float64 matmul with the bit-exact dequantised weights.
 
-`--grid` runs the nine-cell sweep instead (Gemma-3-27B shapes x 62 layers, sparsity 0.3/0.5/0.7
-as 23/16/10 survivors per 32 columns, 2/3/4-bit codes, group 64): per-token linear time of a
-decode step (M=1) and of a 4096-token prefill, and bits per weight, per cell.
+The other benchmark configurations ride in the same JSON line unless `--no-configs` is given:
+`config0_single_layer` (one Mistral-7B MLP up-projection, M=1 and a 256-token prefill, checked
+against the C oracle), `config1_mistral7b_m4/_m8` and `config3_gemma27b_m4/_m8` (the decode step
+at four and eight activation rows), `config2_mistral7b_b3_keep10` (3-bit codes, 10 survivors per
+32 columns, group 64: decode step and MLP prefill) and `config4_grid`, the nine-cell sweep
+(Gemma-3-27B shapes x 62 layers, sparsity 0.3/0.5/0.7 as 23/16/10 survivors per 32 columns,
+2/3/4-bit codes, group 64): per-token linear time of a decode step (M=1) and of a 4096-token
+prefill, and bits per weight, per cell.  `--grid` runs that sweep alone, at more repetitions.
 
 `cpu_baseline` is the torch restatement of the reference's CPU forward (dequantise the packed
 bytes to float32, then matmul: oracle/torch_ref.py) on the host cores, on the same packed bytes
-as the first layer set; the C oracle checks the GPU outputs of that set.
+as the first layer set: the median of five passes over as many matrices of the set as fit the
+time budget, and a 256-token prefill leg on the MLP shapes extrapolated linearly in M to the
+2048 tokens the GPU leg runs; the C oracle checks the GPU outputs of that set.
 
-python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemma27b|mistral7b] [--m M] [--grid]
+`--only per-matrix|row-kernels` runs one leg with host launches or graphs (`--no-graph`) and
+prints a progress line per matrix on stderr: the form a counter-collecting profiler run takes,
+with the profiler's kernel filter set to this library's kernels.
+
+python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemma27b|mistral7b] [--m M]
+                [--grid] [--no-configs] [--only LEG] [--no-graph] [--copy-calibration]
 """
 import argparse
 import ctypes
