@@ -248,7 +248,7 @@ size_t cbk_workspace_bytes(const cbk_desc* in, int M) {
     return t.end + gemm_big_workspace(dense4_view(m, nullptr, t), M);
   }
   // the most any of the three entry points asks for (cbk_gemm runs the prefill kernel at any M)
-  size_t need = (M >= 1 && M <= 16 && gemv_fast_takes(m, 1)) ? gemv_fast_workspace(m, 1) : 0;
+  size_t need = (M >= 1 && M <= 16 && gemv_fast_takes(m, 1)) ? gemv_fast_workspace(m, M) : 0;
   if (gemm_big_takes(m, M)) {
     const size_t b = gemm_big_workspace(m, M);
     return need > b ? need : b;

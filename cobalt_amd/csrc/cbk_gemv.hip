@@ -57,6 +57,11 @@ constexpr int CNT_BYTES = CNT_SLOTS * 4;       // at a fixed place: zeroed befor
 constexpr int X_LDS_BUDGET = 112 * 1024;      // activation digits of one column slab: M * 3 * columns bytes (of 160 KB LDS)
 constexpr int DELTA_LDS_BUDGET = 6 * 1024;    // one float per 128-column chunk and activation row
 constexpr int NDIG = 3;                       // int8 digits per activation
+// The digit rows of the matrix-core kernels lie X_PAD bytes further apart than their length.  The
+// sixteen lanes of a quarter read sixteen bytes each from up to twelve different rows (activation
+// row, digit) at the same column; row lengths are multiples of 128 bytes, and unpadded rows would
+// all start in the same LDS banks.
+constexpr int X_PAD = 16;
 constexpr int GV_MAX_M = 8;                     // 5..8 only in the block-per-quarter arrangement
 constexpr int GV_MAX_BATCH = 8;               // matrices per launch
 
@@ -151,12 +156,12 @@ __device__ inline void stage_load(const uint16_t* x, int64_t ldx, const uint16_t
 
 // conversion of one loaded item into digits and delta in LDS; the eight consecutive lanes of a
 // chunk are always active together (the item count is a multiple of 8)
-// (digits at row stride Ns = 16 * n16 bytes, deltas at the chunk's index in the whole row: ch0 is
+// (digits at row stride Ns = 16 * n16 + pad bytes, deltas at the chunk's index in the whole row: ch0 is
 // the slab's first chunk)
 template <int ORDER>
 __device__ inline void stage_convert(const XLoad& r, bool has_cs, int xdt, int N, int ch0, int n16, int it, bool one_row,
-                                     int8_t* xq, float* delta) {
-  const int NCH = N >> 7, Ns = n16 * 16;
+                                     int8_t* xq, float* delta, int pad = 0) {
+  const int NCH = N >> 7, Ns = n16 * 16 + pad;
   const int row = one_row ? 0 : it / n16, c16 = it - row * n16;
   const uint32_t* xw = (const uint32_t*)r.x;
   const uint32_t* cw = (const uint32_t*)r.c;
@@ -550,12 +555,12 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     if (!first) __syncthreads();                                  // previous matrix fully consumed
     first = false;
     constexpr int XORD = !C::DENSE ? 0 : (BITS == 2 ? 2 : 1);
-    if (xit < xitems) stage_convert<XORD>(xl, m.cs != nullptr, h.xdt, N, ch0, n16, xit, MP == 1, xq, delta);
+    if (xit < xitems) stage_convert<XORD>(xl, m.cs != nullptr, h.xdt, N, ch0, n16, xit, MP == 1, xq, delta, X_PAD);
     if (PRE2 && xit + GV_THREADS < xitems)
-      stage_convert<XORD>(xl2, m.cs != nullptr, h.xdt, N, ch0, n16, xit + GV_THREADS, MP == 1, xq, delta);
+      stage_convert<XORD>(xl2, m.cs != nullptr, h.xdt, N, ch0, n16, xit + GV_THREADS, MP == 1, xq, delta, X_PAD);
     for (xit += (PRE2 ? 2 : 1) * GV_THREADS; xit < xitems; xit += GV_THREADS) {
       stage_load(gm.x, gm.ldx, m.cs, N, col0, n16, xit, MP == 1, gm.par, xl);
-      stage_convert<XORD>(xl, m.cs != nullptr, h.xdt, N, ch0, n16, xit, MP == 1, xq, delta);
+      stage_convert<XORD>(xl, m.cs != nullptr, h.xdt, N, ch0, n16, xit, MP == 1, xq, delta, X_PAD);
     }
     __syncthreads();
 
@@ -587,7 +592,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 #pragma unroll
         for (int g = 0; g < NG; ++g) {
           a_on[g] = a_dig < NDIG && a_m + 4 * g < h.M;
-          a_base[g] = xq_off + (uint32_t)(((a_m + 4 * g) * NDIG + a_dig) * Ns + kq * 32);
+          a_base[g] = xq_off + (uint32_t)(((a_m + 4 * g) * NDIG + a_dig) * (Ns + X_PAD) + kq * 32);
           dm[g] = kq + 4 * g < h.M ? kq + 4 * g : 0;
         }
 #pragma unroll
@@ -636,7 +641,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 #pragma unroll
         for (int p = 0; p < MP; ++p) {
           const bool on = valid && a_slice == kq && a_dig < NDIG && p < h.M;
-          aaddr[p] = on ? xq_off + (uint32_t)((p * NDIG + a_dig) * Ns + (chunk - ch0) * 128) : z_off;
+          aaddr[p] = on ? xq_off + (uint32_t)((p * NDIG + a_dig) * (Ns + X_PAD) + (chunk - ch0) * 128) : z_off;
         }
         // ---- bring the chunk's first code bit to bit 0 of cw[0]
         uint32_t cw[C::ND];
@@ -789,6 +794,241 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       ++mi;
     }
   }
+}
+
+// ------------------------------------------------------------------ long rows, split over the workgroups by columns
+// Rows whose digits do not fit in LDS (M * 3 * N bytes: `down` projections at M >= 4).  The
+// kernel above stages such a row slab after slab in every workgroup, every workgroup converting
+// all M x N activations, with a handful of items per slab for its sixteen wavefronts.  Here a
+// workgroup owns one column slab (whole parts of the row, the parts of one activation row) of a
+// range of tiles: it stages M x (slab) activations once, deals the (tile, part) items of its slab
+// to the wavefronts and writes the part sums to a caller-provided buffer; a second small kernel
+// adds the parts of every output in part order.  Same operations in the same order as for one
+// activation row, so a row's result still does not depend on M.  Block-per-quarter arrangement only.
+struct GsArgs {
+  GvMat g;                 // spi, sk: the parts; sp: parts per slab
+  int M, xdt, ydt;
+  int xq_cap, delta_cap;   // LDS bytes of digits, floats of delta
+  int nslab, wps;          // column slabs, workgroups per slab
+  float* part;             // [ntiles][sk][M][16] part sums
+};
+
+template <int BITS, int KEEP, int GRP, int MP>
+__global__ __launch_bounds__(GV_THREADS) void gemv_split_kernel(GsArgs a) {
+  using C = Cfg<BITS, KEEP, GRP, MP>;
+  static_assert((MP == 4 || MP == 8) && block_split_capable(BITS, KEEP, GRP), "block-per-quarter configurations only");
+  constexpr int NG = MP / 4;                           // groups of four activation rows, one MFMA each per fragment
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  uint2* lut = (uint2*)smem;
+  uint8_t* zreg = smem + LUT_BYTES;
+  int8_t* xq = (int8_t*)zreg + ZERO_BYTES;
+  float* delta = (float*)(xq + a.xq_cap);
+  const GvMat& gm = a.g;
+  const DMat& m = gm.m;
+  const int M = a.M, N = m.N, NCH = N >> 7, nS = gm.nS, spi = gm.spi, SK = gm.sk;
+  if (tid < 256) {
+    const uint2 e = make_selectors((uint32_t)tid, C::SEL_KIND);
+#pragma unroll
+    for (int j = 0; j < LUT_LANES; ++j) lut[tid * LUT_LANES + j] = e;
+  } else if (tid < 256 + ZERO_BYTES / 4) {
+    ((uint32_t*)zreg)[tid - 256] = 0u;
+  } else if (tid < 256 + ZERO_BYTES / 4 + 4 * M) {                  // deltas of the chunks past N
+    const int i = tid - 256 - ZERO_BYTES / 4;
+    delta[(i >> 2) * (NCH + 4) + NCH + (i & 3)] = 0.f;
+  }
+  const int wr = lane & 15, kq = lane >> 4;
+  const uint32_t l16 = lane & (LUT_LANES - 1);
+  const int a_m = wr >> 2, a_dig = wr & 3;             // activation row and digit of this lane's A row
+  const uint32_t xq_off = (uint32_t)((uint8_t*)xq - smem), z_off = (uint32_t)(zreg - smem);
+
+  // this workgroup: slab sl, tiles [T_lo, T_hi)
+  const int bx = (int)blockIdx.x;
+  const int sl = bx / a.wps, wi = bx - sl * a.wps;
+  const int tq = gm.ntiles / a.wps, tr = gm.ntiles % a.wps;
+  const int T_lo = wi * tq + (wi < tr ? wi : tr), T_hi = T_lo + tq + (wi < tr ? 1 : 0);
+  const int ntl = T_hi - T_lo;
+  if (ntl <= 0) return;                                             // uniform over the workgroup
+  const int pa = sl * gm.sp, pn = SK - pa < gm.sp ? SK - pa : gm.sp;        // its parts
+  const int S0 = pa * spi, S1 = (pa + pn) * spi < nS ? (pa + pn) * spi : nS;
+  const int col0 = S0 * 512, Ns = N - col0 < (S1 - S0) * 512 ? N - col0 : (S1 - S0) * 512, ch0 = col0 >> 7;
+
+  const uint8_t* const m_data = m.data;
+  const uint16_t* const m_scale = m.scale;
+  const uint8_t* const m_zero = m.zero;
+  const int m_K = m.K, m_G = m.G, ush = gm.ush, csh = gm.csh;
+  const uint32_t tile_a = gm.tile_a, lane_mul = gm.lane_mul, sz_mul = gm.sz_mul, code_u0 = m.code_off >> 4;
+  const int last_S = nS - 1, last_tile = T_hi - 1;
+
+  // loads of one (tile, macro-step) position: block kq of the chunks 4S .. 4S+3 of row wr
+  auto issue = [&](int tile, int S, Loads<C>& L) {
+    tile = tile < last_tile ? tile : last_tile;
+    S = S < last_S ? S : last_S;
+    const int S4 = 4 * S;
+    const int rlim = m_K - 1 - tile * 16;                           // rows past K repeat row K - 1
+    const uint32_t wrc = (uint32_t)(wr < rlim ? wr : rlim);
+    const uint32_t lane_off = __umul24(wrc, lane_mul);
+    const int klim = NCH - 1 - S4;                                  // chunks past N repeat chunk NCH - 1
+    const uint32_t chl = (uint32_t)(kq < klim ? kq : klim);
+    const uint32_t so_t = (uint32_t)tile * tile_a;
+    const uint32_t so_g = (uint32_t)tile * (uint32_t)(16 * m_G);
+    constexpr uint32_t BB = C::CB / 8;
+    const uint32_t voff_m = lane_off + (uint32_t)kq * 4u;
+    const uint32_t voff_c = lane_off + ((((uint32_t)kq * BB) >> 4) << ush) + (((uint32_t)kq * BB) & 15u);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      int chc = S4 + c;
+      chc = chc < NCH ? chc : NCH - 1;
+      if (!C::DENSE) L.mk[c] = *(const uint32_t*)(m_data + (so_t + ((uint32_t)chc << ush) + voff_m));
+      const uint8_t* cp = m_data + (so_t + ((code_u0 + (uint32_t)chc * (C::CHB / 128)) << ush) + voff_c);
+      if (C::CB == 32) {
+        L.raw[c] = *(const uint32_t*)cp;
+      } else if (C::CB == 64) {
+        const uint2 v = *(const uint2*)cp;
+        L.raw[2 * c] = v.x; L.raw[2 * c + 1] = v.y;
+      } else {
+        const uint4 v = *(const uint4*)cp;
+        L.raw[4 * c] = v.x; L.raw[4 * c + 1] = v.y; L.raw[4 * c + 2] = v.z; L.raw[4 * c + 3] = v.w;
+      }
+    }
+    const uint32_t gv = so_g + ((uint32_t)S4 << csh) + __umul24(wrc, sz_mul) + (chl << csh);
+    L.zraw = (uint32_t)m_zero[gv] | ((uint32_t)m_scale[gv] << 8);
+  };
+
+  // this wave's (tile, part, macro-step) positions: items wave, wave + 16, ... of the slab
+  struct Pos { int tl, part, S; };
+  const int dq_t = GV_WAVES / pn, dq_p = GV_WAVES % pn;
+  auto advance = [&](Pos& p) -> bool {                             // false past the last position
+    const int s_end = (p.part * spi + spi < nS) ? p.part * spi + spi : nS;
+    if (p.S + 1 < s_end) { ++p.S; return true; }
+    p.tl += dq_t; p.part += dq_p;
+    if (p.part >= pa + pn) { p.part -= pn; ++p.tl; }
+    p.S = p.part * spi;
+    return p.tl < ntl;
+  };
+  Pos p0{wave / pn, pa + wave % pn, (pa + wave % pn) * spi};
+  bool v0 = p0.tl < ntl;
+  Pos p1 = p0; bool v1 = v0 && advance(p1);
+
+  // ---- stage the slab's digits (the activation loads go out before the first weight loads)
+  constexpr int XORD = !C::DENSE ? 0 : (BITS == 2 ? 2 : 1);
+  const int n16 = Ns >> 4, xitems = M * n16;                        // a multiple of 8
+  XLoad xl;
+  if (tid < xitems) stage_load(gm.x, gm.ldx, m.cs, N, col0, n16, tid, false, gm.par, xl);
+  Loads<C> LA, LB;
+  issue(T_lo + p0.tl, p0.S, LA);
+  if (tid < xitems) stage_convert<XORD>(xl, m.cs != nullptr, a.xdt, N, ch0, n16, tid, false, xq, delta, X_PAD);
+  for (int xit = tid + GV_THREADS; xit < xitems; xit += GV_THREADS) {
+    stage_load(gm.x, gm.ldx, m.cs, N, col0, n16, xit, false, gm.par, xl);
+    stage_convert<XORD>(xl, m.cs != nullptr, a.xdt, N, ch0, n16, xit, false, xq, delta, X_PAD);
+  }
+  __syncthreads();
+
+  float ysum[MP];
+  auto do_step = [&](Loads<C>& cur, Loads<C>& tgt) {               // decode `cur`, load the next step into `tgt`
+    const int tl = p0.tl, part = p0.part, S = p0.S;
+    const int tile = T_lo + tl;
+    const int s_end = (part * spi + spi < nS) ? part * spi + spi : nS;
+    if (S == part * spi) {
+#pragma unroll
+      for (int p = 0; p < MP; ++p) ysum[p] = 0.f;
+    }
+    issue(T_lo + p1.tl, p1.S, tgt);
+    uint32_t zs[4];                                                 // zero | scale << 8 of the groups 4S .. 4S+3
+#pragma unroll
+    for (int c = 0; c < 4; ++c) zs[c] = (uint32_t)__shfl((int)cur.zraw, wr + 16 * c, 64);
+    bool a_on[NG];
+    uint32_t a_base[NG];
+    int dm[NG];                                                     // the activation rows this quarter sums
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      a_on[g] = a_dig < NDIG && a_m + 4 * g < M;
+      a_base[g] = xq_off + (uint32_t)(((a_m + 4 * g) * NDIG + a_dig) * (Ns + X_PAD) + kq * 32);
+      dm[g] = kq + 4 * g < M ? kq + 4 * g : 0;
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int chunk = 4 * S + c;
+      uint32_t aaddr[NG];
+#pragma unroll
+      for (int g = 0; g < NG; ++g) aaddr[g] = (a_on[g] && chunk < NCH) ? a_base[g] + (uint32_t)(chunk - ch0) * 128u : z_off;
+      uint32_t rkc[4];
+      uint2 selc[4];
+      fetch_selectors<C>(cur.mk[c], lut, l16, rkc, selc);
+      uint32_t st[C::NW];
+#pragma unroll
+      for (int k = 0; k < C::NW; ++k) st[k] = cur.raw[c * C::NW + k];
+      const uint32_t z = zs[c] & 0xFFu;
+      const uint32_t nz = 0x80808080u - z * 0x01010101u;
+      v4i acc[NG];
+#pragma unroll
+      for (int g = 0; g < NG; ++g) acc[g] = (v4i){0, 0, 0, 0};
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        uint32_t bfrag[4];
+        decode_half<C, BITS>(st, rkc, selc, nz, half, bfrag);
+        const v4i bv = (v4i){(int)bfrag[0], (int)bfrag[1], (int)bfrag[2], (int)bfrag[3]};
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+          const v4i av = *(const v4i*)(smem + aaddr[g] + 16 * half);
+          acc[g] = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bv, acc[g], 0, 0, 0);
+          asm("s_nop 1" : "+v"(acc[g]));                            // see the main kernel
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const float dl = delta[dm[g] * (NCH + 4) + chunk];          // 0 past the last chunk
+        const float f = fmaf((float)(acc[g][0] * 256 + acc[g][1]), 256.f, (float)acc[g][2]);
+        ysum[4 * g + c] = fmaf(f, h2f((uint16_t)(zs[c] >> 8)) * dl, ysum[4 * g + c]);
+      }
+    }
+    if (S + 1 == s_end) {
+      // the part is done: lane quarter kq holds activation row 4g + kq of weight row wr
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const float ps = (ysum[4 * g] + ysum[4 * g + 1]) + (ysum[4 * g + 2] + ysum[4 * g + 3]);
+        if (kq + 4 * g < M) a.part[((size_t)(tile * SK + part) * M + kq + 4 * g) * 16 + wr] = ps;
+      }
+    }
+    p0 = p1; v0 = v1;
+    if (v1) v1 = advance(p1);
+  };
+  while (true) {
+    if (!v0) break;
+    do_step(LA, LB);
+    if (!v0) break;
+    do_step(LB, LA);
+  }
+}
+
+// the parts of every output, added in part order; bias; conversion
+constexpr int GS_RED_THREADS = 64;
+__global__ __launch_bounds__(GS_RED_THREADS) void gemv_split_reduce_kernel(GsArgs a) {
+  const GvMat& gm = a.g;
+  const int M = a.M, SK = gm.sk;
+  const int idx = (int)blockIdx.x * GS_RED_THREADS + (int)threadIdx.x;
+  const int wr = idx & 15, t = idx >> 4, tile = t / M, am = t - tile * M;
+  if (tile >= gm.ntiles) return;
+  const int k = tile * 16 + wr;
+  if (k >= gm.m.K) return;
+  int om = am;
+  if (gm.par) {                                                     // the sum scaled for the other parity is dropped
+    if ((om ^ k) & 1) return;
+    om >>= 1;
+  }
+  float pv[16];                                                     // all loads first (at most 16 parts), then the sum in part order
+#pragma unroll
+  for (int j = 0; j < 16; ++j) pv[j] = a.part[((size_t)(tile * SK + (j < SK ? j : SK - 1)) * M + am) * 16 + wr];
+  float v = 0.f;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) v += j < SK ? pv[j] : 0.f;
+  if (gm.bias) v += (a.ydt == CBK_F32) ? ((const float*)gm.bias)[k]
+                  : (a.ydt == CBK_F16) ? h2f(((const uint16_t*)gm.bias)[k]) : bf2f(((const uint16_t*)gm.bias)[k]);
+  const size_t o = (size_t)om * gm.ldy + k;
+  if (a.ydt == CBK_F32) ((float*)gm.y)[o] = v;
+  else if (a.ydt == CBK_F16) ((uint16_t*)gm.y)[o] = f2h(v);
+  else ((uint16_t*)gm.y)[o] = f2bf(v);
 }
 
 // ------------------------------------------------------------------ survivor-stream rows
@@ -1256,7 +1496,7 @@ bool gemv_fast_takes(const DMat& m, int M) {
   if ((uint64_t)((m.K + 15) / 16 * 16) * m.G * 2 >= (1ull << 32)) return false;
   // the digits are staged in column slabs where a whole row does not fit; the per-chunk deltas
   // of all rows stay in LDS for the whole matrix
-  if (M == 1) return (size_t)NDIG * m.N <= (size_t)X_LDS_BUDGET;   // (the one-row kernels stage whole rows only)
+  if (M == 1) return (size_t)NDIG * (m.N + X_PAD) <= (size_t)X_LDS_BUDGET;   // (the one-row kernels stage whole rows only)
   return (size_t)M * (m.N / 128 + 4) * 4 <= (size_t)DELTA_LDS_BUDGET;
 }
 
@@ -1265,7 +1505,23 @@ bool gemv_same_config(const DMat& a, const DMat& b) {
   return da == db && a.bits == b.bits && a.group == b.group && (da || a.keep == b.keep);
 }
 
-size_t gemv_fast_workspace(const DMat&, int) { return 0; }   // activations are staged in LDS
+// Rows whose digits are certainly staged whole need no workspace; longer ones (two to eight
+// activation rows of a block-per-quarter configuration) are split over the workgroups by columns
+// when the caller provides room for the part sums: [tiles][parts <= 16][M][16] floats.
+constexpr size_t SPLIT_MIN_BYTES = 100 * 1024;
+constexpr int SPLIT_MIN_STEPS = 16;           // rows of at least 8192 columns
+static inline int kernel_rows(const DMat& m, int M) {            // activation rows as the kernel counts them, per pass
+  const int v = m.cs_rows == 2 ? 2 : 1;
+  return M * v > GV_MAX_M ? GV_MAX_M : M * v;
+}
+static inline size_t split_part_bytes(int ntiles, int sk, int Mk) { return (size_t)ntiles * sk * Mk * 16 * 4; }
+
+size_t gemv_fast_workspace(const DMat& m, int M) {
+  const int Mk = kernel_rows(m, M);
+  if (Mk < 2 || !block_split_capable(m.bits, family_of(m.layout) == FAM_DENSE ? 0 : m.keep, m.group)) return 0;
+  if ((size_t)Mk * NDIG * (m.N + X_PAD) <= SPLIT_MIN_BYTES || (m.N / 128 + 3) / 4 < SPLIT_MIN_STEPS) return 0;
+  return up256(split_part_bytes((m.K + 15) / 16 + 3, 16, Mk));     // (+3: a q|k|v matrix is run as its three ranges)
+}
 
 struct GvCall {           // one matrix of a batched call, host side
   DMat m;
@@ -1322,69 +1578,97 @@ static int launch_keep(const GvBatch& b, size_t lds, int blocks, hipStream_t st)
   }
 }
 
-// All matrices share one kernel configuration (checked by the caller) and 1 <= M <= 8 (more than
-// four only where gemv_fast_takes says so).
-int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, void* workspace, size_t ws_bytes,
-                           hipStream_t st) {
-  if (n < 1 || n > GV_MAX_BATCH) return CBK_ERR_SHAPE;
-  GvBatch gb;
-  const int par = calls[0].par ? 1 : 0;
-  for (int i = 0; i < n; ++i)
-    if ((calls[i].par ? 1 : 0) != par || (calls[i].m.cs_rows == 2) != (par == 1)) return CBK_ERR_UNSUPPORTED;
-  M *= par + 1;                                                   // activation rows as the kernel counts them
-  if (M > GV_MAX_M) return CBK_ERR_SHAPE;
-  gb.h.n = n; gb.h.M = M; gb.h.xdt = xdt; gb.h.ydt = ydt;
-  int cost = 0, xq_cap = 0, delta_cap = 0, tiles = 0;
+// Workgroups of a launch of the main kernel.  A workgroup takes whole tiles.  Between one and two
+// tiles per workgroup the launch lasts two tiles however they are dealt, and dealing two to each
+// of fewer workgroups (384 tiles: 192 x 2 instead of 128 x 2 + 128 x 1) was measured faster as
+// long as at least three quarters of the CUs still get one (Mistral q,k,v: -1.9 us); with fewer
+// workgroups than that, or more tiles each, having every CU at work counts for more.  Only where
+// every tile costs the same.
+static int gemv_blocks(const GvBatch& gb, int n, int tiles) {
+  int blocks = tiles < 256 ? tiles : 256;                       // one persistent workgroup per CU
+  bool same = true;
+  for (int i = 1; i < n; ++i) same = same && gb.mat[i].nS == gb.mat[0].nS;
+  if (same && tiles > 256 && tiles <= 512 && (tiles + 1) / 2 >= 192) blocks = (tiles + 1) / 2;
+  return blocks;
+}
+
+template <int BITS, int KEEP, int GRP, int MP>
+static int launch_split_cfg(const GsArgs& a, size_t lds, hipStream_t st) {
+  if constexpr ((MP == 4 || MP == 8) && block_split_capable(BITS, KEEP, GRP)) {
+    auto kern = gemv_split_kernel<BITS, KEEP, GRP, MP>;
+    static std::atomic<int> configured{0};
+    if (!configured.load(std::memory_order_acquire)) {
+      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
+        return CBK_ERR_HIP;
+      configured.store(1, std::memory_order_release);
+    }
+    hipLaunchKernelGGL(kern, dim3(a.nslab * a.wps), dim3(GV_THREADS), lds, st, a);
+    if (hipGetLastError() != hipSuccess) return CBK_ERR_HIP;
+    hipLaunchKernelGGL(gemv_split_reduce_kernel, dim3((a.g.ntiles * a.M * 16 + GS_RED_THREADS - 1) / GS_RED_THREADS),
+                       dim3(GS_RED_THREADS), 0, st, a);
+    return hipGetLastError() == hipSuccess ? CBK_OK : CBK_ERR_HIP;
+  } else {
+    return CBK_ERR_UNSUPPORTED;
+  }
+}
+
+// One long-row matrix (spi and sk set) through gemv_split_kernel: parts per slab, workgroups per
+// slab, LDS.  `part` holds split_part_bytes(ntiles, sk, M).
+static int launch_split(const GvMat& g, int M, int xdt, int ydt, float* part, hipStream_t st) {
+  GsArgs a;
+  a.g = g; a.M = M; a.xdt = xdt; a.ydt = ydt; a.part = part;
+  a.delta_cap = M * (g.m.N / 128 + 4);
+  const size_t fixed = (size_t)LUT_BYTES + ZERO_BYTES + (size_t)a.delta_cap * 4 + (size_t)M * NDIG * X_PAD;
+  const size_t per_part = (size_t)M * NDIG * g.spi * 512;
+  if (fixed + per_part > 160 * 1024) return CBK_ERR_UNSUPPORTED;
+  int pps_max = (int)((160 * 1024 - fixed) / per_part);
+  pps_max = pps_max < g.sk ? pps_max : g.sk;
+  // Parts per slab: a workgroup runs ceil(items / 16) rounds of one part per wavefront after
+  // staging its slab (a 512-column step of M = 8 rows costs about 0.15 rounds of one step)
+  float best = 0.f;
+  int best_pps = 0;
+  for (int pps = 1; pps <= pps_max; ++pps) {
+    const int nslab = (g.sk + pps - 1) / pps;
+    int wps = 256 / nslab;
+    wps = wps < 1 ? 1 : (wps > g.ntiles ? g.ntiles : wps);
+    const int tpw = (g.ntiles + wps - 1) / wps;
+    const float c = (float)((tpw * pps + GV_WAVES - 1) / GV_WAVES * g.spi) + 0.15f * (float)M / 8.f * (float)(pps * g.spi);
+    if (best_pps == 0 || c < best) { best = c; best_pps = pps; }
+  }
+  a.g.sp = best_pps;
+  a.nslab = (g.sk + best_pps - 1) / best_pps;
+  a.wps = 256 / a.nslab;
+  a.wps = a.wps < 1 ? 1 : (a.wps > g.ntiles ? g.ntiles : a.wps);
+  const int cols = best_pps * g.spi * 512 < g.m.N ? best_pps * g.spi * 512 : g.m.N;
+  a.xq_cap = M * NDIG * (cols + X_PAD);
+  const size_t lds = (size_t)LUT_BYTES + ZERO_BYTES + a.xq_cap + (size_t)a.delta_cap * 4;
+  if (lds > 160 * 1024) return CBK_ERR_UNSUPPORTED;
+  const DMat& m = g.m;
+  const int keep = family_of(m.layout) == FAM_DENSE ? 0 : m.keep;
+  const bool big = M > 4;
+  if (m.group != 128) return CBK_ERR_UNSUPPORTED;
+  if (m.bits == 4 && keep == 16) return big ? launch_split_cfg<4, 16, 128, 8>(a, lds, st) : launch_split_cfg<4, 16, 128, 4>(a, lds, st);
+  if (m.bits == 4 && keep == 0) return big ? launch_split_cfg<4, 0, 128, 8>(a, lds, st) : launch_split_cfg<4, 0, 128, 4>(a, lds, st);
+  if (m.bits == 2 && keep == 16) return big ? launch_split_cfg<2, 16, 128, 8>(a, lds, st) : launch_split_cfg<2, 16, 128, 4>(a, lds, st);
+  if (m.bits == 2 && keep == 0) return big ? launch_split_cfg<2, 0, 128, 8>(a, lds, st) : launch_split_cfg<2, 0, 128, 4>(a, lds, st);
+  return CBK_ERR_UNSUPPORTED;
+}
+
+// Distribution over the workgroups, LDS and launch of the matrices of `gb` (spi and sk set).
+static int launch_main_batch(GvBatch& gb, hipStream_t st) {
+  const int n = gb.h.n, M = gb.h.M;
+  int cost = 0, tiles = 0, delta_cap = 0, sk_cap = 1, xq_cap = 0;
   for (int i = 0; i < n; ++i) {
-    const DMat& m = calls[i].m;
-    const bool dense = family_of(m.layout) == FAM_DENSE;
     GvMat& g = gb.mat[i];
-    g.m = m; g.x = (const uint16_t*)calls[i].x; g.ldx = calls[i].ldx;
-    g.order = !dense ? 0 : (m.bits == 2 ? 2 : 1);
-    g.par = par;
-    g.y = calls[i].y; g.bias = calls[i].bias; g.ldy = calls[i].ldy;
-    g.ntiles = (m.K + 15) / 16; g.nS = (m.N / 128 + 3) / 4; g.cost0 = cost;
-    g.tile_a = (uint32_t)m.stride * 16u;                          // sixteen rows in either order
-    g.lane_mul = m.tiled ? 16u : (uint32_t)m.stride;
-    g.sz_mul = m.tiled ? 1u : (uint32_t)m.G;
-    g.ush = m.tiled ? 8 : 4; g.csh = m.tiled ? 4 : 0;
+    g.cost0 = cost;
     cost += g.ntiles * g.nS;
     gb.h.cost_end[i] = cost;
     tiles += g.ntiles;
-    delta_cap = delta_cap > M * (m.N / 128 + 4) ? delta_cap : M * (m.N / 128 + 4);
-  }
-  (void)workspace; (void)ws_bytes;
-  for (int i = n; i < GV_MAX_BATCH; ++i) gb.h.cost_end[i] = cost;
-  int blocks = tiles < 256 ? tiles : 256;                       // one persistent workgroup per CU
-  // A workgroup takes whole tiles.  Between one and two tiles per workgroup the launch lasts two
-  // tiles however they are dealt, and dealing two to each of fewer workgroups (384 tiles: 192 x 2
-  // instead of 128 x 2 + 128 x 1) was measured faster as long as at least three quarters of the
-  // CUs still get one (Mistral q,k,v: -1.9 us); with fewer workgroups than that, or more tiles
-  // each, having every CU at work counts for more.  Only where every tile costs the same.
-  {
-    bool same = true;
-    for (int i = 1; i < n; ++i) same = same && gb.mat[i].nS == gb.mat[0].nS;
-    if (same && tiles > 256 && tiles <= 512 && (tiles + 1) / 2 >= 192) blocks = (tiles + 1) / 2;
-  }
-  // macro-steps per work item: about one and a half items per wavefront over the whole launch
-  // (the end of an item costs about as many instructions as a step; measured best between one
-  // and two); a tile is split into at most 16 parts, and into a power of two of them where the
-  // row is long enough: the items then spread evenly over the four SIMDs
-  int spi = (int)((long long)cost * 2 / ((long long)blocks * GV_WAVES * 3));
-  spi = spi < 1 ? 1 : (spi > 8 ? 8 : spi);
-  int sk_cap = 1;
-  for (int i = 0; i < n; ++i) {
-    GvMat& g = gb.mat[i];
-    int s = spi;
-    while ((g.nS + s - 1) / s > 16) ++s;
-    g.sk = (g.nS + s - 1) / s;
-    int p2 = 1;
-    while (p2 < g.sk) p2 <<= 1;
-    if (p2 <= 16 && p2 <= g.nS) g.sk = p2;
-    g.spi = (g.nS + g.sk - 1) / g.sk;                  // equal parts
-    g.sk = (g.nS + g.spi - 1) / g.spi;
+    delta_cap = delta_cap > M * (g.m.N / 128 + 4) ? delta_cap : M * (g.m.N / 128 + 4);
     sk_cap = sk_cap > g.sk ? sk_cap : g.sk;
   }
+  for (int i = n; i < GV_MAX_BATCH; ++i) gb.h.cost_end[i] = cost;
+  const int blocks = gemv_blocks(gb, n, tiles);
   // LDS: selector table, zero row and counters, the deltas, the reduction slots, and the activation
   // digits, which get what the others leave: at least four reduction slots are kept back (up to 24 KB
   // of them where there is room), so that eight rows of 5376 columns (126 KB of digits) are still
@@ -1399,12 +1683,12 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
     GvMat& g = gb.mat[i];
     const int N = g.m.N;
     g.sp = g.sk;
-    if ((size_t)M * NDIG * N > x_budget) {
-      g.sp = (int)(x_budget / ((size_t)M * NDIG * g.spi * 512));
+    if ((size_t)M * NDIG * (N + X_PAD) > x_budget) {
+      g.sp = (int)((x_budget - (size_t)M * NDIG * X_PAD) / ((size_t)M * NDIG * g.spi * 512));
       if (g.sp < 1 || M == 1) return CBK_ERR_UNSUPPORTED;         // (the one-row kernels stage whole rows only)
     }
     const int slab_cols = g.sp >= g.sk ? N : g.sp * g.spi * 512;
-    xq_cap = xq_cap > M * NDIG * slab_cols ? xq_cap : M * NDIG * slab_cols;
+    xq_cap = xq_cap > M * NDIG * (slab_cols + X_PAD) ? xq_cap : M * NDIG * (slab_cols + X_PAD);
   }
   gb.h.xq_cap = xq_cap; gb.h.delta_cap = delta_cap;
   // reduction slots: as many as fit what is left, at most 24 KB: a power of two between 2 and 64
@@ -1422,6 +1706,100 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
   if (bits == 6) return launch_mp<6, 16, 128>(gb, lds, blocks, st);   // BLK1632_6: one configuration
   return bits == 2 ? launch_keep<2>(gb, lds, blocks, st) : bits == 3 ? launch_keep<3>(gb, lds, blocks, st)
        : bits == 4 ? launch_keep<4>(gb, lds, blocks, st) : CBK_ERR_UNSUPPORTED;
+}
+
+// All matrices share one kernel configuration (checked by the caller) and 1 <= M <= 8 (more than
+// four only where gemv_fast_takes says so).
+int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, void* workspace, size_t ws_bytes,
+                           hipStream_t st) {
+  if (n < 1 || n > GV_MAX_BATCH) return CBK_ERR_SHAPE;
+  GvBatch gb;
+  const int par = calls[0].par ? 1 : 0;
+  for (int i = 0; i < n; ++i)
+    if ((calls[i].par ? 1 : 0) != par || (calls[i].m.cs_rows == 2) != (par == 1)) return CBK_ERR_UNSUPPORTED;
+  M *= par + 1;                                                   // activation rows as the kernel counts them
+  if (M > GV_MAX_M) return CBK_ERR_SHAPE;
+  gb.h.n = n; gb.h.M = M; gb.h.xdt = xdt; gb.h.ydt = ydt;
+  int cost = 0, delta_cap = 0, tiles = 0;
+  for (int i = 0; i < n; ++i) {
+    const DMat& m = calls[i].m;
+    const bool dense = family_of(m.layout) == FAM_DENSE;
+    GvMat& g = gb.mat[i];
+    g.m = m; g.x = (const uint16_t*)calls[i].x; g.ldx = calls[i].ldx;
+    g.order = !dense ? 0 : (m.bits == 2 ? 2 : 1);
+    g.par = par;
+    g.y = calls[i].y; g.bias = calls[i].bias; g.ldy = calls[i].ldy;
+    g.ntiles = (m.K + 15) / 16; g.nS = (m.N / 128 + 3) / 4; g.cost0 = cost;
+    g.tile_a = (uint32_t)m.stride * 16u;                          // sixteen rows in either order
+    g.lane_mul = m.tiled ? 16u : (uint32_t)m.stride;
+    g.sz_mul = m.tiled ? 1u : (uint32_t)m.G;
+    g.ush = m.tiled ? 8 : 4; g.csh = m.tiled ? 4 : 0;
+    cost += g.ntiles * g.nS;
+    tiles += g.ntiles;
+    delta_cap = delta_cap > M * (m.N / 128 + 4) ? delta_cap : M * (m.N / 128 + 4);
+  }
+  const int blocks = gemv_blocks(gb, n, tiles);
+  // macro-steps per work item: about one and a half items per wavefront over the whole launch
+  // (the end of an item costs about as many instructions as a step; measured best between one
+  // and two); a tile is split into at most 16 parts, and into a power of two of them where the
+  // row is long enough: the items then spread evenly over the four SIMDs.  The parts depend on
+  // the matrices of the call only, not on M: they fix the order of every row's partial sums.
+  int spi = (int)((long long)cost * 2 / ((long long)blocks * GV_WAVES * 3));
+  spi = spi < 1 ? 1 : (spi > 8 ? 8 : spi);
+  int sk_cap = 1;
+  for (int i = 0; i < n; ++i) {
+    GvMat& g = gb.mat[i];
+    int s = spi;
+    while ((g.nS + s - 1) / s > 16) ++s;
+    g.sk = (g.nS + s - 1) / s;
+    int p2 = 1;
+    while (p2 < g.sk) p2 <<= 1;
+    if (p2 <= 16 && p2 <= g.nS) g.sk = p2;
+    g.spi = (g.nS + g.sk - 1) / g.sk;                  // equal parts
+    g.sk = (g.nS + g.spi - 1) / g.spi;
+    sk_cap = sk_cap > g.sk ? sk_cap : g.sk;
+  }
+  // Long rows (at least SPLIT_MIN_STEPS macro-steps) whose digits do not fit the staging area go
+  // to the column-split kernel, one launch pair per matrix behind the others, where the
+  // configuration has one and the caller has left room for the part sums; otherwise the main
+  // kernel stages them slab by slab.
+  const DMat& m0 = gb.mat[0].m;
+  if (M > 1 && block_split_capable(m0.bits, family_of(m0.layout) == FAM_DENSE ? 0 : m0.keep, m0.group)) {
+    const size_t slot_bytes = (size_t)sk_cap * M * 16 * 4;
+    const size_t fixed = (size_t)LUT_BYTES + ZERO_BYTES + CNT_BYTES + (size_t)delta_cap * 4;
+    const size_t red_floor = 4 * slot_bytes < 24 * 1024 ? 4 * slot_bytes : 24 * 1024;
+    const size_t x_budget = 160 * 1024 - fixed - red_floor;
+    GvMat split[GV_MAX_BATCH];
+    int ns = 0;
+    size_t need = 0;
+    for (int i = 0; i < n; ++i) {
+      const GvMat& g = gb.mat[i];
+      if (g.nS >= SPLIT_MIN_STEPS && (size_t)M * NDIG * (g.m.N + X_PAD) > x_budget) {
+        split[ns++] = g;
+        need += up256(split_part_bytes(g.ntiles, g.sk, M));
+      }
+    }
+    if (ns > 0 && workspace && !((uintptr_t)workspace & 15) && ws_bytes >= need) {
+      int na = 0;
+      for (int i = 0; i < n; ++i) {
+        const GvMat& g = gb.mat[i];
+        if (!(g.nS >= SPLIT_MIN_STEPS && (size_t)M * NDIG * (g.m.N + X_PAD) > x_budget)) gb.mat[na++] = g;
+      }
+      gb.h.n = na;
+      if (na > 0) {
+        const int rc = launch_main_batch(gb, st);
+        if (rc != CBK_OK) return rc;
+      }
+      size_t off = 0;
+      for (int i = 0; i < ns; ++i) {
+        const int rc = launch_split(split[i], M, xdt, ydt, (float*)((uint8_t*)workspace + off), st);
+        if (rc != CBK_OK) return rc;
+        off += up256(split_part_bytes(split[i].ntiles, split[i].sk, M));
+      }
+      return CBK_OK;
+    }
+  }
+  return launch_main_batch(gb, st);
 }
 
 }  // namespace cbk

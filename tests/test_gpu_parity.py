@@ -305,6 +305,10 @@ def test_gemv_rows_longer_than_the_staging_area(case):
             assert float((y.double() - ref).abs().max() / ref.abs().max()) < 2e-5, (K, N, M)
             for i in range(M):
                 assert torch.equal(ops.gemv(pm, x[i:i + 1], out_dtype=torch.float32)[0], y[i]), (K, N, M, i)
+            # without room for the part sums the same rows are staged slab by slab in every
+            # workgroup instead of being split over the workgroups by columns: same bits
+            small = torch.empty(256, dtype=torch.uint8, device=DEV)
+            assert torch.equal(ops.gemv(pm, x, out_dtype=torch.float32, workspace=small), y), (K, N, M)
     # a gate/up matrix stages two scaled copies of every activation row: four rows of 5376 columns
     # are eight staged rows, more than the staging area holds at once
     K, N = 64, 5376
@@ -320,6 +324,31 @@ def test_gemv_rows_longer_than_the_staging_area(case):
         assert float((y.double() - ref).abs().max() / ref.abs().max()) < 2e-5, (K, N, M)
         for i in range(M):
             assert torch.equal(ops.gemv(pm, x[i:i + 1], out_dtype=torch.float32)[0], y[i]), (K, N, M, i)
+
+
+@pytest.mark.parametrize("case", [(F.BLK1632_4, 4, 128, 16), (F.DENSE4, 4, 128, 0), (F.BLKC, 2, 128, 16), (F.DENSEB, 2, 128, 0)], ids=case_id)
+def test_gemv_long_rows_split_by_columns(case):
+    """Two to eight activation rows of rows too long for the staging area, with room for the part
+    sums (cbk_workspace_bytes says how much): every workgroup takes one column slab of a range of
+    tiles and a second kernel adds the parts.  Bias, 16-bit outputs, a gate/up matrix (two col_scale
+    vectors by row parity), a row count off the tile, a column count off the 512-column step; row m
+    of the result is the M = 1 result bit for bit, and so is the result without a workspace."""
+    small = torch.empty(256, dtype=torch.uint8, device=DEV)
+    for (K, N, cs_rows, Ms) in ((72, 14336, 1, (8, 5, 4)), (40, 14336, 2, (4, 3)), (16, 28800, 1, (2, 7)), (4112, 8192, 1, (8,))):
+        pm, W = _fused(case, K, N, cs_rows, (0, 0), seed=K + N + cs_rows, tiled=True)
+        for dt in (torch.float32, torch.bfloat16):
+            bias = acts(1, K, dt, seed=2)[0].to(DEV)
+            for M in Ms:
+                x = acts(M, N, torch.bfloat16, seed=10 * M).to(DEV)
+                if M * cs_rows * 3 * N > 140 * 1024:
+                    assert _lib.lib().cbk_workspace_bytes(ctypes.byref(pm.desc()), M) >= (K + 15) // 16 * 16 * M * cs_rows * 4
+                y = ops.gemv(pm, x, bias=bias, out_dtype=dt)
+                if dt == torch.float32:
+                    assert rel_fro(_np(y), R.forward_ref(W, _np(x)) + _np(bias)[None, :]) < TOL, (K, N, cs_rows, M)
+                for i in range(M):
+                    assert torch.equal(ops.gemv(pm, x[i:i + 1], bias=bias, out_dtype=dt)[0], y[i]), (K, N, cs_rows, M, i)
+                assert torch.equal(ops.gemv(pm, x, bias=bias, out_dtype=dt, workspace=small), y), (K, N, cs_rows, M)
+                assert torch.equal(ops.gemv(pm, x, bias=bias, out_dtype=dt), y)
 
 
 @pytest.mark.parametrize("case", [(F.BLK1632_4, 4, 128, 16), (F.BLKC, 3, 64, 10), (F.DENSE4, 4, 128, 0)], ids=case_id)
