@@ -92,6 +92,11 @@ struct GvMat {
   // zero entry of (row, group g) has index t * 16 * G + r * sz_mul + (g << csh).
   uint32_t tile_a, lane_mul, sz_mul;
   int ush, csh;
+  // Divisions the kernel would otherwise do in software, sixteen wavefronts at a time on the one
+  // scalar unit of a CU: a / nS = (a * inv_nS) >> 32 (inv_nS = 0: not exact for this launch, divide),
+  // w / sp = (w * inv_sp) >> 16 for w <= 16, and 16 / sp, 16 % sp.
+  uint32_t inv_nS, inv_sp;
+  int dq_t, dq_p;
 };
 
 // What every wavefront needs before it can find its work: small, first in the kernel
@@ -101,7 +106,7 @@ struct GvHead {
   int cq, cr;              // cost units per workgroup: cq, and one more for the first cr workgroups
   int xq_cap, delta_cap;   // LDS bytes reserved for digits / floats reserved for delta
   int sk_cap, nslot, red_floats;   // reduction slots: nslot x sk_cap x M x 16 floats
-  int cost_end[GV_MAX_BATCH];      // cost0 + ntiles * nS of every matrix (total cost from entry n on)
+  int cost_end[GV_MAX_BATCH];      // cost0 + ntiles * nS of every matrix (INT_MAX from entry n on)
 };
 
 struct GvBatch {
@@ -384,7 +389,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
   // first matrix with cost units at or after c0
   int mi0 = 0;
 #pragma unroll
-  for (int i = 0; i < GV_MAX_BATCH; ++i) mi0 += (i < h.n && h.cost_end[i] <= c0) ? 1 : 0;
+  for (int i = 0; i < GV_MAX_BATCH - 1; ++i) mi0 += h.cost_end[i] <= c0 ? 1 : 0;     // (entries past n never count)
 
   // The first record is requested together with the header: most workgroups start with it, and
   // for them the second round trip through the argument block before any load goes out is gone.
@@ -400,8 +405,13 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     if (gm.cost0 >= c1) break;                                    // uniform over the workgroup
     const DMat& m = gm.m;
     const int nS = gm.nS;
-    int T_lo = (c0 - gm.cost0 + nS - 1) / nS, T_hi = (c1 - gm.cost0 + nS - 1) / nS;
-    T_lo = T_lo < 0 ? 0 : T_lo;
+    // ceil((c - cost0) / nS), 0 for c <= cost0
+    auto tiles_before = [&](int c) -> int {
+      const int a = c - gm.cost0 + nS - 1;
+      if (a < nS) return 0;
+      return gm.inv_nS ? (int)__umulhi((uint32_t)a, gm.inv_nS) : a / nS;
+    };
+    int T_lo = tiles_before(c0), T_hi = tiles_before(c1);
     T_hi = T_hi > gm.ntiles ? gm.ntiles : T_hi;
     if (T_lo >= T_hi) { ++mi; continue; }                         // uniform over the workgroup
     const int N = m.N, NCH = N >> 7;
@@ -516,7 +526,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     // of loads in flight, slower on large launches)
     struct Pos { int tl, part, S; };
     const int ntl = t_hi - t_lo;
-    const int dq_t = GV_WAVES / pn, dq_p = GV_WAVES % pn;
+    const bool whole = !SLABS || pn == SP;                        // (a shorter last slab divides in software)
+    const int dq_t = whole ? gm.dq_t : GV_WAVES / pn, dq_p = whole ? gm.dq_p : GV_WAVES % pn;
+    const int w_t = whole ? (int)(((uint32_t)wave * gm.inv_sp) >> 16) : wave / pn, w_p = wave - w_t * pn;
     auto advance = [&](Pos& p) -> bool {                           // false past the last position
       const int s_end = (p.part * spi + spi < nS) ? p.part * spi + spi : nS;
       if (p.S + 1 < s_end) { ++p.S; return true; }
@@ -525,7 +537,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
       p.S = p.part * spi;
       return p.tl < ntl;
     };
-    Pos p0{wave / pn, pa + wave % pn, (pa + wave % pn) * spi};
+    Pos p0{w_t, pa + w_p, (pa + w_p) * spi};
     bool v0 = p0.tl < ntl;
     Pos p1 = p0; bool v1 = v0 && advance(p1);
     // The activation loads go out before the first weight loads: the weight prefetch of a whole
@@ -810,6 +822,8 @@ struct GsArgs {
   int M, xdt, ydt;
   int xq_cap, delta_cap;   // LDS bytes of digits, floats of delta
   int nslab, wps;          // column slabs, workgroups per slab
+  int tq, tr;              // ntiles / wps, ntiles % wps
+  uint32_t inv_wps;        // b / wps = (b * inv_wps) >> 32 for the workgroup indices of the launch
   float* part;             // [ntiles][sk][M][16] part sums
 };
 
@@ -845,8 +859,8 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_split_kernel(GsArgs a) {
 
   // this workgroup: slab sl, tiles [T_lo, T_hi)
   const int bx = (int)blockIdx.x;
-  const int sl = bx / a.wps, wi = bx - sl * a.wps;
-  const int tq = gm.ntiles / a.wps, tr = gm.ntiles % a.wps;
+  const int sl = a.wps == 1 ? bx : (int)__umulhi((uint32_t)bx, a.inv_wps), wi = bx - sl * a.wps;
+  const int tq = a.tq, tr = a.tr;
   const int T_lo = wi * tq + (wi < tr ? wi : tr), T_hi = T_lo + tq + (wi < tr ? 1 : 0);
   const int ntl = T_hi - T_lo;
   if (ntl <= 0) return;                                             // uniform over the workgroup
@@ -898,7 +912,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_split_kernel(GsArgs a) {
 
   // this wave's (tile, part, macro-step) positions: items wave, wave + 16, ... of the slab
   struct Pos { int tl, part, S; };
-  const int dq_t = GV_WAVES / pn, dq_p = GV_WAVES % pn;
+  const bool whole = pn == gm.sp;                                  // (a shorter last slab divides in software)
+  const int dq_t = whole ? gm.dq_t : GV_WAVES / pn, dq_p = whole ? gm.dq_p : GV_WAVES % pn;
+  const int w_t = whole ? (int)(((uint32_t)wave * gm.inv_sp) >> 16) : wave / pn, w_p = wave - w_t * pn;
   auto advance = [&](Pos& p) -> bool {                             // false past the last position
     const int s_end = (p.part * spi + spi < nS) ? p.part * spi + spi : nS;
     if (p.S + 1 < s_end) { ++p.S; return true; }
@@ -907,7 +923,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_split_kernel(GsArgs a) {
     p.S = p.part * spi;
     return p.tl < ntl;
   };
-  Pos p0{wave / pn, pa + wave % pn, (pa + wave % pn) * spi};
+  Pos p0{w_t, pa + w_p, (pa + w_p) * spi};
   bool v0 = p0.tl < ntl;
   Pos p1 = p0; bool v1 = v0 && advance(p1);
 
@@ -1639,6 +1655,10 @@ static int launch_split(const GvMat& g, int M, int xdt, int ydt, float* part, hi
   a.nslab = (g.sk + best_pps - 1) / best_pps;
   a.wps = 256 / a.nslab;
   a.wps = a.wps < 1 ? 1 : (a.wps > g.ntiles ? g.ntiles : a.wps);
+  a.tq = g.ntiles / a.wps; a.tr = g.ntiles % a.wps;
+  a.inv_wps = a.wps > 1 ? (uint32_t)(((1ull << 32) + a.wps - 1) / a.wps) : 0u;     // exact: workgroup index * wps < 2^32
+  a.g.inv_sp = (uint32_t)((65536 + best_pps - 1) / best_pps);
+  a.g.dq_t = GV_WAVES / best_pps; a.g.dq_p = GV_WAVES % best_pps;
   const int cols = best_pps * g.spi * 512 < g.m.N ? best_pps * g.spi * 512 : g.m.N;
   a.xq_cap = M * NDIG * (cols + X_PAD);
   const size_t lds = (size_t)LUT_BYTES + ZERO_BYTES + a.xq_cap + (size_t)a.delta_cap * 4;
@@ -1667,7 +1687,7 @@ static int launch_main_batch(GvBatch& gb, hipStream_t st) {
     delta_cap = delta_cap > M * (g.m.N / 128 + 4) ? delta_cap : M * (g.m.N / 128 + 4);
     sk_cap = sk_cap > g.sk ? sk_cap : g.sk;
   }
-  for (int i = n; i < GV_MAX_BATCH; ++i) gb.h.cost_end[i] = cost;
+  for (int i = n; i < GV_MAX_BATCH; ++i) gb.h.cost_end[i] = 0x7fffffff;
   const int blocks = gemv_blocks(gb, n, tiles);
   // LDS: selector table, zero row and counters, the deltas, the reduction slots, and the activation
   // digits, which get what the others leave: at least four reduction slots are kept back (up to 24 KB
@@ -1689,6 +1709,11 @@ static int launch_main_batch(GvBatch& gb, hipStream_t st) {
     }
     const int slab_cols = g.sp >= g.sk ? N : g.sp * g.spi * 512;
     xq_cap = xq_cap > M * NDIG * (slab_cols + X_PAD) ? xq_cap : M * NDIG * (slab_cols + X_PAD);
+    if (g.sp > g.sk) g.sp = g.sk;
+    // exact for every a the kernel divides (a < cost + nS) when (cost + nS) * nS < 2^32
+    g.inv_nS = g.nS > 1 && (uint64_t)(cost + g.nS) * g.nS < (1ull << 32) ? (uint32_t)(((1ull << 32) + g.nS - 1) / g.nS) : 0u;
+    g.inv_sp = (uint32_t)((65536 + g.sp - 1) / g.sp);
+    g.dq_t = GV_WAVES / g.sp; g.dq_p = GV_WAVES % g.sp;
   }
   gb.h.xq_cap = xq_cap; gb.h.delta_cap = delta_cap;
   // reduction slots: as many as fit what is left, at most 24 KB: a power of two between 2 and 64
