@@ -29,7 +29,9 @@
 // The activation digits and the byte-permute selector table live in LDS for the whole launch;
 // where the digits of all rows of a matrix do not fit (two to eight activation rows of a long
 // row) they are staged one column slab at a time, whole split-K parts per slab, while the partial
-// sums of the tiles wait in their LDS slots: the weights are still read once.
+// sums of the tiles wait in their LDS slots: the weights are still read once.  With room for the
+// part sums in the caller's workspace such rows go to gemv_split_kernel instead, where a
+// workgroup owns one column slab of a range of tiles and a second kernel adds the parts.
 //
 // Expansion of the bitmap.  For one mask byte (8 columns, r survivors before it in its
 // 32-column block) the survivor codes r .. r+7 are shifted out of the block's code bits,

@@ -130,11 +130,15 @@ size_t cbk_row_stride(const cbk_desc* d);
  * (pack_cobalt.write_matrix :431-433 `stream_bytes`); SPARSE layouts need data_bytes. */
 size_t cbk_stream_bytes(const cbk_desc* d, size_t sparse_data_bytes);
 
-/* Device scratch needed by cbk_gemv / cbk_gemm / cbk_linear for M activation rows (0 for the
- * decode kernels; the prefill kernel keeps its pre-scaled fp16 activations there:
- * ceil(M/256)*256 * ceil(N/256)*256 * 2 bytes per col_scale vector, i.e. times cs_rows for a
- * fused matrix, one float32 scale per activation row and col_scale vector, plus float32 partial
- * outputs when the library splits the column range of a launch that would not fill the chip).
+/* Device scratch needed by cbk_gemv / cbk_gemm / cbk_linear for M activation rows.  The prefill
+ * kernel keeps its pre-scaled fp16 activations there: ceil(M/256)*256 * ceil(N/256)*256 * 2 bytes
+ * per col_scale vector, i.e. times cs_rows for a fused matrix, one float32 scale per activation
+ * row and col_scale vector, plus float32 partial outputs when the library splits the column range
+ * of a launch that would not fill the chip.  The decode kernels need none, with one optional use:
+ * two to eight activation rows of rows of 8192 columns and more whose activations do not fit in
+ * LDS (M * 3 * N bytes above about 100 KB) are split over the workgroups by columns when there
+ * is room for the float32 part sums, K * 16 * M * 4 bytes at most; with a smaller workspace, or
+ * none, cbk_gemv computes the same bits more slowly and reports no error.
  * Ask, do not compute.  256-byte aligned. */
 size_t cbk_workspace_bytes(const cbk_desc* d, int M);
 
@@ -177,9 +181,10 @@ int cbk_unpack(const cbk_desc* d, void* q, void* mask_bits, void* stream);
 /* Decode path, 1 <= M <= 16: y[m, k] = sum_j x[m, j] * W_hat[k, j] (+ bias[k]).
  * x is [M, ldx] fp16 or bf16, y is [M, ldy] in y_dtype (f32 / f16 / bf16), bias is NULL or
  * K values of y_dtype.  Up to eight activation rows share one pass over the weights on the
- * matrix-core kernel, whatever the row length (two to eight rows of a long row are staged in
- * column slabs); more rows, or configurations that kernel takes four rows of at a time, are
- * passes over the weights.  Row m of the result does not depend on M.  Replaces the harness
+ * matrix-core kernel, whatever the row length (two to eight rows of a long row: split over the
+ * workgroups by columns through the workspace, see cbk_workspace_bytes, or staged in column slabs
+ * without one); more rows, or configurations that kernel takes four rows of at a time, are
+ * passes over the weights.  Row m of the result does not depend on M, nor on the workspace.  Replaces the harness
  * entry `gemv` (test_gemv.cu:187-199) and cbk::gemv_rows (cobalt_gemv.cuh:1196-1213); unlike
  * those it applies col_scale itself. */
 int cbk_gemv(const cbk_desc* d, const void* x, int x_dtype, int M, int64_t ldx,
