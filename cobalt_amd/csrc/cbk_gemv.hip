@@ -407,6 +407,34 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     if (gm.cost0 >= c1) break;                                    // uniform over the workgroup
     const DMat& m = gm.m;
     const int nS = gm.nS;
+    const int N = m.N, NCH = N >> 7;
+    // items: tile tl (local), part j of SK; part j covers macro-steps [j*spi, min(nS,(j+1)*spi))
+    const int SK = gm.sk, spi = gm.spi, SP = SLABS ? gm.sp : SK;
+    const int pn = SLABS && SK - pa >= SP ? SP : SK - pa;         // parts of this slab
+    const int col0 = SLABS ? pa * spi * 512 : 0;                  // its columns: [col0, col0 + Ns)
+    const int Ns = SLABS && N - col0 >= pn * spi * 512 ? pn * spi * 512 : N - col0;
+    const int ch0 = col0 >> 7;
+
+    // The activation loads go out first, as soon as the matrix is known: before the weight loads,
+    // because the weight prefetch of a whole launch is tens of megabytes and a request queued
+    // behind it would keep every wavefront from decoding until that burst has drained; and before
+    // the rest of the set-up, which is a few hundred scalar instructions on the one scalar unit
+    // the sixteen wavefronts share.
+    const int n16 = Ns >> 4, xitems = h.M * n16;                  // a multiple of 8
+    // The first two items of a thread (all there are, but for the longest rows) are loaded here
+    // and converted outside the loop further down: inside it the compiler's wait for an item's
+    // loads has to allow for the trip in which they were issued after the weight loads, and so
+    // waits for the weight loads as well; the conversion would start only once the first weights
+    // have arrived instead of running while they are on their way.
+    // (The second item only where its sixteen registers do not push the kernel into scratch.)
+    constexpr bool PRE2 = MP == 1 || (MP == 4 && QB);
+    int xit = tid;
+    XLoad xl, xl2;
+    if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, N, col0, n16, xit, MP == 1, gm.par, xl);
+    if (PRE2 && xit + GV_THREADS < xitems)
+      stage_load(gm.x, gm.ldx, m.cs, N, col0, n16, xit + GV_THREADS, MP == 1, gm.par, xl2);
+    __builtin_amdgcn_sched_barrier(0);
+
     // ceil((c - cost0) / nS), 0 for c <= cost0
     auto tiles_before = [&](int c) -> int {
       const int a = c - gm.cost0 + nS - 1;
@@ -416,9 +444,6 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     int T_lo = tiles_before(c0), T_hi = tiles_before(c1);
     T_hi = T_hi > gm.ntiles ? gm.ntiles : T_hi;
     if (T_lo >= T_hi) { ++mi; continue; }                         // uniform over the workgroup
-    const int N = m.N, NCH = N >> 7;
-    // items: tile tl (local), part j of SK; part j covers macro-steps [j*spi, min(nS,(j+1)*spi))
-    const int SK = gm.sk, spi = gm.spi, SP = SLABS ? gm.sp : SK;
     // A row whose digits do not fit in LDS is staged and multiplied slab by slab (SP parts of
     // every tile at a time).  A tile's partial sums then wait in their reduction slot across the
     // slabs, so the tiles are taken nslot at a time and the slots are never reused inside a group.
@@ -437,10 +462,6 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     const int t_lo = SLABS && g_lo >= 0 ? g_lo : T_lo;
     const int t_hi = SLABS && t_lo + tgs < T_hi ? t_lo + tgs : T_hi;
     const int last_tile = t_hi - 1;
-    const int pn = SLABS && SK - pa >= SP ? SP : SK - pa;         // parts of this slab
-    const int col0 = SLABS ? pa * spi * 512 : 0;                  // its columns: [col0, col0 + Ns)
-    const int Ns = SLABS && N - col0 >= pn * spi * 512 ? pn * spi * 512 : N - col0;
-    const int ch0 = col0 >> 7;
 
     // ---- issue the loads of one (tile, macro-step) position; out-of-range positions are clamped
     // Everything that depends only on (tile, S) is scalar work; a lane adds a 32-bit offset.
@@ -541,29 +562,14 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
     };
     Pos p0{w_t, pa + w_p, (pa + w_p) * spi};
     bool v0 = p0.tl < ntl;
-    Pos p1 = p0; bool v1 = v0 && advance(p1);
-    // The activation loads go out before the first weight loads: the weight prefetch of a whole
-    // launch is tens of megabytes, and a request queued behind it would keep every wavefront
-    // from decoding until that burst has drained.
-    const int n16 = Ns >> 4, xitems = h.M * n16;                  // a multiple of 8
-    // The first two items of a thread (all there are, but for the longest rows) are loaded here
-    // and converted outside the loop further down: inside it the compiler's wait for an item's
-    // loads has to allow for the trip in which they were issued after the weight loads, and so
-    // waits for the weight loads as well; the conversion would start only once the first weights
-    // have arrived instead of running while they are on their way.
-    // (The second item only where its sixteen registers do not push the kernel into scratch.)
-    constexpr bool PRE2 = MP == 1 || (MP == 4 && QB);
-    int xit = tid;
-    XLoad xl, xl2;
-    if (xit < xitems) stage_load(gm.x, gm.ldx, m.cs, N, col0, n16, xit, MP == 1, gm.par, xl);
-    if (PRE2 && xit + GV_THREADS < xitems)
-      stage_load(gm.x, gm.ldx, m.cs, N, col0, n16, xit + GV_THREADS, MP == 1, gm.par, xl2);
     // Two load buffers swap roles (being decoded, being loaded) by name: copying a buffer would
     // wait for the loads that are still filling it.  One step of loads in flight per wavefront
     // is the measured optimum (sixteen wavefronts per CU already cover the latency; a second
     // step in flight made the Mistral layer set 8 % slower).
     Loads<C> LA, LB;
     issue(t_lo + p0.tl, p0.S, LA);
+    __builtin_amdgcn_sched_barrier(0);                            // (the first loads leave before the rest of the set-up)
+    Pos p1 = p0; bool v1 = v0 && advance(p1);
 
     // ---- stage: selector table and counters (once), activation digits and deltas of this matrix
     if (!first) __syncthreads();                                  // previous matrix fully consumed
