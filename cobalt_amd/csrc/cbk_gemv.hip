@@ -1698,14 +1698,14 @@ static int launch_main_batch(GvBatch& gb, hipStream_t st) {
   for (int i = n; i < GV_MAX_BATCH; ++i) gb.h.cost_end[i] = 0x7fffffff;
   const int blocks = gemv_blocks(gb, n, tiles);
   // LDS: selector table, zero row and counters, the deltas, the reduction slots, and the activation
-  // digits, which get what the others leave: at least four reduction slots are kept back (up to 24 KB
+  // digits, which get what the others leave: at least two reduction slots are kept back (up to 24 KB
   // of them where there is room), so that eight rows of 5376 columns (126 KB of digits) are still
   // staged whole.  Rows whose digits do not fit are staged in column slabs: as many whole parts as the
   // budget holds (a part is at most 8 steps = 4096 columns, 12 KB per activation row, so one part of
   // eight rows always fits).
   const size_t slot_bytes = (size_t)sk_cap * M * 16 * 4;
   const size_t fixed = (size_t)LUT_BYTES + ZERO_BYTES + CNT_BYTES + (size_t)delta_cap * 4;
-  const size_t red_floor = 4 * slot_bytes < 24 * 1024 ? 4 * slot_bytes : 24 * 1024;
+  const size_t red_floor = 2 * slot_bytes < 24 * 1024 ? 2 * slot_bytes : 24 * 1024;
   const size_t x_budget = M == 1 ? (size_t)X_LDS_BUDGET : 160 * 1024 - fixed - red_floor;
   for (int i = 0; i < n; ++i) {
     GvMat& g = gb.mat[i];
@@ -1714,6 +1714,8 @@ static int launch_main_batch(GvBatch& gb, hipStream_t st) {
     if ((size_t)M * NDIG * (N + X_PAD) > x_budget) {
       g.sp = (int)((x_budget - (size_t)M * NDIG * X_PAD) / ((size_t)M * NDIG * g.spi * 512));
       if (g.sp < 1 || M == 1) return CBK_ERR_UNSUPPORTED;         // (the one-row kernels stage whole rows only)
+      const int nsl = (g.sk + g.sp - 1) / g.sp;                   // slabs of equal length, not a short last one
+      g.sp = (g.sk + nsl - 1) / nsl;
     }
     const int slab_cols = g.sp >= g.sk ? N : g.sp * g.spi * 512;
     xq_cap = xq_cap > M * NDIG * (slab_cols + X_PAD) ? xq_cap : M * NDIG * (slab_cols + X_PAD);
@@ -1800,7 +1802,7 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
   if (M > 1 && block_split_capable(m0.bits, family_of(m0.layout) == FAM_DENSE ? 0 : m0.keep, m0.group)) {
     const size_t slot_bytes = (size_t)sk_cap * M * 16 * 4;
     const size_t fixed = (size_t)LUT_BYTES + ZERO_BYTES + CNT_BYTES + (size_t)delta_cap * 4;
-    const size_t red_floor = 4 * slot_bytes < 24 * 1024 ? 4 * slot_bytes : 24 * 1024;
+    const size_t red_floor = 2 * slot_bytes < 24 * 1024 ? 2 * slot_bytes : 24 * 1024;
     const size_t x_budget = 160 * 1024 - fixed - red_floor;
     GvMat split[GV_MAX_BATCH];
     int ns = 0;
