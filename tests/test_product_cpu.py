@@ -123,6 +123,25 @@ def test_descriptor_validation_and_strides():
     assert L.cbk_desc_check(None, ctypes.byref(o)) == -1
 
 
+def test_workspace_sizes_of_the_decode_path():
+    """cbk_workspace_bytes at decode sizes (host arithmetic only, nothing is launched): two to eight
+    activation rows of a long row (8192 columns and more, digits beyond LDS) leave room for the
+    part sums of the column-split kernel, K * M * parts * 4 bytes with 14 parts at 21504 columns;
+    the figure is a multiple of 256, grows with M, and a batch asks for the sum of its matrices."""
+    L = _lib.lib()
+    flags = F.zero_flags(15, 4)
+    long_row = F.CbkDesc(K=5376, N=21504, layout=F.BLK1632_4, flags=flags)
+    short_row = F.CbkDesc(K=21504, N=5376, layout=F.BLK1632_4, flags=flags)
+    last = 0
+    for M in (2, 4, 8):
+        need = L.cbk_workspace_bytes(ctypes.byref(long_row), M)
+        assert need >= 5376 * M * 14 * 4 and need % 256 == 0 and need >= last
+        last = need
+    descs = (F.CbkDesc * 2)(long_row, short_row)
+    assert L.cbk_gemv_batch_workspace_bytes(2, descs, 8) == \
+        L.cbk_workspace_bytes(ctypes.byref(long_row), 8) + L.cbk_workspace_bytes(ctypes.byref(short_row), 8)
+
+
 def test_entry_points_reject_bad_arguments_before_any_launch():
     L = _lib.lib()
     d = F.CbkDesc(K=16, N=256, layout=F.BLK1632_4)
