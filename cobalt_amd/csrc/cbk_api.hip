@@ -328,7 +328,7 @@ int cbk_gemv_batch(int n, const cbk_desc* descs, const void* const* xs, const in
   // activation rows per pass: as many (8, 4, 2 or 1) as the kernel takes for every matrix and
   // their digits fit in LDS with; a gate/up matrix stages two scaled copies of every activation row
   const int vm = fast && calls[0].par ? 2 : 1;
-  int mc = M * vm > 4 ? 8 / vm : (M * vm >= 4 ? 4 / vm : (M * vm >= 2 ? 2 / vm : 1));
+  int mc = M * vm > 4 ? 8 / vm : (M * vm > 2 ? 4 / vm : (M * vm >= 2 ? 2 / vm : 1));   // (three rows: one pass of four)
   for (int i = 0; fast && i < nc; ++i) {
     while (mc > 1 && !gemv_fast_takes(calls[i].m, mc * vm) && gemv_fast_takes(calls[i].m, vm)) mc >>= 1;
     fast = gemv_fast_takes(calls[i].m, vm) && gemv_same_config(calls[0].m, calls[i].m) && calls[i].par == calls[0].par;
