@@ -57,7 +57,9 @@ constexpr int ZERO_BYTES = 256;
 constexpr int CNT_SLOTS = 64;                 // most reduction slots (arrival counters)
 constexpr int CNT_BYTES = CNT_SLOTS * 4;       // at a fixed place: zeroed before the arguments are read
 constexpr int X_LDS_BUDGET = 112 * 1024;      // activation digits of one column slab: M * 3 * columns bytes (of 160 KB LDS)
-constexpr int DELTA_LDS_BUDGET = 6 * 1024;    // one float per 128-column chunk and activation row
+constexpr int DELTA_LDS_BUDGET = 16 * 1024;   // one float per 128-column chunk and activation row (eight rows of 65024
+                                              // columns; the digits take what is left: a part of 4096 columns of
+                                              // eight rows, 96 KB, still fits beside 24 KB of reduction slots)
 constexpr int NDIG = 3;                       // int8 digits per activation
 // The digit rows of the matrix-core kernels lie X_PAD bytes further apart than their length.  The
 // sixteen lanes of a quarter read sixteen bytes each from up to twelve different rows (activation

@@ -292,10 +292,11 @@ def test_gemv_five_to_eight_rows_equal_single_rows(case):
 @pytest.mark.parametrize("case", [(F.BLK1632_4, 4, 128, 16), (F.DENSE4, 4, 128, 0), (F.BLKC, 3, 128, 10)], ids=case_id)
 def test_gemv_rows_longer_than_the_staging_area(case):
     """Rows whose activation digits do not fit in LDS are staged and multiplied in column slabs, the
-    weights still streamed once: one row of 65536 columns, eight rows of 14336 and 21504 columns, and
+    weights still streamed once: one row of 65536 columns, eight rows of 14336, 21504 and 28672
+    columns (the deltas of eight rows of 28672 columns are 7 KB of LDS by themselves), and
     a matrix with several 16-row tiles per workgroup (more tiles than reduction slots).  Checked
     against float64 on the dequantised weights and, bit for bit, against the single-row results."""
-    for (K, N, Ms) in ((16, 65536, (1, 2)), (48, 21504, (8, 3)), (8208, 14336, (8,))):
+    for (K, N, Ms) in ((16, 65536, (1, 2)), (48, 21504, (8, 3)), (8208, 14336, (8,)), (24, 28672, (8, 5))):
         pm = F.synth_packed(K, N, case[0], case[1], case[2], case[3], seed=K + N, device=DEV).to_tiled()
         W = ops.dequant(pm, torch.float32).double()
         for M in Ms:
