@@ -827,15 +827,25 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 // to the wavefronts and writes the part sums to a caller-provided buffer; a second small kernel
 // adds the parts of every output in part order.  Same operations in the same order as for one
 // activation row, so a row's result still does not depend on M.  Block-per-quarter arrangement only.
-struct GsArgs {
+struct GsMat {             // one matrix of a column-split launch
   GvMat g;                 // spi, sk: the parts; sp: parts per slab
-  int M, xdt, ydt;
-  int xq_cap, delta_cap;   // LDS bytes of digits, floats of delta
   int nslab, wps;          // column slabs, workgroups per slab
   int tq, tr;              // ntiles / wps, ntiles % wps
-  uint32_t inv_wps;        // b / wps = (b * inv_wps) >> 32 for the workgroup indices of the launch
+  uint32_t inv_wps;        // b / wps = (b * inv_wps) >> 32 for the matrix's workgroup indices
+  int wg0, th0;            // its first workgroup, and its first thread in the reduce launch
   float* part;             // [ntiles][sk][M][16] part sums
 };
+struct GsHead {
+  int n, M, xdt, ydt;
+  int xq_cap, delta_cap;   // LDS bytes of digits, floats of delta
+  int wg_end[GV_MAX_BATCH];   // workgroups up to and including matrix i (INT_MAX from entry n on)
+  int th_end[GV_MAX_BATCH];   // the same for the threads of the reduce launch
+};
+struct GsArgs {
+  GsHead h;
+  GsMat mat[GV_MAX_BATCH];
+};
+static_assert(sizeof(GsArgs) <= 4096 && sizeof(GvBatch) <= 4096, "kernel argument blocks are at most 4 KB");
 
 template <int BITS, int KEEP, int GRP, int MP>
 __global__ __launch_bounds__(GV_THREADS) void gemv_split_kernel(GsArgs a) {
@@ -848,10 +858,17 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_split_kernel(GsArgs a) {
   uint2* lut = (uint2*)smem;
   uint8_t* zreg = smem + LUT_BYTES;
   int8_t* xq = (int8_t*)zreg + ZERO_BYTES;
-  float* delta = (float*)(xq + a.xq_cap);
-  const GvMat& gm = a.g;
+  const GsHead h = a.h;
+  float* delta = (float*)(xq + h.xq_cap);
+  // the matrix of this workgroup
+  int bx = (int)blockIdx.x, mi = 0;
+#pragma unroll
+  for (int i = 0; i < GV_MAX_BATCH - 1; ++i) mi += bx >= h.wg_end[i] ? 1 : 0;
+  const GsMat gs = a.mat[mi];
+  bx -= gs.wg0;
+  const GvMat& gm = gs.g;
   const DMat& m = gm.m;
-  const int M = a.M, N = m.N, NCH = N >> 7, nS = gm.nS, spi = gm.spi, SK = gm.sk;
+  const int M = h.M, N = m.N, NCH = N >> 7, nS = gm.nS, spi = gm.spi, SK = gm.sk;
   if (tid < 256) {
     const uint2 e = make_selectors((uint32_t)tid, C::SEL_KIND);
 #pragma unroll
@@ -868,9 +885,8 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_split_kernel(GsArgs a) {
   const uint32_t xq_off = (uint32_t)((uint8_t*)xq - smem), z_off = (uint32_t)(zreg - smem);
 
   // this workgroup: slab sl, tiles [T_lo, T_hi)
-  const int bx = (int)blockIdx.x;
-  const int sl = a.wps == 1 ? bx : (int)__umulhi((uint32_t)bx, a.inv_wps), wi = bx - sl * a.wps;
-  const int tq = a.tq, tr = a.tr;
+  const int sl = gs.wps == 1 ? bx : (int)__umulhi((uint32_t)bx, gs.inv_wps), wi = bx - sl * gs.wps;
+  const int tq = gs.tq, tr = gs.tr;
   const int T_lo = wi * tq + (wi < tr ? wi : tr), T_hi = T_lo + tq + (wi < tr ? 1 : 0);
   const int ntl = T_hi - T_lo;
   if (ntl <= 0) return;                                             // uniform over the workgroup
@@ -944,10 +960,10 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_split_kernel(GsArgs a) {
   if (tid < xitems) stage_load(gm.x, gm.ldx, m.cs, N, col0, n16, tid, false, gm.par, xl);
   Loads<C> LA, LB;
   issue(T_lo + p0.tl, p0.S, LA);
-  if (tid < xitems) stage_convert<XORD>(xl, m.cs != nullptr, a.xdt, N, ch0, n16, tid, false, xq, delta, X_PAD);
+  if (tid < xitems) stage_convert<XORD>(xl, m.cs != nullptr, h.xdt, N, ch0, n16, tid, false, xq, delta, X_PAD);
   for (int xit = tid + GV_THREADS; xit < xitems; xit += GV_THREADS) {
     stage_load(gm.x, gm.ldx, m.cs, N, col0, n16, xit, false, gm.par, xl);
-    stage_convert<XORD>(xl, m.cs != nullptr, a.xdt, N, ch0, n16, xit, false, xq, delta, X_PAD);
+    stage_convert<XORD>(xl, m.cs != nullptr, h.xdt, N, ch0, n16, xit, false, xq, delta, X_PAD);
   }
   __syncthreads();
 
@@ -1014,7 +1030,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_split_kernel(GsArgs a) {
 #pragma unroll
       for (int g = 0; g < NG; ++g) {
         const float ps = (ysum[4 * g] + ysum[4 * g + 1]) + (ysum[4 * g + 2] + ysum[4 * g + 3]);
-        if (kq + 4 * g < M) a.part[((size_t)(tile * SK + part) * M + kq + 4 * g) * 16 + wr] = ps;
+        if (kq + 4 * g < M) gs.part[((size_t)(tile * SK + part) * M + kq + 4 * g) * 16 + wr] = ps;
       }
     }
     p0 = p1; v0 = v1;
@@ -1031,9 +1047,14 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_split_kernel(GsArgs a) {
 // the parts of every output, added in part order; bias; conversion
 constexpr int GS_RED_THREADS = 64;
 __global__ __launch_bounds__(GS_RED_THREADS) void gemv_split_reduce_kernel(GsArgs a) {
-  const GvMat& gm = a.g;
-  const int M = a.M, SK = gm.sk;
-  const int idx = (int)blockIdx.x * GS_RED_THREADS + (int)threadIdx.x;
+  const GsHead& h = a.h;
+  int idx = (int)blockIdx.x * GS_RED_THREADS + (int)threadIdx.x, mi = 0;
+#pragma unroll
+  for (int i = 0; i < GV_MAX_BATCH - 1; ++i) mi += idx >= h.th_end[i] ? 1 : 0;     // (uniform over the workgroup)
+  const GsMat& gs = a.mat[mi];
+  idx -= gs.th0;
+  const GvMat& gm = gs.g;
+  const int M = h.M, SK = gm.sk;
   const int wr = idx & 15, t = idx >> 4, tile = t / M, am = t - tile * M;
   if (tile >= gm.ntiles) return;
   const int k = tile * 16 + wr;
@@ -1045,15 +1066,15 @@ __global__ __launch_bounds__(GS_RED_THREADS) void gemv_split_reduce_kernel(GsArg
   }
   float pv[16];                                                     // all loads first (at most 16 parts), then the sum in part order
 #pragma unroll
-  for (int j = 0; j < 16; ++j) pv[j] = a.part[((size_t)(tile * SK + (j < SK ? j : SK - 1)) * M + am) * 16 + wr];
+  for (int j = 0; j < 16; ++j) pv[j] = gs.part[((size_t)(tile * SK + (j < SK ? j : SK - 1)) * M + am) * 16 + wr];
   float v = 0.f;
 #pragma unroll
   for (int j = 0; j < 16; ++j) v += j < SK ? pv[j] : 0.f;
-  if (gm.bias) v += (a.ydt == CBK_F32) ? ((const float*)gm.bias)[k]
-                  : (a.ydt == CBK_F16) ? h2f(((const uint16_t*)gm.bias)[k]) : bf2f(((const uint16_t*)gm.bias)[k]);
+  if (gm.bias) v += (h.ydt == CBK_F32) ? ((const float*)gm.bias)[k]
+                  : (h.ydt == CBK_F16) ? h2f(((const uint16_t*)gm.bias)[k]) : bf2f(((const uint16_t*)gm.bias)[k]);
   const size_t o = (size_t)om * gm.ldy + k;
-  if (a.ydt == CBK_F32) ((float*)gm.y)[o] = v;
-  else if (a.ydt == CBK_F16) ((uint16_t*)gm.y)[o] = f2h(v);
+  if (h.ydt == CBK_F32) ((float*)gm.y)[o] = v;
+  else if (h.ydt == CBK_F16) ((uint16_t*)gm.y)[o] = f2h(v);
   else ((uint16_t*)gm.y)[o] = f2bf(v);
 }
 
@@ -1531,11 +1552,38 @@ bool gemv_same_config(const DMat& a, const DMat& b) {
   return da == db && a.bits == b.bits && a.group == b.group && (da || a.keep == b.keep);
 }
 
-// Rows whose digits are certainly staged whole need no workspace; longer ones (two to eight
-// activation rows of a block-per-quarter configuration) are split over the workgroups by columns
-// when the caller provides room for the part sums: [tiles][parts <= 16][M][16] floats.
-constexpr size_t SPLIT_MIN_BYTES = 100 * 1024;
-constexpr int SPLIT_MIN_STEPS = 16;           // rows of at least 8192 columns
+// Macro-steps per work item of a launch of `cost` tile-steps on `blocks` workgroups: about one and
+// a half items per wavefront over the whole launch (the end of an item costs about as many
+// instructions as a step; measured best between one and two).
+static inline int launch_spi(long long cost, int blocks) {
+  const int spi = (int)(cost * 2 / ((long long)blocks * GV_WAVES * 3));
+  return spi < 1 ? 1 : (spi > 8 ? 8 : spi);
+}
+// The parts of a row of nS macro-steps: at most 16, a power of two of them where the row is long
+// enough (the items then spread evenly over the four SIMDs), of equal length.
+static inline void row_parts(int nS, int spi_launch, int& spi, int& sk) {
+  int s = spi_launch;
+  while ((nS + s - 1) / s > 16) ++s;
+  sk = (nS + s - 1) / s;
+  int p2 = 1;
+  while (p2 < sk) p2 <<= 1;
+  if (p2 <= 16 && p2 <= nS) sk = p2;
+  spi = (nS + sk - 1) / sk;
+  sk = (nS + spi - 1) / spi;
+}
+// LDS left for the activation digits of M rows beside the selector table, the deltas and two
+// reduction slots (up to 24 KB of slots where there is room)
+static inline size_t main_x_budget(int M, int delta_cap, int sk_cap) {
+  const size_t slot_bytes = (size_t)sk_cap * M * 16 * 4;
+  const size_t fixed = (size_t)LUT_BYTES + ZERO_BYTES + CNT_BYTES + (size_t)delta_cap * 4;
+  const size_t red_floor = 2 * slot_bytes < 24 * 1024 ? 2 * slot_bytes : 24 * 1024;
+  return 160 * 1024 - fixed - red_floor;
+}
+
+// Rows whose digits (M * 3 * N bytes) stay within X_LDS_BUDGET need no workspace; longer ones (two
+// to eight activation rows of a block-per-quarter configuration) are split over the workgroups by
+// columns when the caller provides room for the part sums: [tiles][parts <= 16][M][16] floats.
+constexpr int SPLIT_MAX_TILES = 4096;          // (rows that fit are split only in launches of at most this many tiles)
 static inline int kernel_rows(const DMat& m, int M) {            // activation rows as the kernel counts them, per pass
   const int v = m.cs_rows == 2 ? 2 : 1;
   return M * v > GV_MAX_M ? GV_MAX_M : M * v;
@@ -1545,8 +1593,15 @@ static inline size_t split_part_bytes(int ntiles, int sk, int Mk) { return (size
 size_t gemv_fast_workspace(const DMat& m, int M) {
   const int Mk = kernel_rows(m, M);
   if (Mk < 2 || !block_split_capable(m.bits, family_of(m.layout) == FAM_DENSE ? 0 : m.keep, m.group)) return 0;
-  if ((size_t)Mk * NDIG * (m.N + X_PAD) <= SPLIT_MIN_BYTES || (m.N / 128 + 3) / 4 < SPLIT_MIN_STEPS) return 0;
-  return up256(split_part_bytes((m.K + 15) / 16 + 3, 16, Mk));     // (+3: a q|k|v matrix is run as its three ranges)
+  const size_t digits = (size_t)Mk * NDIG * (m.N + X_PAD);
+  if (digits <= (size_t)X_LDS_BUDGET) return 0;
+  // what a call with this matrix alone would do
+  const int ntiles = (m.K + 15) / 16, nS = (m.N / 128 + 3) / 4;
+  int spi, sk;
+  row_parts(nS, launch_spi((long long)ntiles * nS, ntiles < 256 ? ntiles : 256), spi, sk);
+  if (digits <= main_x_budget(Mk, Mk * (m.N / 128 + 4), sk) && ntiles > SPLIT_MAX_TILES) return 0;
+  if (ntiles < 256) sk = nS < 16 ? nS : 16;                       // (in a batch a small matrix may be cut finer)
+  return up256(split_part_bytes(ntiles + 3, sk, Mk));             // (+3: a q|k|v matrix is run as its three ranges)
 }
 
 struct GvCall {           // one matrix of a batched call, host side
@@ -1619,7 +1674,7 @@ static int gemv_blocks(const GvBatch& gb, int n, int tiles) {
 }
 
 template <int BITS, int KEEP, int GRP, int MP>
-static int launch_split_cfg(const GsArgs& a, size_t lds, hipStream_t st) {
+static int launch_split_cfg(const GsArgs& a, size_t lds, int blocks, int red_blocks, hipStream_t st) {
   if constexpr ((MP == 4 || MP == 8) && block_split_capable(BITS, KEEP, GRP)) {
     auto kern = gemv_split_kernel<BITS, KEEP, GRP, MP>;
     static std::atomic<int> configured{0};
@@ -1628,59 +1683,83 @@ static int launch_split_cfg(const GsArgs& a, size_t lds, hipStream_t st) {
         return CBK_ERR_HIP;
       configured.store(1, std::memory_order_release);
     }
-    hipLaunchKernelGGL(kern, dim3(a.nslab * a.wps), dim3(GV_THREADS), lds, st, a);
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(GV_THREADS), lds, st, a);
     if (hipGetLastError() != hipSuccess) return CBK_ERR_HIP;
-    hipLaunchKernelGGL(gemv_split_reduce_kernel, dim3((a.g.ntiles * a.M * 16 + GS_RED_THREADS - 1) / GS_RED_THREADS),
-                       dim3(GS_RED_THREADS), 0, st, a);
+    hipLaunchKernelGGL(gemv_split_reduce_kernel, dim3(red_blocks), dim3(GS_RED_THREADS), 0, st, a);
     return hipGetLastError() == hipSuccess ? CBK_OK : CBK_ERR_HIP;
   } else {
     return CBK_ERR_UNSUPPORTED;
   }
 }
 
-// One long-row matrix (spi and sk set) through gemv_split_kernel: parts per slab, workgroups per
-// slab, LDS.  `part` holds split_part_bytes(ntiles, sk, M).
-static int launch_split(const GvMat& g, int M, int xdt, int ydt, float* part, hipStream_t st) {
+// The matrices `mats` (spi and sk set) through one launch of gemv_split_kernel and one of the
+// reduce kernel: workgroups per matrix by its share of the work, parts per slab, workgroups per
+// slab, LDS.  `ws` holds the part sums of the matrices one after the other, each
+// up256(split_part_bytes(ntiles, sk, M)).
+static int launch_split_batch(const GvMat* mats, int n, int M, int xdt, int ydt, uint8_t* ws, hipStream_t st) {
   GsArgs a;
-  a.g = g; a.M = M; a.xdt = xdt; a.ydt = ydt; a.part = part;
-  a.delta_cap = M * (g.m.N / 128 + 4);
-  const size_t fixed = (size_t)LUT_BYTES + ZERO_BYTES + (size_t)a.delta_cap * 4 + (size_t)M * NDIG * X_PAD;
-  const size_t per_part = (size_t)M * NDIG * g.spi * 512;
-  if (fixed + per_part > 160 * 1024) return CBK_ERR_UNSUPPORTED;
-  int pps_max = (int)((160 * 1024 - fixed) / per_part);
-  pps_max = pps_max < g.sk ? pps_max : g.sk;
-  // Parts per slab: a workgroup runs ceil(items / 16) rounds of one part per wavefront after
-  // staging its slab (a 512-column step of M = 8 rows costs about 0.15 rounds of one step)
-  float best = 0.f;
-  int best_pps = 0;
-  for (int pps = 1; pps <= pps_max; ++pps) {
-    const int nslab = (g.sk + pps - 1) / pps;
-    int wps = 256 / nslab;
-    wps = wps < 1 ? 1 : (wps > g.ntiles ? g.ntiles : wps);
-    const int tpw = (g.ntiles + wps - 1) / wps;
-    const float c = (float)((tpw * pps + GV_WAVES - 1) / GV_WAVES * g.spi) + 0.15f * (float)M / 8.f * (float)(pps * g.spi);
-    if (best_pps == 0 || c < best) { best = c; best_pps = pps; }
+  a.h.n = n; a.h.M = M; a.h.xdt = xdt; a.h.ydt = ydt;
+  long long total = 0;
+  int delta_cap = 0;
+  for (int i = 0; i < n; ++i) {
+    total += (long long)mats[i].ntiles * mats[i].nS;
+    delta_cap = delta_cap > M * (mats[i].m.N / 128 + 4) ? delta_cap : M * (mats[i].m.N / 128 + 4);
   }
-  a.g.sp = best_pps;
-  a.nslab = (g.sk + best_pps - 1) / best_pps;
-  a.wps = 256 / a.nslab;
-  a.wps = a.wps < 1 ? 1 : (a.wps > g.ntiles ? g.ntiles : a.wps);
-  a.tq = g.ntiles / a.wps; a.tr = g.ntiles % a.wps;
-  a.inv_wps = a.wps > 1 ? (uint32_t)(((1ull << 32) + a.wps - 1) / a.wps) : 0u;     // exact: workgroup index * wps < 2^32
-  a.g.inv_sp = (uint32_t)((65536 + best_pps - 1) / best_pps);
-  a.g.dq_t = GV_WAVES / best_pps; a.g.dq_p = GV_WAVES % best_pps;
-  const int cols = best_pps * g.spi * 512 < g.m.N ? best_pps * g.spi * 512 : g.m.N;
-  a.xq_cap = M * NDIG * (cols + X_PAD);
-  const size_t lds = (size_t)LUT_BYTES + ZERO_BYTES + a.xq_cap + (size_t)a.delta_cap * 4;
+  const size_t fixed = (size_t)LUT_BYTES + ZERO_BYTES + (size_t)delta_cap * 4 + (size_t)M * NDIG * X_PAD;
+  int xq_cap = 0, wg = 0, th = 0;
+  size_t off = 0;
+  for (int i = 0; i < n; ++i) {
+    GsMat& q = a.mat[i];
+    const GvMat& g = mats[i];
+    q.g = g;
+    q.part = (float*)(ws + off);
+    off += up256(split_part_bytes(g.ntiles, g.sk, M));
+    // this matrix's share of the 256 workgroups
+    int budget = (int)((long long)256 * g.ntiles * g.nS / total);
+    budget = budget < 1 ? 1 : budget;
+    const size_t per_part = (size_t)M * NDIG * g.spi * 512;
+    if (fixed + per_part > 160 * 1024) return CBK_ERR_UNSUPPORTED;
+    int pps_max = (int)((160 * 1024 - fixed) / per_part);
+    pps_max = pps_max < g.sk ? pps_max : g.sk;
+    // Parts per slab: a workgroup runs ceil(items / 16) rounds of one part per wavefront after
+    // staging its slab (a 512-column step of M = 8 rows costs about 0.15 rounds of one step)
+    float best = 0.f;
+    int best_pps = 0;
+    for (int pps = 1; pps <= pps_max; ++pps) {
+      const int nslab = (g.sk + pps - 1) / pps;
+      if (nslab > budget && pps < pps_max) continue;                // (more slabs than workgroups: longer slabs)
+      int wps = budget / nslab;
+      wps = wps < 1 ? 1 : (wps > g.ntiles ? g.ntiles : wps);
+      const int tpw = (g.ntiles + wps - 1) / wps;
+      const float c = (float)((tpw * pps + GV_WAVES - 1) / GV_WAVES * g.spi) + 0.15f * (float)M / 8.f * (float)(pps * g.spi);
+      if (best_pps == 0 || c < best) { best = c; best_pps = pps; }
+    }
+    q.g.sp = best_pps;
+    q.nslab = (g.sk + best_pps - 1) / best_pps;
+    q.wps = budget / q.nslab;
+    q.wps = q.wps < 1 ? 1 : (q.wps > g.ntiles ? g.ntiles : q.wps);
+    q.tq = g.ntiles / q.wps; q.tr = g.ntiles % q.wps;
+    q.inv_wps = q.wps > 1 ? (uint32_t)(((1ull << 32) + q.wps - 1) / q.wps) : 0u;   // exact: workgroup index * wps < 2^32
+    q.g.inv_sp = (uint32_t)((65536 + best_pps - 1) / best_pps);
+    q.g.dq_t = GV_WAVES / best_pps; q.g.dq_p = GV_WAVES % best_pps;
+    const int cols = best_pps * g.spi * 512 < g.m.N ? best_pps * g.spi * 512 : g.m.N;
+    xq_cap = xq_cap > M * NDIG * (cols + X_PAD) ? xq_cap : M * NDIG * (cols + X_PAD);
+    q.wg0 = wg; wg += q.nslab * q.wps; a.h.wg_end[i] = wg;
+    q.th0 = th; th += (g.ntiles * M * 16 + GS_RED_THREADS - 1) / GS_RED_THREADS * GS_RED_THREADS; a.h.th_end[i] = th;
+  }
+  for (int i = n; i < GV_MAX_BATCH; ++i) { a.h.wg_end[i] = 0x7fffffff; a.h.th_end[i] = 0x7fffffff; }
+  a.h.xq_cap = xq_cap; a.h.delta_cap = delta_cap;
+  const size_t lds = (size_t)LUT_BYTES + ZERO_BYTES + xq_cap + (size_t)delta_cap * 4;
   if (lds > 160 * 1024) return CBK_ERR_UNSUPPORTED;
-  const DMat& m = g.m;
+  const DMat& m = mats[0].m;
   const int keep = family_of(m.layout) == FAM_DENSE ? 0 : m.keep;
   const bool big = M > 4;
+  const int rb = th / GS_RED_THREADS;
   if (m.group != 128) return CBK_ERR_UNSUPPORTED;
-  if (m.bits == 4 && keep == 16) return big ? launch_split_cfg<4, 16, 128, 8>(a, lds, st) : launch_split_cfg<4, 16, 128, 4>(a, lds, st);
-  if (m.bits == 4 && keep == 0) return big ? launch_split_cfg<4, 0, 128, 8>(a, lds, st) : launch_split_cfg<4, 0, 128, 4>(a, lds, st);
-  if (m.bits == 2 && keep == 16) return big ? launch_split_cfg<2, 16, 128, 8>(a, lds, st) : launch_split_cfg<2, 16, 128, 4>(a, lds, st);
-  if (m.bits == 2 && keep == 0) return big ? launch_split_cfg<2, 0, 128, 8>(a, lds, st) : launch_split_cfg<2, 0, 128, 4>(a, lds, st);
+  if (m.bits == 4 && keep == 16) return big ? launch_split_cfg<4, 16, 128, 8>(a, lds, wg, rb, st) : launch_split_cfg<4, 16, 128, 4>(a, lds, wg, rb, st);
+  if (m.bits == 4 && keep == 0) return big ? launch_split_cfg<4, 0, 128, 8>(a, lds, wg, rb, st) : launch_split_cfg<4, 0, 128, 4>(a, lds, wg, rb, st);
+  if (m.bits == 2 && keep == 16) return big ? launch_split_cfg<2, 16, 128, 8>(a, lds, wg, rb, st) : launch_split_cfg<2, 16, 128, 4>(a, lds, wg, rb, st);
+  if (m.bits == 2 && keep == 0) return big ? launch_split_cfg<2, 0, 128, 8>(a, lds, wg, rb, st) : launch_split_cfg<2, 0, 128, 4>(a, lds, wg, rb, st);
   return CBK_ERR_UNSUPPORTED;
 }
 
@@ -1707,8 +1786,7 @@ static int launch_main_batch(GvBatch& gb, hipStream_t st) {
   // eight rows always fits).
   const size_t slot_bytes = (size_t)sk_cap * M * 16 * 4;
   const size_t fixed = (size_t)LUT_BYTES + ZERO_BYTES + CNT_BYTES + (size_t)delta_cap * 4;
-  const size_t red_floor = 2 * slot_bytes < 24 * 1024 ? 2 * slot_bytes : 24 * 1024;
-  const size_t x_budget = M == 1 ? (size_t)X_LDS_BUDGET : 160 * 1024 - fixed - red_floor;
+  const size_t x_budget = M == 1 ? (size_t)X_LDS_BUDGET : main_x_budget(M, delta_cap, sk_cap);
   for (int i = 0; i < n; ++i) {
     GvMat& g = gb.mat[i];
     const int N = g.m.N;
@@ -1776,64 +1854,50 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
     delta_cap = delta_cap > M * (m.N / 128 + 4) ? delta_cap : M * (m.N / 128 + 4);
   }
   const int blocks = gemv_blocks(gb, n, tiles);
-  // macro-steps per work item: about one and a half items per wavefront over the whole launch
-  // (the end of an item costs about as many instructions as a step; measured best between one
-  // and two); a tile is split into at most 16 parts, and into a power of two of them where the
-  // row is long enough: the items then spread evenly over the four SIMDs.  The parts depend on
-  // the matrices of the call only, not on M: they fix the order of every row's partial sums.
-  int spi = (int)((long long)cost * 2 / ((long long)blocks * GV_WAVES * 3));
-  spi = spi < 1 ? 1 : (spi > 8 ? 8 : spi);
+  // The parts depend on the matrices of the call only, not on M: they fix the order of every
+  // row's partial sums.
+  const int spi = launch_spi(cost, blocks);
   int sk_cap = 1;
   for (int i = 0; i < n; ++i) {
     GvMat& g = gb.mat[i];
-    int s = spi;
-    while ((g.nS + s - 1) / s > 16) ++s;
-    g.sk = (g.nS + s - 1) / s;
-    int p2 = 1;
-    while (p2 < g.sk) p2 <<= 1;
-    if (p2 <= 16 && p2 <= g.nS) g.sk = p2;
-    g.spi = (g.nS + g.sk - 1) / g.sk;                  // equal parts
-    g.sk = (g.nS + g.spi - 1) / g.spi;
+    row_parts(g.nS, spi, g.spi, g.sk);
     sk_cap = sk_cap > g.sk ? sk_cap : g.sk;
   }
-  // Long rows (at least SPLIT_MIN_STEPS macro-steps) whose digits do not fit the staging area go
-  // to the column-split kernel, one launch pair per matrix behind the others, where the
-  // configuration has one and the caller has left room for the part sums; otherwise the main
-  // kernel stages them slab by slab.
+  // Matrices for the column-split kernel (one launch pair for all of them, behind the others),
+  // where the configuration has one and the caller has left room for the part sums: rows whose
+  // digits do not fit the staging area of the main kernel, and, in launches of at most
+  // SPLIT_MAX_TILES tiles, rows whose digits take more than X_LDS_BUDGET of it (eight rows of 5376
+  // columns: every workgroup of the main kernel converts all of them before its first step and
+  // is left with four reduction slots; gate,up of that shape 43 us there, 30 + 5 us split).
+  // Otherwise the main kernel stages long rows slab by slab.
   const DMat& m0 = gb.mat[0].m;
   if (M > 1 && block_split_capable(m0.bits, family_of(m0.layout) == FAM_DENSE ? 0 : m0.keep, m0.group)) {
-    const size_t slot_bytes = (size_t)sk_cap * M * 16 * 4;
-    const size_t fixed = (size_t)LUT_BYTES + ZERO_BYTES + CNT_BYTES + (size_t)delta_cap * 4;
-    const size_t red_floor = 2 * slot_bytes < 24 * 1024 ? 2 * slot_bytes : 24 * 1024;
-    const size_t x_budget = 160 * 1024 - fixed - red_floor;
+    const size_t x_budget = main_x_budget(M, delta_cap, sk_cap);
+    auto splits = [&](const GvMat& g) {
+      const size_t digits = (size_t)M * NDIG * (g.m.N + X_PAD);
+      return digits > x_budget || (digits > (size_t)X_LDS_BUDGET && tiles <= SPLIT_MAX_TILES);
+    };
     GvMat split[GV_MAX_BATCH];
     int ns = 0;
     size_t need = 0;
     for (int i = 0; i < n; ++i) {
-      const GvMat& g = gb.mat[i];
-      if (g.nS >= SPLIT_MIN_STEPS && (size_t)M * NDIG * (g.m.N + X_PAD) > x_budget) {
-        split[ns++] = g;
-        need += up256(split_part_bytes(g.ntiles, g.sk, M));
+      if (splits(gb.mat[i])) {
+        split[ns++] = gb.mat[i];
+        need += up256(split_part_bytes(gb.mat[i].ntiles, gb.mat[i].sk, M));
       }
     }
     if (ns > 0 && workspace && !((uintptr_t)workspace & 15) && ws_bytes >= need) {
       int na = 0;
       for (int i = 0; i < n; ++i) {
-        const GvMat& g = gb.mat[i];
-        if (!(g.nS >= SPLIT_MIN_STEPS && (size_t)M * NDIG * (g.m.N + X_PAD) > x_budget)) gb.mat[na++] = g;
+        const GvMat g = gb.mat[i];
+        if (!splits(g)) gb.mat[na++] = g;
       }
       gb.h.n = na;
       if (na > 0) {
         const int rc = launch_main_batch(gb, st);
         if (rc != CBK_OK) return rc;
       }
-      size_t off = 0;
-      for (int i = 0; i < ns; ++i) {
-        const int rc = launch_split(split[i], M, xdt, ydt, (float*)((uint8_t*)workspace + off), st);
-        if (rc != CBK_OK) return rc;
-        off += up256(split_part_bytes(split[i].ntiles, split[i].sk, M));
-      }
-      return CBK_OK;
+      return launch_split_batch(split, ns, M, xdt, ydt, (uint8_t*)workspace, st);
     }
   }
   return launch_main_batch(gb, st);
