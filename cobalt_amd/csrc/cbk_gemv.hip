@@ -1580,9 +1580,11 @@ static inline size_t main_x_budget(int M, int delta_cap, int sk_cap) {
   return 160 * 1024 - fixed - red_floor;
 }
 
-// Rows whose digits (M * 3 * N bytes) stay within X_LDS_BUDGET need no workspace; longer ones (two
+// Rows whose digits (M * 3 * N bytes) stay within SPLIT_MIN_BYTES need no workspace; longer ones (two
 // to eight activation rows of a block-per-quarter configuration) are split over the workgroups by
 // columns when the caller provides room for the part sums: [tiles][parts <= 16][M][16] floats.
+constexpr size_t SPLIT_MIN_BYTES = 90 * 1024;  // digits of a row (M * 3 * N bytes) from which it is split (measured on both layer sets
+                                               // at 56, 72, 90 and 112 KB: six rows of 5376 and eight of 4096 columns gain, seven of 4096 lose)
 constexpr int SPLIT_MAX_TILES = 4096;          // (rows that fit are split only in launches of at most this many tiles)
 static inline int kernel_rows(const DMat& m, int M) {            // activation rows as the kernel counts them, per pass
   const int v = m.cs_rows == 2 ? 2 : 1;
@@ -1594,7 +1596,7 @@ size_t gemv_fast_workspace(const DMat& m, int M) {
   const int Mk = kernel_rows(m, M);
   if (Mk < 2 || !block_split_capable(m.bits, family_of(m.layout) == FAM_DENSE ? 0 : m.keep, m.group)) return 0;
   const size_t digits = (size_t)Mk * NDIG * (m.N + X_PAD);
-  if (digits <= (size_t)X_LDS_BUDGET) return 0;
+  if (digits <= SPLIT_MIN_BYTES) return 0;
   // what a call with this matrix alone would do
   const int ntiles = (m.K + 15) / 16, nS = (m.N / 128 + 3) / 4;
   int spi, sk;
@@ -1866,16 +1868,16 @@ int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, 
   // Matrices for the column-split kernel (one launch pair for all of them, behind the others),
   // where the configuration has one and the caller has left room for the part sums: rows whose
   // digits do not fit the staging area of the main kernel, and, in launches of at most
-  // SPLIT_MAX_TILES tiles, rows whose digits take more than X_LDS_BUDGET of it (eight rows of 5376
-  // columns: every workgroup of the main kernel converts all of them before its first step and
-  // is left with four reduction slots; gate,up of that shape 43 us there, 30 + 5 us split).
+  // SPLIT_MAX_TILES tiles, rows whose digits take more than SPLIT_MIN_BYTES of it (eight rows of
+  // 5376 columns: every workgroup of the main kernel converts all of them before its first step
+  // and is left with four reduction slots; gate,up of that shape 43 us there, 30 + 5 us split).
   // Otherwise the main kernel stages long rows slab by slab.
   const DMat& m0 = gb.mat[0].m;
   if (M > 1 && block_split_capable(m0.bits, family_of(m0.layout) == FAM_DENSE ? 0 : m0.keep, m0.group)) {
     const size_t x_budget = main_x_budget(M, delta_cap, sk_cap);
     auto splits = [&](const GvMat& g) {
       const size_t digits = (size_t)M * NDIG * (g.m.N + X_PAD);
-      return digits > x_budget || (digits > (size_t)X_LDS_BUDGET && tiles <= SPLIT_MAX_TILES);
+      return digits > x_budget || (digits > SPLIT_MIN_BYTES && tiles <= SPLIT_MAX_TILES);
     };
     GvMat split[GV_MAX_BATCH];
     int ns = 0;

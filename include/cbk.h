@@ -135,7 +135,7 @@ size_t cbk_stream_bytes(const cbk_desc* d, size_t sparse_data_bytes);
  * per col_scale vector, i.e. times cs_rows for a fused matrix, one float32 scale per activation
  * row and col_scale vector, plus float32 partial outputs when the library splits the column range
  * of a launch that would not fill the chip.  The decode kernels need none, with one optional use:
- * two to eight activation rows of rows whose activations take more than 112 KB of LDS
+ * two to eight activation rows of rows whose activations take more than 90 KB of LDS
  * (M * 3 * N bytes) are split over the workgroups by columns when there is room for the float32
  * part sums, K * 16 * M * 4 bytes at most; with a smaller workspace, or none, cbk_gemv computes
  * the same bits more slowly and reports no error.
