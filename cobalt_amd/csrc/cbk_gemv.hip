@@ -819,14 +819,16 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_mfma_kernel(GvBatch b) {
 }
 
 // ------------------------------------------------------------------ long rows, split over the workgroups by columns
-// Rows whose digits do not fit in LDS (M * 3 * N bytes: `down` projections at M >= 4).  The
-// kernel above stages such a row slab after slab in every workgroup, every workgroup converting
-// all M x N activations, with a handful of items per slab for its sixteen wavefronts.  Here a
-// workgroup owns one column slab (whole parts of the row, the parts of one activation row) of a
-// range of tiles: it stages M x (slab) activations once, deals the (tile, part) items of its slab
-// to the wavefronts and writes the part sums to a caller-provided buffer; a second small kernel
-// adds the parts of every output in part order.  Same operations in the same order as for one
-// activation row, so a row's result still does not depend on M.  Block-per-quarter arrangement only.
+// Two to eight activation rows of rows whose digits (M * 3 * N bytes) fill most of LDS or do not
+// fit (`down` projections from M = 2 on, 5376 columns from six rows on).  The kernel above has
+// every workgroup convert all M x N activations before its first step, and stages a row that
+// does not fit slab after slab, with a handful of items per slab for its sixteen wavefronts.
+// Here a workgroup owns one column slab (whole parts of the row, the parts of one activation
+// row) of a range of tiles of one matrix of the launch: it stages M x (slab) activations once,
+// deals the (tile, part) items of its slab to the wavefronts and writes the part sums to a
+// caller-provided buffer; a second small kernel adds the parts of every output in part order.
+// Same operations in the same order as for one activation row, so a row's result still does not
+// depend on M.  Block-per-quarter arrangement only.
 struct GsMat {             // one matrix of a column-split launch
   GvMat g;                 // spi, sk: the parts; sp: parts per slab
   int nslab, wps;          // column slabs, workgroups per slab
