@@ -190,6 +190,32 @@ def test_gemv_batch_matches_single_calls():
     assert torch.equal(ys[1], ops.gemv(pm3, xs[1], out_dtype=torch.float32))
 
 
+def test_gemv_batch_of_staged_and_column_split_matrices():
+    """One call over matrices of different row lengths at two to eight activation rows: the long
+    rows go to the column-split kernel (one launch for all of them), the others to the main kernel.
+    Every output against float64 on the dequantised weights, against one call per matrix (to
+    float32 rounding: a row's parts follow the launch), and row m of the batch at M rows against
+    the same batch at one row, bit for bit.  Eight long matrices fill the argument block."""
+    case = (F.BLK1632_4, 4, 128, 16)
+    for shapes in ([(40, 14336), (100, 4096), (16, 21504), (2000, 5376)], [(16 + 16 * i, 8192 + 1024 * i) for i in range(8)]):
+        pms = [F.synth_packed(K, N, *case[:3], case[3], seed=i, device=DEV).to_tiled() for i, (K, N) in enumerate(shapes)]
+        Ws = [ops.dequant(pm, torch.float32).double() for pm in pms]
+        for M in (8, 3):
+            xs = [acts(M, N, torch.bfloat16, seed=N + i).to(DEV) for i, (K, N) in enumerate(shapes)]
+            bs = [torch.randn(K, device=DEV) for K, N in shapes]
+            ys = ops.gemv_batch(pms, xs, biases=bs, out_dtype=torch.float32)
+            again = ops.gemv_batch(pms, xs, biases=bs, out_dtype=torch.float32)
+            rows = [ops.gemv_batch(pms, [x[i:i + 1] for x in xs], biases=bs, out_dtype=torch.float32) for i in range(M)]
+            for j, (pm, W, x, b, y, y2) in enumerate(zip(pms, Ws, xs, bs, ys, again)):
+                ref = x.double() @ W.t() + b.double()
+                assert float((y.double() - ref).abs().max() / ref.abs().max()) < 2e-5, (shapes[j], M)
+                single = ops.gemv(pm, x, bias=b, out_dtype=torch.float32)
+                assert float((y - single).abs().max() / single.abs().max()) < 1e-6, (shapes[j], M)
+                assert torch.equal(y, y2)
+                for i in range(M):
+                    assert torch.equal(rows[i][j][0], y[i]), (shapes[j], M, i)
+
+
 def test_gemv_output_dtypes_bias_and_strided_x():
     case = (F.BLK1632_4, 4, 128, 16)
     K, N = 128, 2048
