@@ -14,7 +14,9 @@ for a token in one graph (a replay boundary costs the GPU several microseconds).
 honoured exactly and inside such graphs: K // P replays of a graph of P steps (whole rotations over
 the distinct layer sets, about 32 steps) plus one replay of a graph holding the K % P steps that
 remain.  Warm-up is `--warmup` steps, and never less than 50 ms of replays (the first launches
-of a process run at a lower clock), both graphs included.  The JSON says what was replayed.
+of a process run at a lower clock), both graphs included; the start event of the timed region is
+enqueued behind one more untimed replay, so that the host's graph-launch latency stays outside
+the region (exactly K steps between the two events).  The JSON says what was replayed.
 
 `value` is algorithmic bytes (packed rows + scales + zeros + col_scale + activations in + outputs
 out) streamed per second.  `roofline` describes the decode kernel: algorithmic bytes per launch
@@ -157,11 +159,18 @@ class GraphTimer:
         n_warm = max(-(-warmup // self.per_graph), int(MIN_WARM_MS / t_replay) + 1)
         self._run(n_warm, rem)
         stream.synchronize()
+        # One more untimed replay goes out in front of the start event, with no synchronisation
+        # behind it: while the GPU runs it the host enqueues the event and the timed replays, so
+        # the host's graph-launch latency (tens of microseconds, several per cent of a 20-step
+        # region) does not sit inside the timed region.  The region itself is exactly `steps` steps.
+        lead = 1 if self.use_graph else 0
+        self._run(lead, 0)
         e0.record(stream)
         self._run(full, rem)
         e1.record(stream)
         stream.synchronize()
-        return {"ms_per_step": e0.elapsed_time(e1) / steps, "warmup_steps_run": (n_warm + 2) * self.per_graph + 2 * rem,
+        return {"ms_per_step": e0.elapsed_time(e1) / steps, "warmup_steps_run": (n_warm + 2 + lead) * self.per_graph + 2 * rem,
+                "untimed_lead_replays": lead,
                 "graph_replays_timed": (full + (1 if rem else 0)) if self.use_graph else 0,
                 "steps_per_full_graph": self.per_graph if self.use_graph else 0,
                 "steps_in_remainder_graph": rem if self.use_graph else 0}
