@@ -1047,7 +1047,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_split_kernel(GsArgs a) {
 }
 
 // the parts of every output, added in part order; bias; conversion
-constexpr int GS_RED_THREADS = 64;
+constexpr int GS_RED_THREADS = 256;
 __global__ __launch_bounds__(GS_RED_THREADS) void gemv_split_reduce_kernel(GsArgs a) {
   const GsHead& h = a.h;
   int idx = (int)blockIdx.x * GS_RED_THREADS + (int)threadIdx.x, mi = 0;
