@@ -1304,12 +1304,367 @@ static int launch_stream_m(const DMat& m, const void* x, int64_t ldx, int xdt, v
   return hipGetLastError() == hipSuccess ? CBK_OK : CBK_ERR_HIP;
 }
 
+// ------------------------------------------------------------------ survivor-stream rows on the matrix cores
+// SPARSE4X / SPARSE4E (a code offset per group in the row) in 16-row tiles on the 16x16x64 int8
+// MFMA, block-per-quarter arrangement: lane (weight row wr, quarter kq) decodes block kq of each
+// of the four groups of a 512-column step, one MFMA covers 64 columns of one group for up to four
+// activation rows, a second one the rows 4..7.  The rows of a tile have different lengths, so
+// every lane finds its codes itself: the group's mask words and code offset are loaded a step
+// ahead of the codes, whose address they give (survivors in the group's earlier blocks).  A lane
+// loads the mask words and the offset of one group (group 4S + kq), forms the nibble address of
+// each of its four blocks, and the four lanes of a weight row exchange what they hold with a
+// 4 x 4 transpose over the lane quarters (four row-swap instructions per register set).  Against
+// the row kernel above: the dot products and the digit reads of every activation row are gone
+// (about half the instructions at one activation row), and the time hardly grows with M.
+//
+// Work split: a workgroup takes a range of tiles; a tile's row is cut into SK parts of spi steps,
+// wavefront w of a round works on part w % SK of the round's tile w / SK; after the round the
+// part sums meet in LDS and are added in part order.  SK and spi depend on the matrix shape only,
+// and every activation row goes through the same operations in the same order whatever M is.
+// Reference semantics: cbk::gemv_sparse4 (src/cobaltkernel/csrc/cobalt_gemv.cuh:216-301).
+struct SmArgs {
+  DMat m;
+  const uint16_t* x;
+  int64_t ldx;
+  void* y;
+  int64_t ldy;
+  const void* bias;
+  int M, xdt, ydt;
+  int ntiles, tq, tr;      // tiles per workgroup: tq, one more for the first tr workgroups
+  int nS, spi, sk;         // steps per row, steps per part, parts
+  uint32_t inv_sk;         // w / sk = (w * inv_sk) >> 16 for w < 16
+  int hdr;                 // bytes of a row before its codes
+};
+struct SmMask { uint4 mk; uint32_t go; };                           // mask words and code offset of group 4S + kq
+struct SmCodes { uint32_t e[4][5]; uint32_t mw[4], sh[4]; uint32_t zs; };   // codes (16 bytes + skew), mask word, bit skew per group
+
+template <int NG>
+__global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const DMat& m = a.m;
+  const int M = a.M, N = m.N, NCH = N >> 7, Ns = N + X_PAD;
+  uint2* lut = (uint2*)smem;
+  uint8_t* zreg = smem + LUT_BYTES;
+  int8_t* xq = (int8_t*)zreg + ZERO_BYTES;
+  float* delta = (float*)(xq + (size_t)M * NDIG * Ns);
+  float* red = delta + M * (NCH + 4);                             // [2][M][16 wavefronts][16 rows]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wr = lane & 15, kq = lane >> 4;
+  const uint32_t l16 = lane & (LUT_LANES - 1);
+  const int bx = (int)blockIdx.x;
+  const int T_lo = bx * a.tq + (bx < a.tr ? bx : a.tr), T_hi = T_lo + a.tq + (bx < a.tr ? 1 : 0);
+  const int SK = a.sk, spi = a.spi, nS = a.nS;
+  const int TPR = GV_WAVES / SK;                                  // tiles per round (scalar, once)
+  const int R = (T_hi - T_lo + TPR - 1) / TPR;                    // rounds
+  const int tir = (int)(((uint32_t)wave * a.inv_sk) >> 16), part = wave - tir * SK;
+  const bool idle = tir >= TPR;                                   // wavefronts past the last whole tile of a round
+  const int s0 = part * spi, s1 = s0 + spi < nS ? s0 + spi : nS;  // this wavefront's steps (never empty: host)
+  const uint8_t* const m_data = m.data;
+  const uint32_t* const m_row_off = m.row_off;
+  const int m_K = m.K, m_G = m.G;
+  const uint32_t hdr = (uint32_t)a.hdr, go_off = (uint32_t)(N >> 3);
+
+  auto tile_of = [&](int round) { const int t = T_lo + round * TPR + (idle ? 0 : tir); return t < T_hi ? t : T_hi - 1; };
+  auto row_of = [&](int tile) { const int k = tile * 16 + wr; return k < m_K ? k : m_K - 1; };
+
+  // Positions (round, step) of this wavefront, in order; past the last one it repeats.  The row
+  // offsets of a round's tile are fetched a round ahead.
+  struct Pos { int round, S; uint32_t ro; };
+  uint32_t ro_next = m_row_off[row_of(tile_of(1 < R ? 1 : 0))];
+  auto advance = [&](Pos& p) {
+    if (p.S + 1 < s1) { ++p.S; return; }
+    if (p.round + 1 >= R) return;
+    ++p.round; p.S = s0; p.ro = ro_next;
+    ro_next = m_row_off[row_of(tile_of(p.round + 1 < R ? p.round + 1 : p.round))];
+  };
+  auto issue_mask = [&](const Pos& p, SmMask& k) {
+    const uint8_t* row = m_data + p.ro;
+    int g = 4 * p.S + kq;
+    g = g < m_G ? g : m_G - 1;                                      // groups past the row repeat the last one
+    k.mk = ((const uint4*)row)[g];
+    k.go = (uint32_t)((const uint16_t*)(row + go_off))[g];
+  };
+  // r0..r3 hold, in lane quarter q, the values (q, 0..3); afterwards register i holds (i, q):
+  // the upper two quarters of r0 / r1 change places with the lower two of r2 / r3, then the odd
+  // quarters of r0 / r2 with the even ones of r1 / r3.  (Inline assembly as in quarter_sum.)
+  auto transpose4 = [&](uint32_t& r0, uint32_t& r1, uint32_t& r2, uint32_t& r3) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(r0), "+v"(r2));
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(r1), "+v"(r3));
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(r0), "+v"(r1));
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(r2), "+v"(r3));
+  };
+  auto issue_codes = [&](const Pos& p, const SmMask& k, SmCodes& c) {
+    const uint32_t cbase = p.ro + hdr;                              // the row's codes (16-byte aligned)
+    // nibble address, in the row's codes, of the four blocks of this lane's group
+    const uint32_t n0 = 2u * k.go;
+    const uint32_t n1 = n0 + (uint32_t)__popc(k.mk.x), n2 = n1 + (uint32_t)__popc(k.mk.y), n3 = n2 + (uint32_t)__popc(k.mk.z);
+    uint32_t na[4] = {n0, n1, n2, n3};
+    c.mw[0] = k.mk.x; c.mw[1] = k.mk.y; c.mw[2] = k.mk.z; c.mw[3] = k.mk.w;
+    transpose4(c.mw[0], c.mw[1], c.mw[2], c.mw[3]);                 // now of block kq of the groups 4S .. 4S+3
+    transpose4(na[0], na[1], na[2], na[3]);
+#pragma unroll
+    for (int ci = 0; ci < 4; ++ci) {
+      c.sh[ci] = na[ci] << 2;                                       // (used modulo 32: the nibble inside the dword)
+      const uint32_t* cp = (const uint32_t*)(m_data + (cbase + ((na[ci] >> 1) & ~3u)));
+#pragma unroll
+      for (int i = 0; i < 5; ++i) c.e[ci][i] = cp[i];               // 16 bytes + skew; rows end in a readable tail
+    }
+    int g = 4 * p.S + kq;
+    g = g < m_G ? g : m_G - 1;
+    const size_t gi = (size_t)row_of(tile_of(p.round)) * m_G + g;
+    c.zs = (uint32_t)m.zero[gi] | ((uint32_t)m.scale[gi] << 8);    // of group 4S + kq; the other quarters fetch it from this lane
+  };
+
+  // role of this lane's row in the A operand: activation row a_m (+ 4 per row group), digit a_dig
+  // (digit 3 is an all-zero row); in the result, lane quarter kq holds the three digit sums of
+  // activation row kq (+ 4 per row group) for weight row wr
+  const int a_m = wr >> 2, a_dig = wr & 3;
+  const uint32_t xq_off = (uint32_t)((uint8_t*)xq - smem), z_off = (uint32_t)(zreg - smem);
+  bool a_on[NG];
+  uint32_t a_base[NG];
+  int dm[NG];
+#pragma unroll
+  for (int g = 0; g < NG; ++g) {
+    a_on[g] = a_dig < NDIG && a_m + 4 * g < M;
+    a_base[g] = xq_off + (uint32_t)(((a_m + 4 * g) * NDIG + a_dig) * Ns + kq * 32);
+    dm[g] = kq + 4 * g < M ? kq + 4 * g : 0;
+  }
+
+  float ysum[4 * NG];
+#pragma unroll
+  for (int i = 0; i < 4 * NG; ++i) ysum[i] = 0.f;
+
+  // the part sums of a round, added in part order; all threads, after the round's barrier
+  auto finish_round = [&](int round) {
+    const float* rb = red + (size_t)(round & 1) * M * 256;
+    for (int o = tid; o < M * 256; o += GV_THREADS) {
+      const int r = o & 15, t = (o >> 4) & 15, am = o >> 8;
+      const int tile = T_lo + round * TPR + t;
+      const int k = tile * 16 + r;
+      if (t >= TPR || tile >= T_hi || k >= m_K) continue;
+      float pv[16];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) pv[j] = rb[(am * 16 + t * SK + (j < SK ? j : SK - 1)) * 16 + r];
+      float v = 0.f;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) v += j < SK ? pv[j] : 0.f;
+      if (a.bias) v += (a.ydt == CBK_F32) ? ((const float*)a.bias)[k]
+                     : (a.ydt == CBK_F16) ? h2f(((const uint16_t*)a.bias)[k]) : bf2f(((const uint16_t*)a.bias)[k]);
+      const size_t oi = (size_t)am * a.ldy + k;
+      if (a.ydt == CBK_F32) ((float*)a.y)[oi] = v;
+      else if (a.ydt == CBK_F16) ((uint16_t*)a.y)[oi] = f2h(v);
+      else ((uint16_t*)a.y)[oi] = f2bf(v);
+    }
+  };
+
+  auto compute = [&](const Pos& p, const SmCodes& c) {
+    const int S = p.S;
+    uint32_t zs[4];
+#pragma unroll
+    for (int ci = 0; ci < 4; ++ci) zs[ci] = (uint32_t)__shfl((int)c.zs, wr + 16 * ci, 64);
+#pragma unroll
+    for (int ci = 0; ci < 4; ++ci) {
+      const int chunk = 4 * S + ci;
+      uint32_t aaddr[NG];
+#pragma unroll
+      for (int g = 0; g < NG; ++g) aaddr[g] = (a_on[g] && chunk < NCH) ? a_base[g] + (uint32_t)chunk * 128u : z_off;
+      uint32_t w[4];                                                // the block's codes from bit 0 on
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w[i] = __builtin_amdgcn_alignbit(c.e[ci][i + 1], c.e[ci][i], c.sh[ci]);
+      const uint32_t mw = c.mw[ci];
+      uint32_t mb[4], rk[4];
+      mb[0] = mw & 0xFFu; mb[1] = __builtin_amdgcn_ubfe(mw, 8, 8); mb[2] = __builtin_amdgcn_ubfe(mw, 16, 8); mb[3] = mw >> 24;
+      rk[1] = (uint32_t)__popc(mb[0]);                              // <= 8
+      rk[2] = rk[1] + (uint32_t)__popc(mb[1]);                      // <= 16
+      rk[3] = rk[2] + (uint32_t)__popc(mb[2]);                      // <= 24
+      uint2 sel[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) sel[j] = lut[mb[j] * LUT_LANES + l16];
+      // 32 bits of the stream from nibble rk[j] on
+      uint32_t win[4];
+      win[0] = w[0];
+      win[1] = (uint32_t)((((uint64_t)w[1] << 32) | w[0]) >> (4u * rk[1]));
+      {
+        const uint32_t r = rk[2];                                   // dwords r / 8 and r / 8 + 1 of w[0..3], r / 8 <= 2
+        const uint32_t m8 = (uint32_t)__builtin_amdgcn_sbfe((int)r, 3, 1), m16 = (uint32_t)__builtin_amdgcn_sbfe((int)r, 4, 1);
+        const uint32_t lo = mask_select(m16, mask_select(m8, w[0], w[1]), w[2]);
+        const uint32_t hi = mask_select(m16, mask_select(m8, w[1], w[2]), w[3]);
+        win[2] = __builtin_amdgcn_alignbit(hi, lo, r * 4u);
+      }
+      {
+        const uint32_t r = rk[3];                                   // r / 8 <= 3, and a shift of 0 at r = 24
+        const uint32_t m8 = (uint32_t)__builtin_amdgcn_sbfe((int)r, 3, 1), m16 = (uint32_t)__builtin_amdgcn_sbfe((int)r, 4, 1);
+        const uint32_t lo = mask_select(m16, mask_select(m8, w[0], w[1]), mask_select(m8, w[2], w[3]));
+        const uint32_t hi = mask_select(m16, mask_select(m8, w[1], w[2]), w[3] & ~m8);
+        win[3] = __builtin_amdgcn_alignbit(hi, lo, r * 4u);
+      }
+      const uint32_t nz = 0x80808080u - (zs[ci] & 0xFFu) * 0x01010101u;
+      v4i acc[NG];
+#pragma unroll
+      for (int g = 0; g < NG; ++g) acc[g] = (v4i){0, 0, 0, 0};
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        uint32_t bfrag[4];
+#pragma unroll
+        for (int jj2 = 0; jj2 < 2; ++jj2) {
+          const int jj = 2 * half + jj2;
+          const uint32_t p0 = bias_pool(win[jj] & 0x0F0F0F0Fu, nz), p1 = bias_pool((win[jj] >> 4) & 0x0F0F0F0Fu, nz);
+          bfrag[2 * jj2] = perm(p1, p0, sel[jj].x);                 // q - zero of columns 0-3 of the mask byte; pruned: 0
+          bfrag[2 * jj2 + 1] = perm(p1, p0, sel[jj].y);             // columns 4-7
+        }
+        const v4i bv = (v4i){(int)bfrag[0], (int)bfrag[1], (int)bfrag[2], (int)bfrag[3]};
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+          const v4i av = *(const v4i*)(smem + aaddr[g] + 16 * half);
+          acc[g] = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bv, acc[g], 0, 0, 0);
+          asm("s_nop 1" : "+v"(acc[g]));                            // as in the kernels above
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const float dl = delta[dm[g] * (NCH + 4) + chunk];          // 0 past the last chunk
+        const float f = fmaf((float)(acc[g][0] * 256 + acc[g][1]), 256.f, (float)acc[g][2]);
+        ysum[4 * g + ci] = fmaf(f, h2f((uint16_t)(zs[ci] >> 8)) * dl, ysum[4 * g + ci]);
+      }
+    }
+    if (S + 1 == s1) {                                              // the item is done
+      float* rb = red + (size_t)(p.round & 1) * M * 256;
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const int q = 4 * g;
+        const float ps = (ysum[q] + ysum[q + 1]) + (ysum[q + 2] + ysum[q + 3]);
+        if (kq + 4 * g < M) rb[((kq + 4 * g) * 16 + wave) * 16 + wr] = ps;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ysum[q + i] = 0.f;
+      }
+      __syncthreads();
+      finish_round(p.round);
+    }
+  };
+
+  // ---- the first loads (row offsets, then mask words), then selector table and activation digits
+  Pos pc{0, s0, m_row_off[row_of(tile_of(0))]};
+  SmMask mk;
+  SmCodes ca, cb;                                                  // swap roles by name (a copy would wait for the loads)
+  issue_mask(pc, mk);
+  if (tid < 256) {
+    const uint2 e = make_selectors((uint32_t)tid, 0);
+#pragma unroll
+    for (int j = 0; j < LUT_LANES; ++j) lut[tid * LUT_LANES + j] = e;
+  } else if (tid < 256 + ZERO_BYTES / 4) {
+    ((uint32_t*)zreg)[tid - 256] = 0u;
+  }
+  const int n16 = N >> 4, xitems = M * n16;                        // a multiple of 8
+  for (int it = tid; it < xitems; it += GV_THREADS) {
+    XLoad xl;
+    stage_load(a.x, a.ldx, m.cs, N, 0, n16, it, false, 0, xl);
+    stage_convert<0>(xl, m.cs != nullptr, a.xdt, N, 0, n16, it, false, xq, delta, X_PAD);
+  }
+  __syncthreads();
+  if (idle) {                                                      // (uniform over the wavefront) no item, every barrier
+    for (int round = 0; round < R; ++round) {
+      __syncthreads();
+      finish_round(round);
+    }
+    return;
+  }
+  issue_codes(pc, mk, ca);
+  Pos pb = pc;                                                     // position whose codes are fetched next
+  advance(pb);
+  issue_mask(pb, mk);
+  Pos pa = pb;                                                     // position whose mask words are being fetched
+  const int total = R * (s1 - s0);
+  for (int q = 0; q < total; q += 2) {
+    issue_codes(pb, mk, cb);
+    advance(pa);
+    issue_mask(pa, mk);
+    compute(pc, ca);
+    pc = pb; pb = pa;
+    if (q + 1 >= total) break;
+    issue_codes(pb, mk, ca);
+    advance(pa);
+    issue_mask(pa, mk);
+    compute(pc, cb);
+    pc = pb; pb = pa;
+  }
+}
+
+constexpr int STREAM_MFMA_MIN_STEPS = 3072;     // tile-steps (16 rows x 512 columns) from which the matrix-core kernel is used
+
+template <int NG>
+static int launch_stream_mfma_ng(const SmArgs& a, size_t lds, int blocks, hipStream_t st) {
+  auto kern = gemv_stream_mfma_kernel<NG>;
+  static std::atomic<int> configured{0};
+  if (!configured.load(std::memory_order_acquire)) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
+      return CBK_ERR_HIP;
+    configured.store(1, std::memory_order_release);
+  }
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(GV_THREADS), lds, st, a);
+  return hipGetLastError() == hipSuccess ? CBK_OK : CBK_ERR_HIP;
+}
+
+// LDS of the kernel for mp activation rows of N columns
+static inline size_t stream_mfma_lds(int N, int mp) {
+  return (size_t)LUT_BYTES + ZERO_BYTES + (size_t)mp * NDIG * (N + X_PAD) + (size_t)mp * (N / 128 + 4) * 4 + (size_t)2 * mp * 256 * 4;
+}
+
+// CBK_ERR_UNSUPPORTED: not a case of this kernel.
+static int launch_gemv_stream_mfma(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
+                                   const void* bias, hipStream_t st) {
+  if (m.layout != CBK_SPARSE4X && m.layout != CBK_SPARSE4E) return CBK_ERR_UNSUPPORTED;
+  if (m.N % 128 != 0 || m.K < 1) return CBK_ERR_UNSUPPORTED;
+  int mc = GV_MAX_M;                                                // activation rows per pass: what fits in LDS
+  while (mc > 0 && stream_mfma_lds(m.N, mc) > (size_t)160 * 1024) --mc;
+  if (mc == 0) return CBK_ERR_UNSUPPORTED;
+  SmArgs a;
+  a.m = m; a.ldx = ldx; a.ldy = ldy; a.bias = bias; a.xdt = xdt; a.ydt = ydt;
+  a.ntiles = (m.K + 15) / 16;
+  // Below three quarters of a step per wavefront of the GPU the row kernel is faster at one
+  // activation row (4096 x 4096: 8.8 against 12.2 us; 6144 x 4096: 12.7 against 12.3 us).  By the
+  // shape alone: which kernel runs must not depend on M, or a row's result would.
+  if ((long long)a.ntiles * ((m.N / 128 + 3) / 4) < STREAM_MFMA_MIN_STEPS) return CBK_ERR_UNSUPPORTED;
+  const int blocks = a.ntiles < 256 ? a.ntiles : 256;               // one persistent workgroup per CU
+  a.tq = a.ntiles / blocks; a.tr = a.ntiles % blocks;
+  a.nS = (m.N / 128 + 3) / 4;
+  a.hdr = ((m.N >> 3) + ((m.G * 2 + 15) & ~15) + 15) & ~15;
+  // Parts per tile: all sixteen wavefronts of a workgroup should have an item, in as few rounds
+  // of as few steps as possible (a round costs about a step and a half beside its steps); no
+  // part may be empty.
+  const int tmax = a.tq + (a.tr ? 1 : 0);
+  float best = 0.f;
+  a.sk = 1; a.spi = a.nS;
+  for (int sk = 1; sk <= GV_WAVES && sk <= a.nS; ++sk) {
+    const int spi = (a.nS + sk - 1) / sk;
+    if ((sk - 1) * spi >= a.nS) continue;
+    const int tpr = GV_WAVES / sk, rounds = (tmax + tpr - 1) / tpr;
+    const float c = (float)rounds * ((float)spi + 1.5f);
+    if (sk == 1 || c < best) { best = c; a.sk = sk; a.spi = spi; }
+  }
+  a.inv_sk = (uint32_t)((65536 + a.sk - 1) / a.sk);
+  for (int m0 = 0; m0 < M; m0 += mc) {
+    const int mp = M - m0 < mc ? M - m0 : mc;
+    a.x = (const uint16_t*)x + (size_t)m0 * ldx;
+    a.y = (uint8_t*)y + (size_t)m0 * ldy * (ydt == CBK_F32 ? 4 : 2);
+    a.M = mp;
+    const size_t lds = stream_mfma_lds(m.N, mp);
+    const int rc = mp > 4 ? launch_stream_mfma_ng<2>(a, lds, blocks, st) : launch_stream_mfma_ng<1>(a, lds, blocks, st);
+    if (rc) return rc;
+  }
+  return CBK_OK;
+}
+
 // CBK_ERR_UNSUPPORTED: not a case of this kernel (the caller falls back on the float row kernel).
 int launch_gemv_stream(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
                        const void* bias, hipStream_t st) {
   if (family_of(m.layout) != FAM_SPARSE || m.bits != 4 || m.group != 128 || m.cs_rows > 1) return CBK_ERR_UNSUPPORTED;
   if (!(m.flags & CBK_FLAG_ZERO_LE_128)) return CBK_ERR_UNSUPPORTED;
   if (xdt != CBK_F16 && xdt != CBK_BF16T) return CBK_ERR_DTYPE;
+  {
+    const int rc = launch_gemv_stream_mfma(m, x, xdt, M, ldx, y, ydt, ldy, bias, st);   // the layouts with group offsets
+    if (rc != CBK_ERR_UNSUPPORTED) return rc;
+  }
   if ((size_t)NDIG * m.N > (size_t)ST_X_BUDGET) return CBK_ERR_UNSUPPORTED;
   int mc = (int)((size_t)ST_X_BUDGET / ((size_t)NDIG * m.N));      // activation rows per pass
   mc = mc > ST_MAX_M ? ST_MAX_M : mc;

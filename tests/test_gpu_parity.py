@@ -142,6 +142,38 @@ def test_gemv_integer_dot_row_kernels(case):
                 assert torch.equal(y1[0], y[M - 1]), (case_id(case), K, N, M)
 
 
+@pytest.mark.parametrize("shape", [(49200, 128), (24600, 640), (1768, 14336), (6160, 4096)], ids=lambda s: f"{s[0]}x{s[1]}")
+def test_gemv_survivor_streams_on_matrix_cores(shape):
+    """SPARSE4X / SPARSE4E from 3072 tile-steps (16 rows x 512 columns) on: the 16-row matrix-core
+    kernel for rows of different lengths.  One step per row and thirteen rounds of sixteen tiles
+    (49200 x 128), a last step with one group of four (640 columns), one tile per workgroup cut
+    into fourteen parts with two wavefronts idle (14336 columns, two activation rows per pass), two
+    tiles per round (6160 x 4096); a last tile of fewer than sixteen rows in each.  One to nine
+    activation rows, both activation types, a bias, run-to-run identical, and a row's result does
+    not depend on how many rows the call has."""
+    K, N = shape
+    for case in ([(F.SPARSE4X, 4, 128, 0), (F.SPARSE4E, 4, 128, 0)] if N == 640 else [(F.SPARSE4X, 4, 128, 0)]):
+        raw = make_raw(case, K, N, seed=K + N + case[0])
+        pk = oracle_pack(case, raw)
+        pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV)
+        W = R.dequant(pk, K, N, case[0], col_scale=raw["col_scale"], **kw_of(case))
+        bias = acts(1, K, torch.float32, seed=K)[0]
+        for M, dtype in ((1, torch.float16), (2, torch.bfloat16), (4, torch.float16), (5, torch.bfloat16), (8, torch.float16),
+                         (9, torch.float16)):
+            x = acts(M, N, dtype, seed=M + N)
+            ref = R.forward_ref(W, _np(x))
+            y = ops.gemv(pm, x.to(DEV), out_dtype=torch.float32)
+            assert rel_fro(_np(y), ref) < 1e-5, (case_id(case), K, N, M)
+            assert np.abs(_np(y) - ref).max() / np.abs(ref).max() < 2e-5
+            assert torch.equal(ops.gemv(pm, x.to(DEV), out_dtype=torch.float32), y)
+            y1 = ops.gemv(pm, x[M - 1:M].to(DEV), out_dtype=torch.float32)
+            assert torch.equal(y1[0], y[M - 1]), (case_id(case), K, N, M)
+            if M in (1, 8):
+                yb = ops.gemv(pm, x.to(DEV), bias=bias.to(DEV), out_dtype=dtype)
+                want = (y + bias.to(DEV).to(dtype).float()[None, :]).to(dtype)      # (the bias has the output's type)
+                assert torch.equal(yb, want), (case_id(case), K, N, M)
+
+
 ALL_MFMA_CASES = [(F.BLKC, b, g, k) for b in (2, 3, 4) for g in (64, 128) for k in (10, 16, 23)] + \
                  [(F.DENSEB, b, g, 0) for b in (2, 3, 4) for g in (64, 128)]
 
