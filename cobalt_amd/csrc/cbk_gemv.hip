@@ -1408,7 +1408,12 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) 
       c.sh[ci] = na[ci] << 2;                                       // (used modulo 32: the nibble inside the dword)
       const uint32_t* cp = (const uint32_t*)(m_data + (cbase + ((na[ci] >> 1) & ~3u)));
 #pragma unroll
-      for (int i = 0; i < 5; ++i) c.e[ci][i] = cp[i];               // 16 bytes + skew; rows end in a readable tail
+      for (int i = 0; i < 4; ++i) c.e[ci][i] = cp[i];               // rows end in a readable tail
+      // A fifth dword only where the block's survivors reach into it (more than 25 of 32 kept, or
+      // fewer behind a skew): as a second load of the cache line the first one has just
+      // requested it would wait in the cache for that line, and every wavefront behind it.
+      c.e[ci][4] = 0u;
+      if ((na[ci] & 7u) + (uint32_t)__popc(c.mw[ci]) > 32u) c.e[ci][4] = cp[4];
     }
     int g = 4 * p.S + kq;
     g = g < m_G ? g : m_G - 1;
@@ -1463,6 +1468,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) 
     uint32_t zs[4];
 #pragma unroll
     for (int ci = 0; ci < 4; ++ci) zs[ci] = (uint32_t)__shfl((int)c.zs, wr + 16 * ci, 64);
+    // (uniform over the wavefront: in the last round a wavefront may be left without a tile; it
+    // has loaded the last tile again, multiplies nothing and goes on to the round's barrier)
+    if (T_lo + p.round * TPR + tir < T_hi)
 #pragma unroll
     for (int ci = 0; ci < 4; ++ci) {
       const int chunk = 4 * S + ci;
@@ -1643,6 +1651,7 @@ static int launch_gemv_stream_mfma(const DMat& m, const void* x, int xdt, int M,
     if (sk == 1 || c < best) { best = c; a.sk = sk; a.spi = spi; }
   }
   a.inv_sk = (uint32_t)((65536 + a.sk - 1) / a.sk);
+  mc = (M + (M + mc - 1) / mc - 1) / ((M + mc - 1) / mc);            // the same number of passes, of equal size
   for (int m0 = 0; m0 < M; m0 += mc) {
     const int mp = M - m0 < mc ? M - m0 : mc;
     a.x = (const uint16_t*)x + (size_t)m0 * ldx;
