@@ -1598,7 +1598,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) 
   }
 }
 
-constexpr int STREAM_MFMA_MIN_STEPS = 3072;     // tile-steps (16 rows x 512 columns) from which the matrix-core kernel is used
+constexpr int STREAM_MFMA_MIN_STEPS = 1536;     // tile-steps (16 rows x 512 columns) from which the matrix-core kernel is used
 
 template <int NG>
 static int launch_stream_mfma_ng(const SmArgs& a, size_t lds, int blocks, hipStream_t st) {
@@ -1629,17 +1629,23 @@ static int launch_gemv_stream_mfma(const DMat& m, const void* x, int xdt, int M,
   SmArgs a;
   a.m = m; a.ldx = ldx; a.ldy = ldy; a.bias = bias; a.xdt = xdt; a.ydt = ydt;
   a.ntiles = (m.K + 15) / 16;
-  // Below three quarters of a step per wavefront of the GPU the row kernel is faster at one
-  // activation row (4096 x 4096: 8.8 against 12.2 us; 6144 x 4096: 12.7 against 12.3 us).  By the
-  // shape alone: which kernel runs must not depend on M, or a row's result would.
+  // Small matrices stay on the row kernel, which is faster there at one activation row
+  // (4096 x 2048, 1024 tile-steps: 6.6 against 8.3 us; 2048 x 4096: 8.4 against 8.8 us, but 12.2
+  // against 10.1 us at M = 4; 4096 x 4096, 2048 tile-steps: 8.8 / 13.0 / 19.4 us at M = 1 / 4 / 8
+  // against 9.2 / 10.7 / 15.1 us here; 1024 x 14336, 1792: 17.8 against 15.7 us at M = 1).  By
+  // the shape alone: which kernel runs must not depend on M, or a row's result would.
   if ((long long)a.ntiles * ((m.N / 128 + 3) / 4) < STREAM_MFMA_MIN_STEPS) return CBK_ERR_UNSUPPORTED;
   const int blocks = a.ntiles < 256 ? a.ntiles : 256;               // one persistent workgroup per CU
   a.tq = a.ntiles / blocks; a.tr = a.ntiles % blocks;
   a.nS = (m.N / 128 + 3) / 4;
   a.hdr = ((m.N >> 3) + ((m.G * 2 + 15) & ~15) + 15) & ~15;
-  // Parts per tile: all sixteen wavefronts of a workgroup should have an item, in as few rounds
-  // of as few steps as possible (a round costs about a step and a half beside its steps); no
-  // part may be empty.
+  // Parts per tile: as few steps per wavefront as possible, and few tiles per round.  With one
+  // or two tiles in a round the sixteen wavefronts read the same 16 or 32 rows side by side: the
+  // cache lines of their offsets, scales and zero points (64 groups or more each) and of their
+  // mask words and codes serve several wavefronts before they are displaced, and a step is
+  // 15-25 % faster (65536 x 4096 at M = 1: 49.0 us with sixteen tiles in one round, 44.1 us with
+  // two in each of eight rounds; 32768 x 8192: 49.8 / 49.0 / 45.2 us with eight / two / one).  A
+  // round costs about an eighth of a step beside its steps.  No part may be empty.
   const int tmax = a.tq + (a.tr ? 1 : 0);
   float best = 0.f;
   a.sk = 1; a.spi = a.nS;
@@ -1647,7 +1653,7 @@ static int launch_gemv_stream_mfma(const DMat& m, const void* x, int xdt, int M,
     const int spi = (a.nS + sk - 1) / sk;
     if ((sk - 1) * spi >= a.nS) continue;
     const int tpr = GV_WAVES / sk, rounds = (tmax + tpr - 1) / tpr;
-    const float c = (float)rounds * ((float)spi + 1.5f);
+    const float c = (float)rounds * ((float)spi * (tpr == 1 ? 0.75f : tpr == 2 ? 0.85f : 1.f) + 0.12f);
     if (sk == 1 || c < best) { best = c; a.sk = sk; a.spi = spi; }
   }
   a.inv_sk = (uint32_t)((65536 + a.sk - 1) / a.sk);

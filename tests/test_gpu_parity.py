@@ -144,7 +144,7 @@ def test_gemv_integer_dot_row_kernels(case):
 
 @pytest.mark.parametrize("shape", [(49200, 128), (24600, 640), (1768, 14336), (6160, 4096)], ids=lambda s: f"{s[0]}x{s[1]}")
 def test_gemv_survivor_streams_on_matrix_cores(shape):
-    """SPARSE4X / SPARSE4E from 3072 tile-steps (16 rows x 512 columns) on: the 16-row matrix-core
+    """SPARSE4X / SPARSE4E from 1536 tile-steps (16 rows x 512 columns) on: the 16-row matrix-core
     kernel for rows of different lengths.  One step per row and thirteen rounds of sixteen tiles
     (49200 x 128), a last step with one group of four (640 columns), one tile per workgroup cut
     into fourteen parts with two wavefronts idle (14336 columns, two activation rows per pass), two
