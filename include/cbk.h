@@ -85,8 +85,10 @@ enum cbk_status {
  *             matrix-core decode kernel needs q - zero to fit a signed byte; without the flag
  *             cbk_gemv runs the slower float row kernel, which takes any uint8 zero point.
  *             (The matrix-core kernels take layouts 1, 6, 7, 8, 9 with 2/3/4-bit codes, or 6-bit
- *             for layout 7; SPARSE4/4X/4E and DENSE8 decode with integer-dot row kernels of their
- *             own, 8-bit prefill goes through the generic tile reader.)
+ *             for layout 7; SPARSE4X/4E decode on the matrix cores too, 16 rows of different
+ *             lengths at a time, SPARSE4, small stream matrices and DENSE8 with integer-dot row
+ *             kernels of their own, all of them with the flag only; 8-bit prefill goes through
+ *             the generic tile reader.)
  *             CBK_FLAG_TILED16: data / scale / zero are in 16-row tile-interleaved order, a
  *             permutation of the same bytes made once at load time so that the sixteen rows a
  *             wavefront decodes together are contiguous in HBM: with s = cbk_row_stride(),
