@@ -1494,20 +1494,18 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) 
       win[0] = w[0];
       win[1] = (uint32_t)((((uint64_t)w[1] << 32) | w[0]) >> (4u * rk[1]));
       {
-        const uint32_t r = rk[2];                                   // dwords r / 8 and r / 8 + 1 of w[0..3], r / 8 <= 2
+        // the 64 bits from nibble rk[2] (<= 16) on: dwords r / 8 .. r / 8 + 2 of w[0..3], then the
+        // window of the fourth mask byte is those 64 bits shifted by the third byte's survivors
+        const uint32_t r = rk[2];
         const uint32_t m8 = (uint32_t)__builtin_amdgcn_sbfe((int)r, 3, 1), m16 = (uint32_t)__builtin_amdgcn_sbfe((int)r, 4, 1);
-        const uint32_t lo = mask_select(m16, mask_select(m8, w[0], w[1]), w[2]);
-        const uint32_t hi = mask_select(m16, mask_select(m8, w[1], w[2]), w[3]);
-        win[2] = __builtin_amdgcn_alignbit(hi, lo, r * 4u);
+        const uint32_t d0 = mask_select(m16, mask_select(m8, w[0], w[1]), w[2]);
+        const uint32_t d1 = mask_select(m16, mask_select(m8, w[1], w[2]), w[3]);
+        const uint32_t d2 = mask_select(m8, w[2], w[3]) & ~m16;
+        win[2] = __builtin_amdgcn_alignbit(d1, d0, r * 4u);
+        const uint32_t h1 = __builtin_amdgcn_alignbit(d2, d1, r * 4u);
+        win[3] = (uint32_t)((((uint64_t)h1 << 32) | win[2]) >> (4u * (rk[3] - rk[2])));
       }
-      {
-        const uint32_t r = rk[3];                                   // r / 8 <= 3, and a shift of 0 at r = 24
-        const uint32_t m8 = (uint32_t)__builtin_amdgcn_sbfe((int)r, 3, 1), m16 = (uint32_t)__builtin_amdgcn_sbfe((int)r, 4, 1);
-        const uint32_t lo = mask_select(m16, mask_select(m8, w[0], w[1]), mask_select(m8, w[2], w[3]));
-        const uint32_t hi = mask_select(m16, mask_select(m8, w[1], w[2]), w[3] & ~m8);
-        win[3] = __builtin_amdgcn_alignbit(hi, lo, r * 4u);
-      }
-      const uint32_t nz = 0x80808080u - (zs[ci] & 0xFFu) * 0x01010101u;
+      const uint32_t nz = 0x80808080u - perm(0u, zs[ci], 0x00000000u);      // (the zero point in every byte)
       v4i acc[NG];
 #pragma unroll
       for (int g = 0; g < NG; ++g) acc[g] = (v4i){0, 0, 0, 0};
