@@ -1318,8 +1318,9 @@ static int launch_stream_m(const DMat& m, const void* x, int64_t ldx, int xdt, v
 // (about half the instructions at one activation row), and the time hardly grows with M.
 //
 // Work split: a workgroup takes a range of tiles; a tile's row is cut into SK parts of spi steps,
-// wavefront w of a round works on part w % SK of the round's tile w / SK; after the round the
-// part sums meet in LDS and are added in part order.  SK and spi depend on the matrix shape only,
+// wavefront w of a round works on part w % SK of the round's tile w / SK; the part sums meet in
+// LDS and are added in part order: by the wavefront that finishes a tile's round last, or (BAR,
+// used for one activation row, where it measured faster) by all threads behind a barrier.  SK and spi depend on the matrix shape only,
 // and every activation row goes through the same operations in the same order whatever M is.
 // Reference semantics: cbk::gemv_sparse4 (src/cobaltkernel/csrc/cobalt_gemv.cuh:216-301).
 struct SmArgs {
@@ -1338,16 +1339,18 @@ struct SmArgs {
 struct SmMask { uint4 mk; uint32_t go; };                           // mask words and code offset of group 4S + kq
 struct SmCodes { uint32_t e[4][5]; uint32_t mw[4], sh[4]; uint32_t zs; };   // codes (16 bytes + skew), mask word, bit skew per group
 
-template <int NG>
+template <int NG, bool BAR>
 __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const DMat& m = a.m;
   const int M = a.M, N = m.N, NCH = N >> 7, Ns = N + X_PAD;
   uint2* lut = (uint2*)smem;
   uint8_t* zreg = smem + LUT_BYTES;
-  int8_t* xq = (int8_t*)zreg + ZERO_BYTES;
+  int* arrived = (int*)(zreg + ZERO_BYTES);                       // [2][16] part sums written, by round parity and tile of the round
+  int* summed = arrived + 2 * GV_WAVES;                           // [16] rounds whose part sums have been added
+  int8_t* xq = (int8_t*)zreg + ZERO_BYTES + CNT_BYTES;
   float* delta = (float*)(xq + (size_t)M * NDIG * Ns);
-  float* red = delta + M * (NCH + 4);                             // [2][M][16 wavefronts][16 rows]
+  float* red = delta + M * (NCH + 4);                             // [2][M][16 wavefronts][16 rows], by round parity
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wr = lane & 15, kq = lane >> 4;
@@ -1440,7 +1443,29 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) 
 #pragma unroll
   for (int i = 0; i < 4 * NG; ++i) ysum[i] = 0.f;
 
-  // the part sums of a round, added in part order; all threads, after the round's barrier
+  auto emit = [&](int am, int k, float v) {
+    const size_t oi = (size_t)am * a.ldy + k;
+    if (a.ydt == CBK_F32) ((float*)a.y)[oi] = v;
+    else if (a.ydt == CBK_F16) ((uint16_t*)a.y)[oi] = f2h(v);
+    else ((uint16_t*)a.y)[oi] = f2bf(v);
+  };
+  // (Two separate paths on purpose.  With the bias added behind a common join the wait for its
+  // load stood there for calls without a bias too, and a wait for a load issued last is a wait
+  // for every load in flight, the next step's codes and mask words included: once per round,
+  // in the wavefront that was last already.)
+  auto store = [&](int am, int tile, float v) {
+    const int k = tile * 16 + wr;
+    if (k >= m_K) return;
+    if (a.bias) {
+      const float b = (a.ydt == CBK_F32) ? ((const float*)a.bias)[k]
+                    : (a.ydt == CBK_F16) ? h2f(((const uint16_t*)a.bias)[k]) : bf2f(((const uint16_t*)a.bias)[k]);
+      emit(am, k, v + b);
+    } else {
+      emit(am, k, v);
+    }
+  };
+
+  // BAR: the part sums of a round, added in part order by all threads after the round's barrier
   auto finish_round = [&](int round) {
     const float* rb = red + (size_t)(round & 1) * M * 256;
     for (int o = tid; o < M * 256; o += GV_THREADS) {
@@ -1456,10 +1481,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) 
       for (int j = 0; j < 16; ++j) v += j < SK ? pv[j] : 0.f;
       if (a.bias) v += (a.ydt == CBK_F32) ? ((const float*)a.bias)[k]
                      : (a.ydt == CBK_F16) ? h2f(((const uint16_t*)a.bias)[k]) : bf2f(((const uint16_t*)a.bias)[k]);
-      const size_t oi = (size_t)am * a.ldy + k;
-      if (a.ydt == CBK_F32) ((float*)a.y)[oi] = v;
-      else if (a.ydt == CBK_F16) ((uint16_t*)a.y)[oi] = f2h(v);
-      else ((uint16_t*)a.y)[oi] = f2bf(v);
+      emit(am, k, v);
     }
   };
 
@@ -1469,8 +1491,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) 
 #pragma unroll
     for (int ci = 0; ci < 4; ++ci) zs[ci] = (uint32_t)__shfl((int)c.zs, wr + 16 * ci, 64);
     // (uniform over the wavefront: in the last round a wavefront may be left without a tile; it
-    // has loaded the last tile again, multiplies nothing and goes on to the round's barrier)
-    if (T_lo + p.round * TPR + tir < T_hi)
+    // has loaded the last tile again and multiplies nothing)
+    const bool live = T_lo + p.round * TPR + tir < T_hi;
+    if (live)
 #pragma unroll
     for (int ci = 0; ci < 4; ++ci) {
       const int chunk = 4 * S + ci;
@@ -1534,7 +1557,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) 
         ysum[4 * g + ci] = fmaf(f, h2f((uint16_t)(zs[ci] >> 8)) * dl, ysum[4 * g + ci]);
       }
     }
-    if (S + 1 == s1) {                                              // the item is done
+    if (BAR && S + 1 == s1) {                                       // the item is done: every wavefront meets at the barrier
       float* rb = red + (size_t)(p.round & 1) * M * 256;
 #pragma unroll
       for (int g = 0; g < NG; ++g) {
@@ -1547,6 +1570,64 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) 
       __syncthreads();
       finish_round(p.round);
     }
+    if (!BAR && S + 1 == s1 && live) {                              // the item is done
+      // Lane quarter kq holds the sums of activation rows kq and 4 + kq.  The parts of a tile meet
+      // in LDS, in the buffer of the round's parity, and the wavefront that arrives last adds them
+      // in part order (not arrival order).  No barrier: a wavefront may be rounds ahead of the
+      // others of its tile, so before it writes into a buffer it waits until the sums of the
+      // round that used the buffer last have been added (by a wavefront that waits for nobody
+      // who is behind it: all of them arrived at that round before this one could get here).
+      const int tile = T_lo + p.round * TPR + tir;
+      float ps[NG];
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const int q = 4 * g;
+        ps[g] = (ysum[q] + ysum[q + 1]) + (ysum[q + 2] + ysum[q + 3]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ysum[q + i] = 0.f;
+      }
+      if (SK == 1) {
+#pragma unroll
+        for (int g = 0; g < NG; ++g)
+          if (kq + 4 * g < M) store(kq + 4 * g, tile, ps[g]);
+      } else {
+        float* rb = red + (size_t)(p.round & 1) * M * 256;
+        if (p.round >= 2)
+          while (__hip_atomic_load(&summed[tir], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < p.round - 1)
+            __builtin_amdgcn_s_sleep(1);
+#pragma unroll
+        for (int g = 0; g < NG; ++g)
+          if (kq + 4 * g < M) rb[((kq + 4 * g) * 16 + wave) * 16 + wr] = ps[g];
+        // release: this wavefront's sums are in LDS before its arrival is counted; acquire: the
+        // last one reads the others' sums only after it has seen all their arrivals
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        int old = 0;
+        int* const arr = &arrived[(p.round & 1) * GV_WAVES + tir];   // (the next round counts in the other one; the one
+        if (lane == 0) old = atomicAdd(arr, 1);                     //  after it starts only when this one is back at zero)
+        old = __builtin_amdgcn_readfirstlane(old);
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+        if (old == SK - 1) {                                        // uniform over the wavefront
+#pragma unroll
+          for (int g = 0; g < NG; ++g) {
+            const int am = kq + 4 * g;
+            if (am < M) {
+              float v = 0.f;                                        // (four at a time; parts past SK re-read the last one and do not count)
+              for (int j0 = 0; j0 < SK; j0 += 4) {
+                float pv[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) pv[j] = rb[(am * 16 + tir * SK + (j0 + j < SK ? j0 + j : SK - 1)) * 16 + wr];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v += j0 + j < SK ? pv[j] : 0.f;
+              }
+              store(am, tile, v);
+            }
+          }
+          if (lane == 0) *arr = 0;
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");          // the sums have been read, the counter is back at zero
+          if (lane == 0) __hip_atomic_store(&summed[tir], p.round + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+      }
+    }
   };
 
   // ---- the first loads (row offsets, then mask words), then selector table and activation digits
@@ -1558,8 +1639,8 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) 
     const uint2 e = make_selectors((uint32_t)tid, 0);
 #pragma unroll
     for (int j = 0; j < LUT_LANES; ++j) lut[tid * LUT_LANES + j] = e;
-  } else if (tid < 256 + ZERO_BYTES / 4) {
-    ((uint32_t*)zreg)[tid - 256] = 0u;
+  } else if (tid < 256 + (ZERO_BYTES + CNT_BYTES) / 4) {
+    ((uint32_t*)zreg)[tid - 256] = 0u;                             // zero row and counters
   }
   const int n16 = N >> 4, xitems = M * n16;                        // a multiple of 8
   for (int it = tid; it < xitems; it += GV_THREADS) {
@@ -1568,11 +1649,12 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) 
     stage_convert<0>(xl, m.cs != nullptr, a.xdt, N, 0, n16, it, false, xq, delta, X_PAD);
   }
   __syncthreads();
-  if (idle) {                                                      // (uniform over the wavefront) no item, every barrier
-    for (int round = 0; round < R; ++round) {
-      __syncthreads();
-      finish_round(round);
-    }
+  if (idle) {                                                      // (uniform over the wavefront) no item
+    if (BAR)
+      for (int round = 0; round < R; ++round) {
+        __syncthreads();
+        finish_round(round);
+      }
     return;
   }
   issue_codes(pc, mk, ca);
@@ -1598,9 +1680,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) 
 
 constexpr int STREAM_MFMA_MIN_STEPS = 1536;     // tile-steps (16 rows x 512 columns) from which the matrix-core kernel is used
 
-template <int NG>
+template <int NG, bool BAR>
 static int launch_stream_mfma_ng(const SmArgs& a, size_t lds, int blocks, hipStream_t st) {
-  auto kern = gemv_stream_mfma_kernel<NG>;
+  auto kern = gemv_stream_mfma_kernel<NG, BAR>;
   static std::atomic<int> configured{0};
   if (!configured.load(std::memory_order_acquire)) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
@@ -1613,7 +1695,7 @@ static int launch_stream_mfma_ng(const SmArgs& a, size_t lds, int blocks, hipStr
 
 // LDS of the kernel for mp activation rows of N columns
 static inline size_t stream_mfma_lds(int N, int mp) {
-  return (size_t)LUT_BYTES + ZERO_BYTES + (size_t)mp * NDIG * (N + X_PAD) + (size_t)mp * (N / 128 + 4) * 4 + (size_t)2 * mp * 256 * 4;
+  return (size_t)LUT_BYTES + ZERO_BYTES + CNT_BYTES + (size_t)mp * NDIG * (N + X_PAD) + (size_t)mp * (N / 128 + 4) * 4 + (size_t)2 * mp * 256 * 4;
 }
 
 // CBK_ERR_UNSUPPORTED: not a case of this kernel.
@@ -1662,7 +1744,11 @@ static int launch_gemv_stream_mfma(const DMat& m, const void* x, int xdt, int M,
     a.y = (uint8_t*)y + (size_t)m0 * ldy * (ydt == CBK_F32 ? 4 : 2);
     a.M = mp;
     const size_t lds = stream_mfma_lds(m.N, mp);
-    const int rc = mp > 4 ? launch_stream_mfma_ng<2>(a, lds, blocks, st) : launch_stream_mfma_ng<1>(a, lds, blocks, st);
+    // One activation row: the round ends in a barrier; more: arrival counters (the same sums in
+    // the same order either way).  65536 x 4096, us per call with barrier / counters: M = 1
+    // 42.4 / 44.3, M = 2 44.4 / 44.4, M = 3 47.4 / 44.8, M = 4 49.1 / 45.6, M = 8 62 / 51.
+    const int rc = mp > 4 ? launch_stream_mfma_ng<2, false>(a, lds, blocks, st)
+                 : mp == 1 ? launch_stream_mfma_ng<1, true>(a, lds, blocks, st) : launch_stream_mfma_ng<1, false>(a, lds, blocks, st);
     if (rc) return rc;
   }
   return CBK_OK;
