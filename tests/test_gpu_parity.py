@@ -174,6 +174,36 @@ def test_gemv_survivor_streams_on_matrix_cores(shape):
                 assert torch.equal(yb, want), (case_id(case), K, N, M)
 
 
+def test_gemv_survivor_streams_of_uneven_density():
+    """The matrix-core stream kernel on rows whose groups keep nothing, a tenth, half, nine tenths
+    or all of their columns, group by group at random, with whole rows kept and whole rows pruned:
+    blocks of 0 to 32 survivors at every skew of the code stream (the fifth code dword of a block
+    is loaded only where its survivors reach it)."""
+    K, N = 4112, 3072
+    case = (F.SPARSE4X, 4, 128, 0)
+    raw = make_raw(case, K, N, seed=5)
+    rng = np.random.default_rng(11)
+    dens = rng.choice(np.array([0.0, 0.1, 0.5, 0.9, 1.0]), size=(K, N // 128))
+    keep = rng.random((K, N)) < np.repeat(dens, 128, axis=1)
+    keep[::97] = True
+    keep[5::101] = False
+    raw["q"] = (rng.integers(0, 16, (K, N), dtype=np.uint8) * keep).astype(np.uint8)
+    raw["mask"] = R.pack_bits(keep)
+    pk = oracle_pack(case, raw)
+    pm = packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV)
+    W = R.dequant(pk, K, N, case[0], col_scale=raw["col_scale"], **kw_of(case))
+    assert (W[5::101] == 0).all()
+    for M, dtype in ((1, torch.float16), (3, torch.bfloat16), (8, torch.float16)):
+        x = acts(M, N, dtype, seed=M + N)
+        ref = R.forward_ref(W, _np(x))
+        y = ops.gemv(pm, x.to(DEV), out_dtype=torch.float32)
+        assert rel_fro(_np(y), ref) < 1e-5, M
+        assert np.abs(_np(y) - ref).max() / np.abs(ref).max() < 2e-5
+        assert (_np(y)[:, 5::101] == 0).all()
+        y1 = ops.gemv(pm, x[M - 1:M].to(DEV), out_dtype=torch.float32)
+        assert torch.equal(y1[0], y[M - 1]), M
+
+
 ALL_MFMA_CASES = [(F.BLKC, b, g, k) for b in (2, 3, 4) for g in (64, 128) for k in (10, 16, 23)] + \
                  [(F.DENSEB, b, g, 0) for b in (2, 3, 4) for g in (64, 128)]
 
