@@ -6,8 +6,9 @@
 
 namespace cbk {
 int launch_dequant(const DMat&, int, int, int, void*, int, int64_t, hipStream_t);
-int launch_gemv_generic(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*,
+int launch_gemv_generic(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*, void*, size_t,
                         hipStream_t);
+size_t gemv_stream_workspace(const DMat&, int M);
 struct GvCall { DMat m; const void* x; int64_t ldx; void* y; int64_t ldy; const void* bias; int par; };
 int launch_gemv_fast_batch(int n, const GvCall* calls, int xdt, int M, int ydt, void* ws, size_t ws_bytes,
                            hipStream_t);
@@ -243,7 +244,8 @@ size_t cbk_workspace_bytes(const cbk_desc* in, int M) {
   DMat m;
   if (to_dmat(in, &m, false)) return 0;
   if (family_of(m.layout) == FAM_SPARSE) {                          // cbk_gemm / cbk_linear above 16 rows: see Transient
-    if (M <= 16 || !sparse_repackable(m)) return 0;                 // the row kernel needs none
+    if (M <= 16) return gemv_stream_workspace(m, M);                // part sums of long rows split by columns, else none
+    if (!sparse_repackable(m)) return 0;
     const Transient t = transient_dense4(m);
     return t.end + gemm_big_workspace(dense4_view(m, nullptr, t), M);
   }
@@ -351,17 +353,19 @@ int cbk_gemv_batch(int n, const cbk_desc* descs, const void* const* xs, const in
   if (n == 1) {
     DMat m;
     to_dmat(descs, &m, true);
-    return launch_gemv_generic(m, xs[0], x_dtype, M, ldxs[0], ys[0], y_dtype, ldys[0], biases ? biases[0] : nullptr, st);
+    return launch_gemv_generic(m, xs[0], x_dtype, M, ldxs[0], ys[0], y_dtype, ldys[0], biases ? biases[0] : nullptr,
+                               workspace, workspace_bytes, st);
   }
   // mixed or unsupported configurations: one matrix at a time
   size_t off = 0;
   for (int i = 0; i < n; ++i) {
+    // (cbk_gemv uses a workspace where it has one and computes the same bits without)
     const size_t need = cbk_workspace_bytes(descs + i, M);
-    if (need && (!workspace || off + need > workspace_bytes)) return CBK_ERR_WORKSPACE;
+    const bool room = need && workspace && off + need <= workspace_bytes;
     int rc = cbk_gemv(descs + i, xs[i], x_dtype, M, ldxs[i], ys[i], y_dtype, ldys[i], biases ? biases[i] : nullptr,
-                      need ? (uint8_t*)workspace + off : nullptr, need, stream);
+                      room ? (uint8_t*)workspace + off : nullptr, room ? need : 0, stream);
     if (rc) return rc;
-    off += need;
+    if (room) off += need;
   }
   return CBK_OK;
 }

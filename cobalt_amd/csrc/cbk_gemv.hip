@@ -1048,6 +1048,8 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_split_kernel(GsArgs a) {
 
 // the parts of every output, added in part order; bias; conversion
 constexpr int GS_RED_THREADS = 256;
+static inline size_t up256(size_t v) { return (v + 255) & ~(size_t)255; }
+static inline size_t split_part_bytes(int ntiles, int sk, int Mk) { return (size_t)ntiles * sk * Mk * 16 * 4; }   // [tiles][parts][M][16] floats
 __global__ __launch_bounds__(GS_RED_THREADS) void gemv_split_reduce_kernel(GsArgs a) {
   const GsHead& h = a.h;
   int idx = (int)blockIdx.x * GS_RED_THREADS + (int)threadIdx.x, mi = 0;
@@ -1335,32 +1337,46 @@ struct SmArgs {
   int nS, spi, sk;         // steps per row, steps per part, parts
   uint32_t inv_sk;         // w / sk = (w * inv_sk) >> 16 for w < 16
   int hdr;                 // bytes of a row before its codes
+  // column-split launches: a workgroup owns pps consecutive parts (one column slab) of a range of
+  // tiles, wps workgroups per slab (tq, tr: tiles over the workgroups of a slab), and writes the
+  // part sums to part[tile][sk][M][16]
+  int pps, wps;
+  float* part;
 };
 struct SmMask { uint4 mk; uint32_t go; };                           // mask words and code offset of group 4S + kq
 struct SmCodes { uint32_t e[4][5]; uint32_t mw[4], sh[4]; uint32_t zs; };   // codes (16 bytes + skew), mask word, bit skew per group
 
-template <int NG, bool BAR>
+template <int NG, bool BAR, bool SPLIT>
 __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) {
+  static_assert(!(BAR && SPLIT), "a column-split launch adds nothing itself");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const DMat& m = a.m;
-  const int M = a.M, N = m.N, NCH = N >> 7, Ns = N + X_PAD;
+  const int M = a.M, N = m.N, NCH = N >> 7;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int spi = a.spi, nS = a.nS;
+  // the workgroup's parts [p_lo, p_lo + SK) of the a.sk parts of a row, its columns and tiles
+  const int sl = SPLIT ? (int)blockIdx.x / a.wps : 0;
+  const int bx = SPLIT ? (int)blockIdx.x - sl * a.wps : (int)blockIdx.x;
+  const int p_lo = SPLIT ? sl * a.pps : 0;
+  const int SK = SPLIT ? (a.sk - p_lo < a.pps ? a.sk - p_lo : a.pps) : a.sk;
+  const int col0 = p_lo * spi * 512;
+  const int cols = SPLIT ? (N - col0 < SK * spi * 512 ? N - col0 : SK * spi * 512) : N;
+  const int ch0 = col0 >> 7, Ns = cols + X_PAD;
   uint2* lut = (uint2*)smem;
   uint8_t* zreg = smem + LUT_BYTES;
   int* arrived = (int*)(zreg + ZERO_BYTES);                       // [2][16] part sums written, by round parity and tile of the round
   int* summed = arrived + 2 * GV_WAVES;                           // [16] rounds whose part sums have been added
   int8_t* xq = (int8_t*)zreg + ZERO_BYTES + CNT_BYTES;
-  float* delta = (float*)(xq + (size_t)M * NDIG * Ns);
+  float* delta = (float*)(xq + (size_t)M * NDIG * (SPLIT ? a.pps * spi * 512 + X_PAD : Ns));
   float* red = delta + M * (NCH + 4);                             // [2][M][16 wavefronts][16 rows], by round parity
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wr = lane & 15, kq = lane >> 4;
   const uint32_t l16 = lane & (LUT_LANES - 1);
-  const int bx = (int)blockIdx.x;
   const int T_lo = bx * a.tq + (bx < a.tr ? bx : a.tr), T_hi = T_lo + a.tq + (bx < a.tr ? 1 : 0);
-  const int SK = a.sk, spi = a.spi, nS = a.nS;
   const int TPR = GV_WAVES / SK;                                  // tiles per round (scalar, once)
   const int R = (T_hi - T_lo + TPR - 1) / TPR;                    // rounds
-  const int tir = (int)(((uint32_t)wave * a.inv_sk) >> 16), part = wave - tir * SK;
+  const int tir = SPLIT ? wave / SK : (int)(((uint32_t)wave * a.inv_sk) >> 16);
+  const int part = p_lo + wave - tir * SK;
   const bool idle = tir >= TPR;                                   // wavefronts past the last whole tile of a round
   const int s0 = part * spi, s1 = s0 + spi < nS ? s0 + spi : nS;  // this wavefront's steps (never empty: host)
   const uint8_t* const m_data = m.data;
@@ -1499,7 +1515,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) 
       const int chunk = 4 * S + ci;
       uint32_t aaddr[NG];
 #pragma unroll
-      for (int g = 0; g < NG; ++g) aaddr[g] = (a_on[g] && chunk < NCH) ? a_base[g] + (uint32_t)chunk * 128u : z_off;
+      for (int g = 0; g < NG; ++g) aaddr[g] = (a_on[g] && chunk < NCH) ? a_base[g] + (uint32_t)(chunk - ch0) * 128u : z_off;
       uint32_t w[4];                                                // the block's codes from bit 0 on
 #pragma unroll
       for (int i = 0; i < 4; ++i) w[i] = __builtin_amdgcn_alignbit(c.e[ci][i + 1], c.e[ci][i], c.sh[ci]);
@@ -1570,7 +1586,18 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) 
       __syncthreads();
       finish_round(p.round);
     }
-    if (!BAR && S + 1 == s1 && live) {                              // the item is done
+    if (SPLIT && S + 1 == s1 && live) {                             // the item is done: its sums go to the caller's buffer
+      const int tile = T_lo + p.round * TPR + tir;
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const int q = 4 * g;
+        const float ps = (ysum[q] + ysum[q + 1]) + (ysum[q + 2] + ysum[q + 3]);
+        if (kq + 4 * g < M) a.part[(((size_t)tile * a.sk + part) * M + kq + 4 * g) * 16 + wr] = ps;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ysum[q + i] = 0.f;
+      }
+    }
+    if (!BAR && !SPLIT && S + 1 == s1 && live) {                    // the item is done
       // Lane quarter kq holds the sums of activation rows kq and 4 + kq.  The parts of a tile meet
       // in LDS, in the buffer of the round's parity, and the wavefront that arrives last adds them
       // in part order (not arrival order).  No barrier: a wavefront may be rounds ahead of the
@@ -1641,12 +1668,15 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) 
     for (int j = 0; j < LUT_LANES; ++j) lut[tid * LUT_LANES + j] = e;
   } else if (tid < 256 + (ZERO_BYTES + CNT_BYTES) / 4) {
     ((uint32_t*)zreg)[tid - 256] = 0u;                             // zero row and counters
+  } else if (SPLIT && tid < 256 + (ZERO_BYTES + CNT_BYTES) / 4 + 4 * M) {       // deltas of the chunks past N
+    const int i = tid - 256 - (ZERO_BYTES + CNT_BYTES) / 4;
+    delta[(i >> 2) * (NCH + 4) + NCH + (i & 3)] = 0.f;
   }
-  const int n16 = N >> 4, xitems = M * n16;                        // a multiple of 8
+  const int n16 = cols >> 4, xitems = M * n16;                     // a multiple of 8
   for (int it = tid; it < xitems; it += GV_THREADS) {
     XLoad xl;
-    stage_load(a.x, a.ldx, m.cs, N, 0, n16, it, false, 0, xl);
-    stage_convert<0>(xl, m.cs != nullptr, a.xdt, N, 0, n16, it, false, xq, delta, X_PAD);
+    stage_load(a.x, a.ldx, m.cs, N, col0, n16, it, false, 0, xl);
+    stage_convert<0>(xl, m.cs != nullptr, a.xdt, N, ch0, n16, it, false, xq, delta, X_PAD);
   }
   __syncthreads();
   if (idle) {                                                      // (uniform over the wavefront) no item
@@ -1680,9 +1710,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) 
 
 constexpr int STREAM_MFMA_MIN_STEPS = 1536;     // tile-steps (16 rows x 512 columns) from which the matrix-core kernel is used
 
-template <int NG, bool BAR>
+template <int NG, bool BAR, bool SPLIT = false>
 static int launch_stream_mfma_ng(const SmArgs& a, size_t lds, int blocks, hipStream_t st) {
-  auto kern = gemv_stream_mfma_kernel<NG, BAR>;
+  auto kern = gemv_stream_mfma_kernel<NG, BAR, SPLIT>;
   static std::atomic<int> configured{0};
   if (!configured.load(std::memory_order_acquire)) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
@@ -1698,27 +1728,25 @@ static inline size_t stream_mfma_lds(int N, int mp) {
   return (size_t)LUT_BYTES + ZERO_BYTES + CNT_BYTES + (size_t)mp * NDIG * (N + X_PAD) + (size_t)mp * (N / 128 + 4) * 4 + (size_t)2 * mp * 256 * 4;
 }
 
-// CBK_ERR_UNSUPPORTED: not a case of this kernel.
-static int launch_gemv_stream_mfma(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
-                                   const void* bias, hipStream_t st) {
-  if (m.layout != CBK_SPARSE4X && m.layout != CBK_SPARSE4E) return CBK_ERR_UNSUPPORTED;
-  if (m.N % 128 != 0 || m.K < 1) return CBK_ERR_UNSUPPORTED;
-  int mc = GV_MAX_M;                                                // activation rows per pass: what fits in LDS
-  while (mc > 0 && stream_mfma_lds(m.N, mc) > (size_t)160 * 1024) --mc;
-  if (mc == 0) return CBK_ERR_UNSUPPORTED;
-  SmArgs a;
-  a.m = m; a.ldx = ldx; a.ldy = ldy; a.bias = bias; a.xdt = xdt; a.ydt = ydt;
-  a.ntiles = (m.K + 15) / 16;
+// What the matrix-core stream kernel does with a matrix: false if it is not one of its cases.
+// By the shape alone: which kernel runs, and how a row is cut into parts, must not depend on M,
+// or a row's result would.
+struct SmPlan { int ntiles, blocks, tq, tr, nS, sk, spi, mc; };
+static bool stream_mfma_plan(const DMat& m, SmPlan& p) {
+  if (m.layout != CBK_SPARSE4X && m.layout != CBK_SPARSE4E) return false;
+  if (m.N % 128 != 0 || m.K < 1) return false;
+  p.mc = GV_MAX_M;                                                  // activation rows per pass of whole rows: what fits in LDS
+  while (p.mc > 0 && stream_mfma_lds(m.N, p.mc) > (size_t)160 * 1024) --p.mc;
+  if (p.mc == 0) return false;
+  p.ntiles = (m.K + 15) / 16;
+  p.nS = (m.N / 128 + 3) / 4;
   // Small matrices stay on the row kernel, which is faster there at one activation row
   // (4096 x 2048, 1024 tile-steps: 6.6 against 8.3 us; 2048 x 4096: 8.4 against 8.8 us, but 12.2
   // against 10.1 us at M = 4; 4096 x 4096, 2048 tile-steps: 8.8 / 13.0 / 19.4 us at M = 1 / 4 / 8
-  // against 9.2 / 10.7 / 15.1 us here; 1024 x 14336, 1792: 17.8 against 15.7 us at M = 1).  By
-  // the shape alone: which kernel runs must not depend on M, or a row's result would.
-  if ((long long)a.ntiles * ((m.N / 128 + 3) / 4) < STREAM_MFMA_MIN_STEPS) return CBK_ERR_UNSUPPORTED;
-  const int blocks = a.ntiles < 256 ? a.ntiles : 256;               // one persistent workgroup per CU
-  a.tq = a.ntiles / blocks; a.tr = a.ntiles % blocks;
-  a.nS = (m.N / 128 + 3) / 4;
-  a.hdr = ((m.N >> 3) + ((m.G * 2 + 15) & ~15) + 15) & ~15;
+  // against 9.2 / 10.7 / 15.1 us here; 1024 x 14336, 1792: 17.8 against 15.7 us at M = 1).
+  if ((long long)p.ntiles * p.nS < STREAM_MFMA_MIN_STEPS) return false;
+  p.blocks = p.ntiles < 256 ? p.ntiles : 256;                       // one persistent workgroup per CU
+  p.tq = p.ntiles / p.blocks; p.tr = p.ntiles % p.blocks;
   // Parts per tile: as few steps per wavefront as possible, and few tiles per round.  With one
   // or two tiles in a round the sixteen wavefronts read the same 16 or 32 rows side by side: the
   // cache lines of their offsets, scales and zero points (64 groups or more each) and of their
@@ -1726,29 +1754,106 @@ static int launch_gemv_stream_mfma(const DMat& m, const void* x, int xdt, int M,
   // 15-25 % faster (65536 x 4096 at M = 1: 49.0 us with sixteen tiles in one round, 44.1 us with
   // two in each of eight rounds; 32768 x 8192: 49.8 / 49.0 / 45.2 us with eight / two / one).  A
   // round costs about an eighth of a step beside its steps.  No part may be empty.
-  const int tmax = a.tq + (a.tr ? 1 : 0);
+  const int tmax = p.tq + (p.tr ? 1 : 0);
   float best = 0.f;
-  a.sk = 1; a.spi = a.nS;
-  for (int sk = 1; sk <= GV_WAVES && sk <= a.nS; ++sk) {
-    const int spi = (a.nS + sk - 1) / sk;
-    if ((sk - 1) * spi >= a.nS) continue;
+  p.sk = 1; p.spi = p.nS;
+  for (int sk = 1; sk <= GV_WAVES && sk <= p.nS; ++sk) {
+    const int spi = (p.nS + sk - 1) / sk;
+    if ((sk - 1) * spi >= p.nS) continue;
     const int tpr = GV_WAVES / sk, rounds = (tmax + tpr - 1) / tpr;
     const float c = (float)rounds * ((float)spi * (tpr == 1 ? 0.75f : tpr == 2 ? 0.85f : 1.f) + 0.12f);
-    if (sk == 1 || c < best) { best = c; a.sk = sk; a.spi = spi; }
+    if (sk == 1 || c < best) { best = c; p.sk = sk; p.spi = spi; }
   }
+  return true;
+}
+
+// Room for the part sums of a call whose activation rows do not fit in LDS as whole rows; 0: none needed.
+size_t gemv_stream_workspace(const DMat& m, int M) {
+  SmPlan p;
+  if (family_of(m.layout) != FAM_SPARSE || m.bits != 4 || m.group != 128 || m.cs_rows > 1) return 0;
+  const int Ms = M < GV_MAX_M ? M : GV_MAX_M;                        // rows of a pass over the weights
+  if (!(m.flags & CBK_FLAG_ZERO_LE_128) || !stream_mfma_plan(m, p) || Ms <= p.mc || p.sk < 2) return 0;
+  return up256(split_part_bytes(p.ntiles, p.sk, Ms));
+}
+
+// CBK_ERR_UNSUPPORTED: not a case of this kernel.
+static int launch_gemv_stream_mfma(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
+                                   const void* bias, void* ws, size_t ws_bytes, hipStream_t st) {
+  SmPlan p;
+  if (!stream_mfma_plan(m, p)) return CBK_ERR_UNSUPPORTED;
+  SmArgs a;
+  a.m = m; a.ldx = ldx; a.ldy = ldy; a.bias = bias; a.xdt = xdt; a.ydt = ydt;
+  a.ntiles = p.ntiles; a.tq = p.tq; a.tr = p.tr; a.nS = p.nS; a.sk = p.sk; a.spi = p.spi;
+  a.hdr = ((m.N >> 3) + ((m.G * 2 + 15) & ~15) + 15) & ~15;
   a.inv_sk = (uint32_t)((65536 + a.sk - 1) / a.sk);
-  mc = (M + (M + mc - 1) / mc - 1) / ((M + mc - 1) / mc);            // the same number of passes, of equal size
+  a.pps = a.sk; a.wps = p.blocks; a.part = nullptr;
+  const size_t ysz = ydt == CBK_F32 ? 4 : 2;
+  // More activation rows than fit in LDS as whole rows: with room for the part sums the
+  // workgroups split the row by columns (whole parts: the same parts, added in the same order by
+  // the reduce kernel of the column-split path above, so the same bits), up to eight activation
+  // rows per pass over the weights; without it the rows go in passes of what fits.
+  const int Ms = M < GV_MAX_M ? M : GV_MAX_M;
+  if (Ms > p.mc && p.sk >= 2 && ws && !((uintptr_t)ws & 15) && ws_bytes >= split_part_bytes(p.ntiles, p.sk, Ms)) {
+    const size_t fixed = (size_t)LUT_BYTES + ZERO_BYTES + CNT_BYTES + (size_t)Ms * (m.N / 128 + 4) * 4 + (size_t)Ms * NDIG * X_PAD;
+    const size_t per_part = (size_t)Ms * NDIG * p.spi * 512;
+    int pps_max = fixed < (size_t)160 * 1024 ? (int)(((size_t)160 * 1024 - fixed) / per_part) : 0;
+    pps_max = pps_max < p.sk ? pps_max : p.sk;
+    if (pps_max >= 1) {
+      // parts per slab: rounds of one part per wavefront after staging the slab (a 512-column
+      // step of eight rows costs about 0.15 rounds of one step to stage)
+      float best = 0.f;
+      int best_pps = 0, best_wps = 1;
+      for (int pps = 1; pps <= pps_max; ++pps) {
+        const int nslab = (p.sk + pps - 1) / pps;
+        if (nslab > 256) continue;
+        int wps = 256 / nslab;
+        wps = wps > p.ntiles ? p.ntiles : wps;
+        const int tpw = (p.ntiles + wps - 1) / wps, tpr = GV_WAVES / pps;
+        const float c = (float)((tpw + tpr - 1) / tpr * p.spi) + 0.15f * (float)Ms / 8.f * (float)(pps * p.spi);
+        if (best_pps == 0 || c < best) { best = c; best_pps = pps; best_wps = wps; }
+      }
+      if (best_pps > 0) {
+        const int nslab = (p.sk + best_pps - 1) / best_pps;
+        a.pps = best_pps; a.wps = best_wps;
+        a.tq = p.ntiles / best_wps; a.tr = p.ntiles % best_wps;
+        a.part = (float*)ws;
+        const size_t lds = fixed + (size_t)Ms * NDIG * best_pps * p.spi * 512;
+        GsArgs r = {};                                                // the reduce launch: one matrix
+        r.h.n = 1; r.h.ydt = ydt; r.h.xdt = xdt; r.h.xq_cap = 0; r.h.delta_cap = 0;
+        for (int i = 0; i < GV_MAX_BATCH; ++i) { r.h.wg_end[i] = 0x7fffffff; r.h.th_end[i] = 0x7fffffff; }
+        GsMat& q = r.mat[0];
+        q.g.m = m; q.g.par = 0; q.g.bias = bias; q.g.ldy = ldy; q.g.ntiles = p.ntiles; q.g.sk = p.sk;
+        q.th0 = 0; q.wg0 = 0; q.part = (float*)ws;
+        for (int m0 = 0; m0 < M; m0 += GV_MAX_M) {
+          const int mp = M - m0 < GV_MAX_M ? M - m0 : GV_MAX_M;
+          a.x = (const uint16_t*)x + (size_t)m0 * ldx;
+          a.M = mp;
+          const int rc = mp > 4 ? launch_stream_mfma_ng<2, false, true>(a, lds, nslab * best_wps, st)
+                                : launch_stream_mfma_ng<1, false, true>(a, lds, nslab * best_wps, st);
+          if (rc) return rc;
+          r.h.M = mp;
+          q.g.y = (uint8_t*)y + (size_t)m0 * ldy * ysz;
+          const int th = (p.ntiles * mp * 16 + GS_RED_THREADS - 1) / GS_RED_THREADS * GS_RED_THREADS;
+          r.h.th_end[0] = th;
+          hipLaunchKernelGGL(gemv_split_reduce_kernel, dim3(th / GS_RED_THREADS), dim3(GS_RED_THREADS), 0, st, r);
+          if (hipGetLastError() != hipSuccess) return CBK_ERR_HIP;
+        }
+        return CBK_OK;
+      }
+    }
+  }
+  int mc = (M + (M + p.mc - 1) / p.mc - 1) / ((M + p.mc - 1) / p.mc);   // as few passes as fit, of equal size
   for (int m0 = 0; m0 < M; m0 += mc) {
     const int mp = M - m0 < mc ? M - m0 : mc;
     a.x = (const uint16_t*)x + (size_t)m0 * ldx;
-    a.y = (uint8_t*)y + (size_t)m0 * ldy * (ydt == CBK_F32 ? 4 : 2);
+    a.y = (uint8_t*)y + (size_t)m0 * ldy * ysz;
     a.M = mp;
     const size_t lds = stream_mfma_lds(m.N, mp);
     // One activation row: the round ends in a barrier; more: arrival counters (the same sums in
     // the same order either way).  65536 x 4096, us per call with barrier / counters: M = 1
     // 42.4 / 44.3, M = 2 44.4 / 44.4, M = 3 47.4 / 44.8, M = 4 49.1 / 45.6, M = 8 62 / 51.
-    const int rc = mp > 4 ? launch_stream_mfma_ng<2, false>(a, lds, blocks, st)
-                 : mp == 1 ? launch_stream_mfma_ng<1, true>(a, lds, blocks, st) : launch_stream_mfma_ng<1, false>(a, lds, blocks, st);
+    const int rc = mp > 4 ? launch_stream_mfma_ng<2, false>(a, lds, p.blocks, st)
+                 : mp == 1 ? launch_stream_mfma_ng<1, true>(a, lds, p.blocks, st) : launch_stream_mfma_ng<1, false>(a, lds, p.blocks, st);
     if (rc) return rc;
   }
   return CBK_OK;
@@ -1756,12 +1861,12 @@ static int launch_gemv_stream_mfma(const DMat& m, const void* x, int xdt, int M,
 
 // CBK_ERR_UNSUPPORTED: not a case of this kernel (the caller falls back on the float row kernel).
 int launch_gemv_stream(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
-                       const void* bias, hipStream_t st) {
+                       const void* bias, void* ws, size_t ws_bytes, hipStream_t st) {
   if (family_of(m.layout) != FAM_SPARSE || m.bits != 4 || m.group != 128 || m.cs_rows > 1) return CBK_ERR_UNSUPPORTED;
   if (!(m.flags & CBK_FLAG_ZERO_LE_128)) return CBK_ERR_UNSUPPORTED;
   if (xdt != CBK_F16 && xdt != CBK_BF16T) return CBK_ERR_DTYPE;
   {
-    const int rc = launch_gemv_stream_mfma(m, x, xdt, M, ldx, y, ydt, ldy, bias, st);   // the layouts with group offsets
+    const int rc = launch_gemv_stream_mfma(m, x, xdt, M, ldx, y, ydt, ldy, bias, ws, ws_bytes, st);   // the layouts with group offsets
     if (rc != CBK_ERR_UNSUPPORTED) return rc;
   }
   if ((size_t)NDIG * m.N > (size_t)ST_X_BUDGET) return CBK_ERR_UNSUPPORTED;
@@ -1979,7 +2084,6 @@ int launch_gemv_dense8(const DMat& m, const void* x, int xdt, int M, int64_t ldx
 }
 
 // ------------------------------------------------------------------ host side
-static inline size_t up256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 static bool keep_supported(int keep) { return keep == 10 || keep == 16 || keep == 23; }
 
@@ -2046,7 +2150,6 @@ static inline int kernel_rows(const DMat& m, int M) {            // activation r
   const int v = m.cs_rows == 2 ? 2 : 1;
   return M * v > GV_MAX_M ? GV_MAX_M : M * v;
 }
-static inline size_t split_part_bytes(int ntiles, int sk, int Mk) { return (size_t)ntiles * sk * Mk * 16 * 4; }
 
 size_t gemv_fast_workspace(const DMat& m, int M) {
   const int Mk = kernel_rows(m, M);

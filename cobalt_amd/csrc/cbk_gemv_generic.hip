@@ -275,14 +275,14 @@ static int launch_m(const DMat& m, const void* x, int M, int64_t ldx, void* y, i
   return launch_p<XDT, 3>(m, x, M, ldx, y, ydt, ldy, bias, st);
 }
 
-int launch_gemv_stream(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*, hipStream_t);
+int launch_gemv_stream(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*, void*, size_t, hipStream_t);
 int launch_gemv_dense8(const DMat&, const void*, int, int, int64_t, void*, int, int64_t, const void*, hipStream_t);
 
 int launch_gemv_generic(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt,
-                        int64_t ldy, const void* bias, hipStream_t st) {
+                        int64_t ldy, const void* bias, void* ws, size_t ws_bytes, hipStream_t st) {
   if (family_of(m.layout) == FAM_SPARSE || m.layout == CBK_DENSE8) {   // integer-dot kernels where they apply
     const int rc = m.layout == CBK_DENSE8 ? launch_gemv_dense8(m, x, xdt, M, ldx, y, ydt, ldy, bias, st)
-                                          : launch_gemv_stream(m, x, xdt, M, ldx, y, ydt, ldy, bias, st);
+                                          : launch_gemv_stream(m, x, xdt, M, ldx, y, ydt, ldy, bias, ws, ws_bytes, st);
     if (rc != CBK_ERR_UNSUPPORTED) return rc;
   }
   if (xdt == CBK_F16) return launch_m<CBK_F16>(m, x, M, ldx, y, ydt, ldy, bias, st);

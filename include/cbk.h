@@ -139,8 +139,10 @@ size_t cbk_stream_bytes(const cbk_desc* d, size_t sparse_data_bytes);
  * of a launch that would not fill the chip.  The decode kernels need none, with one optional use:
  * two to eight activation rows of rows whose activations take more than 90 KB of LDS
  * (M * 3 * N bytes) are split over the workgroups by columns when there is room for the float32
- * part sums, K * 16 * M * 4 bytes at most; with a smaller workspace, or none, cbk_gemv computes
- * the same bits more slowly and reports no error.
+ * part sums, K * 16 * M * 4 bytes at most, and so are the rows of SPARSE4X / SPARSE4E matrices on
+ * the matrix-core stream kernel when the activation rows of a pass (up to eight) do not fit in
+ * LDS as whole rows (M * 3 * N bytes beyond about 140 KB); with a smaller workspace, or none,
+ * cbk_gemv computes the same bits more slowly and reports no error.
  * Ask, do not compute.  256-byte aligned. */
 size_t cbk_workspace_bytes(const cbk_desc* d, int M);
 

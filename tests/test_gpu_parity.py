@@ -152,6 +152,7 @@ def test_gemv_survivor_streams_on_matrix_cores(shape):
     activation rows, both activation types, a bias, run-to-run identical, and a row's result does
     not depend on how many rows the call has."""
     K, N = shape
+    small = torch.empty(256, dtype=torch.uint8, device=DEV)
     for case in ([(F.SPARSE4X, 4, 128, 0), (F.SPARSE4E, 4, 128, 0)] if N == 640 else [(F.SPARSE4X, 4, 128, 0)]):
         raw = make_raw(case, K, N, seed=K + N + case[0])
         pk = oracle_pack(case, raw)
@@ -168,6 +169,12 @@ def test_gemv_survivor_streams_on_matrix_cores(shape):
             assert torch.equal(ops.gemv(pm, x.to(DEV), out_dtype=torch.float32), y)
             y1 = ops.gemv(pm, x[M - 1:M].to(DEV), out_dtype=torch.float32)
             assert torch.equal(y1[0], y[M - 1]), (case_id(case), K, N, M)
+            # More rows than fit in LDS as whole rows (14336 columns: from four on): split over the
+            # workgroups by columns where the caller has left room for the part sums, in passes
+            # of fewer rows where not; the same bits either way.
+            need = _lib.lib().cbk_workspace_bytes(ctypes.byref(pm.desc()), M)
+            assert (need >= (K + 15) // 16 * 2 * min(M, 8) * 16 * 4) == (N == 14336 and M >= 4), (K, N, M, need)
+            assert torch.equal(ops.gemv(pm, x.to(DEV), out_dtype=torch.float32, workspace=small), y), (case_id(case), K, N, M)
             if M in (1, 8):
                 yb = ops.gemv(pm, x.to(DEV), bias=bias.to(DEV), out_dtype=dtype)
                 want = (y + bias.to(DEV).to(dtype).float()[None, :]).to(dtype)      # (the bias has the output's type)
