@@ -248,6 +248,49 @@ def unpack(pm: PackedMatrix):
     return mask, q
 
 
+def with_group_offsets(pm: PackedMatrix) -> PackedMatrix:
+    """A SPARSE4 matrix as SPARSE4X: the same mask words and code bytes, plus, behind the mask
+    plane of every row, the table of 16-bit byte offsets of its groups' codes that SPARSE4X / 4E
+    rows carry (pack_cobalt.py:201-250: the running sum of ceil(survivors / 2) over the groups
+    before), padded to 16 bytes.  Two bytes per group (0.125 bits per weight) more; with them the
+    rows are served by the 16-row matrix-core stream kernel instead of the row kernel, which has
+    to sum the offsets of every row itself.  Runs on the device the matrix is on."""
+    from . import format as F
+    if pm.layout != F.SPARSE4:
+        raise ValueError("only SPARSE4 rows lack the offset table")
+    K, N, G = pm.K, pm.N, pm.G
+    dev = pm.device
+    data = pm.array("data")
+    ro = pm.array("row_off").to(torch.int64) & 0xFFFFFFFF                     # [K + 1]
+    nm = N // 8
+    gp = (2 * G + 15) // 16 * 16
+    ar = lambda n: torch.arange(n, device=dev, dtype=torch.int64)
+    mask = data[ro[:K, None] + ar(nm)[None, :]]                               # [K, N / 8]
+    popc = torch.tensor([bin(i).count("1") for i in range(256)], dtype=torch.int64, device=dev)
+    cnt = popc[mask.to(torch.int64)].view(K, G, pm.group // 8).sum(-1)
+    gbytes = (cnt + 1) // 2
+    goff = torch.cumsum(gbytes, 1) - gbytes
+    if int(goff.max()) >= 1 << 16:
+        raise ValueError("a row's codes exceed the 16-bit offsets of SPARSE4X")
+    total = int(ro[K])
+    new_ro = ro + ar(K + 1) * gp
+    if int(new_ro[K]) >= 1 << 32:
+        raise ValueError("the image would exceed 32-bit row offsets")
+    out = torch.zeros(total + K * gp + F.BLOB_TAIL, dtype=torch.uint8, device=dev)
+    out[new_ro[:K, None] + ar(nm)[None, :]] = mask
+    gb = torch.stack([goff & 0xFF, goff >> 8], -1).to(torch.uint8).view(K, 2 * G)
+    out[new_ro[:K, None] + nm + ar(2 * G)[None, :]] = gb
+    clen = ro[1:] - ro[:K] - nm                                               # code bytes (with padding) of every row
+    row = torch.repeat_interleave(ar(K), clen)
+    within = ar(int(clen.sum())) - torch.repeat_interleave(torch.cumsum(clen, 0) - clen, clen)
+    out[new_ro[row] + nm + gp + within] = data[ro[row] + nm + within]
+    cs = pm.array("col_scale").view(pm.cs_rows, N) if pm.cs_rows else None
+    res = F.from_arrays(out, pm.array("scale").view(K, G), pm.array("zero").view(K, G), cs, K, N, F.SPARSE4X,
+                        pm.bits, pm.group, None, row_off=new_ro.to(torch.int32), cs_splits=pm.cs_splits, device=dev)
+    res.n_survivors = pm.n_survivors
+    return res
+
+
 def transcode(pm: PackedMatrix, layout: int, bits=None, group=None, keep=None, tiled=True) -> PackedMatrix:
     """The same weights in another fixed-stride layout (same codes, scales, zero points and column
     scales; every weight dequantises to the same value).  The use: a survivor-stream matrix

@@ -245,6 +245,29 @@ def test_survivor_stream_with_zero_points_off_the_code_grid():
     assert rel_fro(y, R.forward_ref(W, x.float().numpy())) < 1e-3
 
 
+def test_module_with_sparse4_rows_gets_group_offsets_in_device_order():
+    """to_device_order on a SPARSE4 matrix (the packer's default, pack_cobalt.py:561): the same codes
+    as SPARSE4X, which the matrix-core stream kernel takes; values and results unchanged."""
+    case = (F.SPARSE4, 4, 128, 0)
+    K, N = 4112, 3072
+    raw = R.synth_raw_matrix(K, N, 0.5, 4, seed=8)
+    pk = oracle_pack(case, raw)
+    W = R.dequant(pk, K, N, F.SPARSE4, col_scale=raw["col_scale"])
+    lin = CobaltLinear(packed_from_oracle(case, pk, raw["col_scale"], K, N, DEV))
+    x = acts(5, N, torch.float16, seed=1).to(DEV)
+    y4 = ops.gemv(lin._pm(), x, out_dtype=torch.float32)
+    lin.to_device_order()
+    pm = lin._pm()
+    assert pm.layout == F.SPARSE4X and not pm.tiled
+    px = R.pack_matrix(raw["mask"], raw["q"], raw["scale"], raw["zero"], R.SPARSE4X)
+    assert np.array_equal(pm.array("data").cpu().numpy(), px["data"])
+    assert np.array_equal(lin.dequantize().cpu().numpy() + np.float32(0), W + np.float32(0))
+    yx = ops.gemv(pm, x, out_dtype=torch.float32)
+    ref = R.forward_ref(W, x.float().cpu().numpy())
+    assert rel_fro(yx.cpu().numpy(), ref) < 1e-5 and rel_fro(y4.cpu().numpy(), ref) < 1e-5
+    assert lin.to_device_order()._pm().layout == F.SPARSE4X                     # and stays
+
+
 def test_module_with_a_survivor_stream_matrix_can_be_repacked_at_load():
     case = (F.SPARSE4E, 4, 128, 0)
     K, N = 96, 1024

@@ -80,6 +80,36 @@ def test_stream_helpers_roundtrip():
 
 
 # ------------------------------------------------------------------ C ABI
+def test_group_offsets_turn_sparse4_rows_into_the_oracles_sparse4x_bytes():
+    """ops.with_group_offsets: the SPARSE4 image of a matrix plus the offset tables is, byte for
+    byte, the SPARSE4X image the packer writes for the same matrix (pack_cobalt.py:201-250);
+    groups with no, one and all survivors, a row count off the 16-row grid."""
+    from cobalt_amd import ops
+    from helpers import packed_from_oracle
+    K, N = 37, 1024
+    raw = R.synth_raw_matrix(K, N, 0.5, 4, seed=21)
+    rng = np.random.default_rng(3)
+    keep = R.unpack_bits(raw["mask"], N)
+    keep[3, :256] = False
+    keep[4, 128:384] = True
+    keep[5] = False
+    keep[5, 700] = True
+    raw["q"] = (rng.integers(0, 16, (K, N), dtype=np.uint8) * keep).astype(np.uint8)
+    raw["mask"] = R.pack_bits(keep)
+    p4 = R.pack_matrix(raw["mask"], raw["q"], raw["scale"], raw["zero"], R.SPARSE4)
+    px = R.pack_matrix(raw["mask"], raw["q"], raw["scale"], raw["zero"], R.SPARSE4X)
+    pm4 = packed_from_oracle((F.SPARSE4, 4, 128, 0), p4, raw["col_scale"], K, N, "cpu")
+    pmx = ops.with_group_offsets(pm4)
+    assert pmx.layout == F.SPARSE4X and pmx.validate(deep=True) is pmx
+    assert np.array_equal(pmx.array("row_off").numpy().view(np.uint32), px["row_off"])
+    assert np.array_equal(pmx.array("data").numpy(), px["data"])
+    assert np.array_equal(pmx.array("scale").numpy().view(np.uint16), np.asarray(px["scale"]).view(np.uint16).reshape(-1))
+    assert np.array_equal(pmx.array("zero").numpy(), np.asarray(px["zero"]).reshape(-1))
+    assert torch.equal(pmx.array("col_scale"), pm4.array("col_scale"))
+    with pytest.raises(ValueError):
+        ops.with_group_offsets(pmx)
+
+
 def test_library_exports_every_declared_symbol():
     hdr = open(os.path.join(ROOT, "include", "cbk.h")).read()
     names = set(re.findall(r"\b(cbk_[a-z_]+)\s*\(", hdr))
