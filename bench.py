@@ -894,12 +894,14 @@ def main():
     }
     if not a.no_secondary:
         out["per_matrix"] = per_matrix(torch, F, L, dev, shapes, layout, a.bits, a.group, a.keep, M, dt, use_graph=not a.no_graph)
-        # the layouts that decode on the row kernels (integer dot products), on the workload's gate matrix
+        # the layouts off the main kernel, on the workload's gate matrix: SPARSE4X (rows of different
+        # lengths: the 16-row matrix-core stream kernel) at one and at eight activation rows, DENSE8
+        # (integer-dot row kernel)
         gate = [sh for sh in shapes if sh[0] == "gate"]
         out["row_kernel_layouts"] = [
-            dict(layout=F.LAYOUT_NAME[lay], **per_matrix(torch, F, L, dev, gate, lay, b, 128, None, M, dt, tiled=False,
-                                                         use_graph=not a.no_graph)[0])
-            for lay, b in ((F.SPARSE4X, 4), (F.DENSE8, 8))]
+            dict(layout=F.LAYOUT_NAME[lay], M=m_, **per_matrix(torch, F, L, dev, gate, lay, b, 128, None, m_, dt, tiled=False,
+                                                               use_graph=not a.no_graph)[0])
+            for lay, b, m_ in ((F.SPARSE4X, 4, M), (F.SPARSE4X, 4, 8), (F.DENSE8, 8, M))]
         other = "mistral7b" if a.workload == "gemma27b" else "gemma27b"
         oshapes, odt = SHAPES[other], torch_dtype(torch, WORKLOAD_DTYPE[other])
         osets, _ = make_sets(torch, F, dev, oshapes, layout, a.bits, a.group, a.keep, 2 * INFINITY_CACHE)
