@@ -1322,8 +1322,12 @@ static int launch_stream_m(const DMat& m, const void* x, int64_t ldx, int xdt, v
 // Work split: a workgroup takes a range of tiles; a tile's row is cut into SK parts of spi steps,
 // wavefront w of a round works on part w % SK of the round's tile w / SK; the part sums meet in
 // LDS and are added in part order: by the wavefront that finishes a tile's round last, or (BAR,
-// used for one activation row, where it measured faster) by all threads behind a barrier.  SK and spi depend on the matrix shape only,
-// and every activation row goes through the same operations in the same order whatever M is.
+// used for one activation row, where it measured faster) by all threads behind a barrier.  SK
+// and spi depend on the matrix shape only, and every activation row goes through the same
+// operations in the same order whatever M is.  SPLIT: for activation rows that do not fit in LDS
+// as whole rows a workgroup takes one column slab (some of the SK parts) of a range of tiles and
+// writes its part sums to the caller's workspace; gemv_split_reduce_kernel adds them, in the
+// same order.
 // Reference semantics: cbk::gemv_sparse4 (src/cobaltkernel/csrc/cobalt_gemv.cuh:216-301).
 struct SmArgs {
   DMat m;

@@ -181,6 +181,29 @@ def test_gemv_survivor_streams_on_matrix_cores(shape):
                 assert torch.equal(yb, want), (case_id(case), K, N, M)
 
 
+def test_gemv_survivor_streams_over_many_rounds():
+    """The matrix-core stream kernel where a workgroup goes through several rounds of two tiles
+    with eight parts each (20496 x 4096: five or six tiles per workgroup): the part sums of a
+    round meet in one of two LDS buffers, behind a barrier at one activation row, through arrival
+    counters from two rows on (a wavefront that is rounds ahead waits for the buffer).  Checked
+    against float64 products with the library's own dequantised matrix (itself bit-exact against
+    the oracle in the tests above): every M, run to run, and row by row against M = 1."""
+    K, N = 20496, 4096
+    pm = F.synth_packed(K, N, F.SPARSE4X, 4, 128, None, seed=17, device=DEV)
+    W = ops.dequant(pm, torch.float32).double()
+    x8 = acts(8, N, torch.float16, seed=3).to(DEV)
+    rows = [ops.gemv(pm, x8[i:i + 1], out_dtype=torch.float32)[0] for i in range(8)]
+    for M in (1, 2, 3, 4, 5, 8):
+        x = x8[:M]
+        y = ops.gemv(pm, x, out_dtype=torch.float32)
+        ref = x.double() @ W.T
+        assert float((y.double() - ref).norm() / ref.norm()) < 1e-5, M
+        for _ in range(3):
+            assert torch.equal(ops.gemv(pm, x, out_dtype=torch.float32), y), M
+        for i in range(M):
+            assert torch.equal(y[i], rows[i]), (M, i)
+
+
 def test_gemv_survivor_streams_of_uneven_density():
     """The matrix-core stream kernel on rows whose groups keep nothing, a tenth, half, nine tenths
     or all of their columns, group by group at random, with whole rows kept and whole rows pruned:
