@@ -1336,7 +1336,9 @@ struct SmArgs {
   void* y;
   int64_t ldy;
   const void* bias;
-  int M, xdt, ydt;
+  int M, xdt, ydt;         // M: activation rows as the kernel counts them
+  int par;                 // 1: two col_scale vectors by row parity (a fused gate/up matrix): kernel row v is row v / 2 of
+                           // x scaled by vector v % 2, and weight row k keeps the rows v = k (mod 2)
   int ntiles, tq, tr;      // tiles per workgroup: tq, one more for the first tr workgroups
   int nS, spi, sk;         // steps per row, steps per part, parts
   uint32_t inv_sk;         // w / sk = (w * inv_sk) >> 16 for w < 16
@@ -1464,6 +1466,10 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) 
   for (int i = 0; i < 4 * NG; ++i) ysum[i] = 0.f;
 
   auto emit = [&](int am, int k, float v) {
+    if (a.par) {                                                    // the sum scaled for the other parity is dropped
+      if ((am ^ k) & 1) return;
+      am >>= 1;
+    }
     const size_t oi = (size_t)am * a.ldy + k;
     if (a.ydt == CBK_F32) ((float*)a.y)[oi] = v;
     else if (a.ydt == CBK_F16) ((uint16_t*)a.y)[oi] = f2h(v);
@@ -1679,7 +1685,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_stream_mfma_kernel(SmArgs a) 
   const int n16 = cols >> 4, xitems = M * n16;                     // a multiple of 8
   for (int it = tid; it < xitems; it += GV_THREADS) {
     XLoad xl;
-    stage_load(a.x, a.ldx, m.cs, N, col0, n16, it, false, 0, xl);
+    stage_load(a.x, a.ldx, m.cs, N, col0, n16, it, false, a.par, xl);
     stage_convert<0>(xl, m.cs != nullptr, a.xdt, N, ch0, n16, it, false, xq, delta, X_PAD);
   }
   __syncthreads();
@@ -1774,8 +1780,9 @@ static bool stream_mfma_plan(const DMat& m, SmPlan& p) {
 // Room for the part sums of a call whose activation rows do not fit in LDS as whole rows; 0: none needed.
 size_t gemv_stream_workspace(const DMat& m, int M) {
   SmPlan p;
-  if (family_of(m.layout) != FAM_SPARSE || m.bits != 4 || m.group != 128 || m.cs_rows > 1) return 0;
-  const int Ms = M < GV_MAX_M ? M : GV_MAX_M;                        // rows of a pass over the weights
+  if (family_of(m.layout) != FAM_SPARSE || m.bits != 4 || m.group != 128 || m.cs_rows > 2) return 0;
+  const int vm = m.cs_rows == 2 ? 2 : 1;
+  const int Ms = M * vm < GV_MAX_M ? M * vm : GV_MAX_M;              // kernel rows of a pass over the weights
   if (!(m.flags & CBK_FLAG_ZERO_LE_128) || !stream_mfma_plan(m, p) || Ms <= p.mc || p.sk < 2) return 0;
   return up256(split_part_bytes(p.ntiles, p.sk, Ms));
 }
@@ -1791,12 +1798,16 @@ static int launch_gemv_stream_mfma(const DMat& m, const void* x, int xdt, int M,
   a.hdr = ((m.N >> 3) + ((m.G * 2 + 15) & ~15) + 15) & ~15;
   a.inv_sk = (uint32_t)((65536 + a.sk - 1) / a.sk);
   a.pps = a.sk; a.wps = p.blocks; a.part = nullptr;
+  // a fused gate/up matrix (two col_scale vectors by row parity) stages two scaled copies of every activation row
+  const int vm = m.cs_rows == 2 ? 2 : 1;
+  a.par = vm == 2 ? 1 : 0;
+  if (p.mc < vm) return CBK_ERR_UNSUPPORTED;
   const size_t ysz = ydt == CBK_F32 ? 4 : 2;
   // More activation rows than fit in LDS as whole rows: with room for the part sums the
   // workgroups split the row by columns (whole parts: the same parts, added in the same order by
   // the reduce kernel of the column-split path above, so the same bits), up to eight activation
   // rows per pass over the weights; without it the rows go in passes of what fits.
-  const int Ms = M < GV_MAX_M ? M : GV_MAX_M;
+  const int Ms = M * vm < GV_MAX_M ? M * vm : GV_MAX_M;              // kernel rows of a pass
   if (Ms > p.mc && p.sk >= 2 && ws && !((uintptr_t)ws & 15) && ws_bytes >= split_part_bytes(p.ntiles, p.sk, Ms)) {
     const size_t fixed = (size_t)LUT_BYTES + ZERO_BYTES + CNT_BYTES + (size_t)Ms * (m.N / 128 + 4) * 4 + (size_t)Ms * NDIG * X_PAD;
     const size_t per_part = (size_t)Ms * NDIG * p.spi * 512;
@@ -1826,10 +1837,10 @@ static int launch_gemv_stream_mfma(const DMat& m, const void* x, int xdt, int M,
         r.h.n = 1; r.h.ydt = ydt; r.h.xdt = xdt; r.h.xq_cap = 0; r.h.delta_cap = 0;
         for (int i = 0; i < GV_MAX_BATCH; ++i) { r.h.wg_end[i] = 0x7fffffff; r.h.th_end[i] = 0x7fffffff; }
         GsMat& q = r.mat[0];
-        q.g.m = m; q.g.par = 0; q.g.bias = bias; q.g.ldy = ldy; q.g.ntiles = p.ntiles; q.g.sk = p.sk;
+        q.g.m = m; q.g.par = a.par; q.g.bias = bias; q.g.ldy = ldy; q.g.ntiles = p.ntiles; q.g.sk = p.sk;
         q.th0 = 0; q.wg0 = 0; q.part = (float*)ws;
-        for (int m0 = 0; m0 < M; m0 += GV_MAX_M) {
-          const int mp = M - m0 < GV_MAX_M ? M - m0 : GV_MAX_M;
+        for (int m0 = 0; m0 < M; m0 += GV_MAX_M / vm) {
+          const int mp = (M - m0 < GV_MAX_M / vm ? M - m0 : GV_MAX_M / vm) * vm;      // kernel rows
           a.x = (const uint16_t*)x + (size_t)m0 * ldx;
           a.M = mp;
           const int rc = mp > 4 ? launch_stream_mfma_ng<2, false, true>(a, lds, nslab * best_wps, st)
@@ -1846,9 +1857,10 @@ static int launch_gemv_stream_mfma(const DMat& m, const void* x, int xdt, int M,
       }
     }
   }
-  int mc = (M + (M + p.mc - 1) / p.mc - 1) / ((M + p.mc - 1) / p.mc);   // as few passes as fit, of equal size
+  const int mr = p.mc / vm;                                             // activation rows that fit
+  const int mc = (M + (M + mr - 1) / mr - 1) / ((M + mr - 1) / mr);     // as few passes as fit, of equal size
   for (int m0 = 0; m0 < M; m0 += mc) {
-    const int mp = M - m0 < mc ? M - m0 : mc;
+    const int mp = (M - m0 < mc ? M - m0 : mc) * vm;                    // kernel rows
     a.x = (const uint16_t*)x + (size_t)m0 * ldx;
     a.y = (uint8_t*)y + (size_t)m0 * ldy * ysz;
     a.M = mp;
@@ -1866,13 +1878,14 @@ static int launch_gemv_stream_mfma(const DMat& m, const void* x, int xdt, int M,
 // CBK_ERR_UNSUPPORTED: not a case of this kernel (the caller falls back on the float row kernel).
 int launch_gemv_stream(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
                        const void* bias, void* ws, size_t ws_bytes, hipStream_t st) {
-  if (family_of(m.layout) != FAM_SPARSE || m.bits != 4 || m.group != 128 || m.cs_rows > 1) return CBK_ERR_UNSUPPORTED;
+  if (family_of(m.layout) != FAM_SPARSE || m.bits != 4 || m.group != 128 || m.cs_rows > 2) return CBK_ERR_UNSUPPORTED;
   if (!(m.flags & CBK_FLAG_ZERO_LE_128)) return CBK_ERR_UNSUPPORTED;
   if (xdt != CBK_F16 && xdt != CBK_BF16T) return CBK_ERR_DTYPE;
   {
     const int rc = launch_gemv_stream_mfma(m, x, xdt, M, ldx, y, ydt, ldy, bias, ws, ws_bytes, st);   // the layouts with group offsets
     if (rc != CBK_ERR_UNSUPPORTED) return rc;
   }
+  if (m.cs_rows > 1) return CBK_ERR_UNSUPPORTED;                     // (fused gate/up: the matrix-core kernel only)
   if ((size_t)NDIG * m.N > (size_t)ST_X_BUDGET) return CBK_ERR_UNSUPPORTED;
   int mc = (int)((size_t)ST_X_BUDGET / ((size_t)NDIG * m.N));      // activation rows per pass
   mc = mc > ST_MAX_M ? ST_MAX_M : mc;

@@ -181,6 +181,34 @@ def test_gemv_survivor_streams_on_matrix_cores(shape):
                 assert torch.equal(yb, want), (case_id(case), K, N, M)
 
 
+@pytest.mark.parametrize("shape", [(6160, 4096), (1768, 14336)], ids=lambda s: f"{s[0]}x{s[1]}")
+def test_gemv_survivor_streams_fused_gate_up(shape):
+    """A fused gate/up matrix (two col_scale vectors by row parity, docs/FORMAT.md:126-151) as
+    SPARSE4X on the matrix-core stream kernel: every activation row is staged twice, once per
+    vector, and a weight row keeps the sums of its own parity.  Whole rows in LDS (4096 columns)
+    and split by columns or in passes of one row (14336 columns); bias; row by row against M = 1."""
+    K, N = shape
+    case = (F.SPARSE4X, 4, 128, 0)
+    raw = make_raw(case, K, N, seed=K + N)
+    pk = oracle_pack(case, raw)
+    rng = np.random.default_rng(K)
+    cs = (rng.random((2, N)) * 1.5 + 0.5).astype(np.float16)
+    pm = packed_from_oracle(case, pk, cs, K, N, DEV)
+    W = R.dequant(pk, K, N, case[0], col_scale=cs, cs_splits=(0, 0))
+    small = torch.empty(256, dtype=torch.uint8, device=DEV)
+    bias = acts(1, K, torch.float32, seed=K)[0].to(DEV)
+    for M, dtype in ((1, torch.float16), (2, torch.bfloat16), (3, torch.float16), (5, torch.bfloat16), (8, torch.float16)):
+        x = acts(M, N, dtype, seed=M + N)
+        ref = R.forward_ref(W, _np(x))
+        y = ops.gemv(pm, x.to(DEV), out_dtype=torch.float32)
+        assert rel_fro(_np(y), ref) < 1e-5, (K, N, M)
+        assert torch.equal(ops.gemv(pm, x.to(DEV), out_dtype=torch.float32, workspace=small), y), (K, N, M)
+        y1 = ops.gemv(pm, x[M - 1:M].to(DEV), out_dtype=torch.float32)
+        assert torch.equal(y1[0], y[M - 1]), (K, N, M)
+        yb = ops.gemv(pm, x.to(DEV), bias=bias, out_dtype=torch.float32)
+        assert torch.equal(yb, y + bias[None, :]), (K, N, M)
+
+
 def test_gemv_survivor_streams_over_many_rounds():
     """The matrix-core stream kernel where a workgroup goes through several rounds of two tiles
     with eight parts each (20496 x 4096: five or six tiles per workgroup): the part sums of a
