@@ -1777,8 +1777,42 @@ static bool stream_mfma_plan(const DMat& m, SmPlan& p) {
   return true;
 }
 
+// The q | k | v ranges of a survivor-stream matrix with three col_scale vectors, each as a matrix
+// with one vector (the rows of such a matrix are found through row_off, so any row starts a
+// range).  Returns how many are not empty.
+static int stream_row_ranges(const DMat& m, DMat (&sub)[3], int (&lo)[3]) {
+  const int b0 = m.cs_split0, b1 = m.cs_split0 + m.cs_split1;
+  const int l[3] = {0, b0, b1}, h[3] = {b0, b1, m.K};
+  int n = 0;
+  for (int r = 0; r < 3; ++r) {
+    if (h[r] <= l[r]) continue;
+    DMat d = m;
+    d.row_off = m.row_off + l[r];
+    d.scale = m.scale + (size_t)l[r] * m.G;
+    d.zero = m.zero + (size_t)l[r] * m.G;
+    d.K = h[r] - l[r];
+    d.cs = m.cs + (size_t)r * m.N;
+    d.cs_rows = 1;
+    d.cs_split0 = d.cs_split1 = 0;
+    sub[n] = d; lo[n] = l[r];
+    ++n;
+  }
+  return n;
+}
+
 // Room for the part sums of a call whose activation rows do not fit in LDS as whole rows; 0: none needed.
 size_t gemv_stream_workspace(const DMat& m, int M) {
+  if (family_of(m.layout) == FAM_SPARSE && m.cs_rows == 3 && m.cs) {   // run range by range, on the same bytes
+    DMat sub[3];
+    int lo[3];
+    size_t need = 0;
+    const int n = stream_row_ranges(m, sub, lo);
+    for (int i = 0; i < n; ++i) {
+      const size_t b = gemv_stream_workspace(sub[i], M);
+      need = need > b ? need : b;
+    }
+    return need;
+  }
   SmPlan p;
   if (family_of(m.layout) != FAM_SPARSE || m.bits != 4 || m.group != 128 || m.cs_rows > 2) return 0;
   const int vm = m.cs_rows == 2 ? 2 : 1;
@@ -1878,9 +1912,24 @@ static int launch_gemv_stream_mfma(const DMat& m, const void* x, int xdt, int M,
 // CBK_ERR_UNSUPPORTED: not a case of this kernel (the caller falls back on the float row kernel).
 int launch_gemv_stream(const DMat& m, const void* x, int xdt, int M, int64_t ldx, void* y, int ydt, int64_t ldy,
                        const void* bias, void* ws, size_t ws_bytes, hipStream_t st) {
-  if (family_of(m.layout) != FAM_SPARSE || m.bits != 4 || m.group != 128 || m.cs_rows > 2) return CBK_ERR_UNSUPPORTED;
+  if (family_of(m.layout) != FAM_SPARSE || m.bits != 4 || m.group != 128 || m.cs_rows > 3) return CBK_ERR_UNSUPPORTED;
   if (!(m.flags & CBK_FLAG_ZERO_LE_128)) return CBK_ERR_UNSUPPORTED;
   if (xdt != CBK_F16 && xdt != CBK_BF16T) return CBK_ERR_DTYPE;
+  if (m.cs_rows == 3) {
+    // a fused q | k | v matrix: its three row ranges one after the other, each with its own
+    // col_scale vector (and, by its own shape, on the matrix-core or on the row kernel)
+    if (!m.cs || (size_t)NDIG * m.N > (size_t)ST_X_BUDGET) return CBK_ERR_UNSUPPORTED;
+    DMat sub[3];
+    int lo[3];
+    const int n = stream_row_ranges(m, sub, lo);
+    const size_t ysz = ydt == CBK_F32 ? 4 : 2;
+    for (int i = 0; i < n; ++i) {
+      const int rc = launch_gemv_stream(sub[i], x, xdt, M, ldx, (uint8_t*)y + (size_t)lo[i] * ysz, ydt, ldy,
+                                        bias ? (const uint8_t*)bias + (size_t)lo[i] * ysz : nullptr, ws, ws_bytes, st);
+      if (rc) return rc;
+    }
+    return CBK_OK;
+  }
   {
     const int rc = launch_gemv_stream_mfma(m, x, xdt, M, ldx, y, ydt, ldy, bias, ws, ws_bytes, st);   // the layouts with group offsets
     if (rc != CBK_ERR_UNSUPPORTED) return rc;

@@ -209,6 +209,31 @@ def test_gemv_survivor_streams_fused_gate_up(shape):
         assert torch.equal(yb, y + bias[None, :]), (K, N, M)
 
 
+@pytest.mark.parametrize("case", SPARSE_CASES, ids=case_id)
+def test_gemv_survivor_streams_fused_qkv(case):
+    """A fused q | k | v matrix (three col_scale vectors by row range, docs/FORMAT.md:126-151) of
+    survivor streams: run range by range, each with its vector (here the q range is large enough
+    for the matrix-core kernel where the layout has group offsets, k and v go to the row kernel);
+    range boundaries off the 16-row grid."""
+    kq, kk, kv, N = 4100, 1020, 1024, 4096
+    K = kq + kk + kv
+    raw = make_raw(case, K, N, seed=K + case[0])
+    pk = oracle_pack(case, raw)
+    rng = np.random.default_rng(K)
+    cs = (rng.random((3, N)) * 1.5 + 0.5).astype(np.float16)
+    pm = packed_from_oracle(case, pk, cs, K, N, DEV, cs_splits=(kq, kk))
+    W = R.dequant(pk, K, N, case[0], col_scale=cs, cs_splits=(kq, kk))
+    bias = acts(1, K, torch.float32, seed=K)[0].to(DEV)
+    for M, dtype in ((1, torch.float16), (3, torch.bfloat16), (8, torch.float16)):
+        x = acts(M, N, dtype, seed=M + N)
+        ref = R.forward_ref(W, _np(x))
+        y = ops.gemv(pm, x.to(DEV), out_dtype=torch.float32)
+        assert rel_fro(_np(y), ref) < 1e-5, (case_id(case), M)
+        y1 = ops.gemv(pm, x[M - 1:M].to(DEV), out_dtype=torch.float32)
+        assert torch.equal(y1[0], y[M - 1]), (case_id(case), M)
+        assert torch.equal(ops.gemv(pm, x.to(DEV), bias=bias, out_dtype=torch.float32), y + bias[None, :]), (case_id(case), M)
+
+
 def test_gemv_survivor_streams_over_many_rounds():
     """The matrix-core stream kernel where a workgroup goes through several rounds of two tiles
     with eight parts each (20496 x 4096: five or six tiles per workgroup): the part sums of a
