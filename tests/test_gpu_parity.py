@@ -361,6 +361,35 @@ def test_gemv_batch_of_staged_and_column_split_matrices():
                     assert torch.equal(rows[i][j][0], y[i]), (shapes[j], M, i)
 
 
+def test_gemv_batch_of_mixed_layouts_with_and_without_workspace():
+    """A batch that the one-launch path does not take (a survivor-stream matrix with long rows
+    beside fixed-stride ones) runs matrix by matrix, each with its slice of the workspace; with
+    no workspace at all the call still succeeds (cbk_gemv does without) and gives the same bits."""
+    pms = [F.synth_packed(2048, 14336, F.SPARSE4X, 4, 128, None, seed=1, device=DEV),
+           F.synth_packed(64, 14336, F.BLK1632_4, 4, 128, 16, seed=2, device=DEV).to_tiled(),
+           F.synth_packed(4112, 3072, F.SPARSE4, 4, 128, None, seed=3, device=DEV)]
+    M = 8
+    xs = [acts(M, pm.N, torch.float16, seed=i).to(DEV) for i, pm in enumerate(pms)]
+    ys = ops.gemv_batch(pms, xs, out_dtype=torch.float32)
+    L = _lib.lib()
+    n = len(pms)
+    P = ctypes.c_void_p
+    descs = (_lib.CbkDesc * n)(*[pm.desc() for pm in pms])
+    assert L.cbk_gemv_batch_workspace_bytes(n, descs, M) > 0
+    outs = [torch.empty(M, pm.K, dtype=torch.float32, device=DEV) for pm in pms]
+    rc = L.cbk_gemv_batch(n, descs, (P * n)(*[x.data_ptr() for x in xs]), (ctypes.c_int64 * n)(*[pm.N for pm in pms]),
+                          F.dtype_code(torch.float16), M, (P * n)(*[o.data_ptr() for o in outs]),
+                          (ctypes.c_int64 * n)(*[pm.K for pm in pms]), F.dtype_code(torch.float32), None, None, 0,
+                          torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, L.cbk_strerror(rc)
+    torch.cuda.synchronize()
+    for pm, x, y, o in zip(pms, xs, ys, outs):
+        ref = x.double() @ ops.dequant(pm, torch.float32).double().t()
+        assert float((y.double() - ref).norm() / ref.norm()) < 1e-5
+        assert torch.equal(y, o)
+        assert torch.equal(y, ops.gemv(pm, x, out_dtype=torch.float32))
+
+
 def test_gemv_output_dtypes_bias_and_strided_x():
     case = (F.BLK1632_4, 4, 128, 16)
     K, N = 128, 2048
